@@ -1,0 +1,160 @@
+#!/usr/bin/env python3
+"""Headline benchmark: one fused pair on one MI355X, against the same two kernels launched
+back to back.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--pair N] [--no-cpu]
+
+A step is one launch of the fused kernel over device-resident synthetic inputs.  The
+workload is pair 2 of the synthetic set (BERT-base shapes: GEMM fp32 [512x768].[768x2304]
+block-fused with LayerNorm [512x768]); `--pair` selects another pair.
+
+Prints ONE JSON line.  `value` is the fused kernel's GPU-side duration in microseconds (mean
+over the K timed launches, from the start/end timestamps of each dispatch).  Beside it:
+  back_to_back_us   first start -> second end of the two unfused kernels on one stream
+  serial_sum_us     sum of the two unfused kernel durations (the reference's "serial",
+                    scripts/analyze_test_suite.py:425-428)
+  batched_*_us      wall-clock microseconds per launch with K launches queued back to back
+                    (includes dispatch gaps, lets consecutive launches overlap their ramp-up)
+  roofline          algorithmic flops (or bytes) of the pair / fused duration vs the MI355X peak
+  cpu_baseline      the OpenMP CPU reference (oracle/) timed on this host's cores
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+import numpy as np  # noqa: E402
+
+
+def cpu_baseline(pair_number, I1, F1, I2, F2, passes=5):
+    """Times the CPU oracle (the checker, not the product) on this host."""
+    from oracle import oracle as orf
+    from tests import oracle_cases
+    best = None
+    for _ in range(passes):
+        t0 = time.perf_counter()
+        oracle_cases.expected(pair_number, I1, F1, I2, F2)
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    return {"value": round(best * 1e6, 1), "unit": "us", "cores": orf.num_threads(), "kind": "port",
+            "sample": f"best of {passes} full passes of pair {pair_number} (both operators, OpenMP, double accumulation)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--pair", type=int, default=2)
+    ap.add_argument("--fusion", default="", help="kind[:suffix][@k1,k2] to pin the fused variant (default: headline)")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one fused pair on ONE GPU: the path has no cross-device data flow and "
+                 "this build launches nothing on a second GPU; run with --gpus 1")
+
+    import bfuse_project_amd as bf
+    from bfuse_project_amd.workloads import PAIRS, HEADLINE
+
+    pair = PAIRS[args.pair]
+    k1, k2, kind, suffix = HEADLINE[args.pair]
+    if args.fusion:
+        spec, _, ks = args.fusion.partition("@")
+        kind, _, suffix = spec.partition(":")
+        if ks:
+            k1, k2 = ks.split(",")
+    K, W = args.steps, args.warmup
+    I1, F1, I2, F2 = pair.inputs()
+
+    with bf.Operation(k1, k2) as op:
+        dev = bf.operation.device_name()
+        op.upload(0, I1, F1)
+        op.upload(1, I2, F2)
+        fused = op.fused(kind, suffix)
+
+        # correctness inside the bench: fused output must equal the unfused kernels bit for bit
+        op.zero_outputs()
+        op.launch("serial")
+        U1, U2 = op.download(0), op.download(1)
+        op.zero_outputs()
+        op.launch(kind, fused)
+        Q1, Q2 = op.download(0), op.download(1)
+        bit_exact = bool(np.array_equal(U1.view(np.uint8), Q1.view(np.uint8)) and
+                         np.array_equal(U2.view(np.uint8), Q2.view(np.uint8)))
+
+        # GPU-side durations (dispatch timestamps), W warm-up + K timed launches each
+        t_f = op.time(kind, fused, warmup=W, reps=K)[0]
+        t_ser, t_a, t_b = op.time("serial", warmup=W, reps=K)
+        t_par = op.time("parallel", warmup=W, reps=K)[0]
+        t_f2 = op.time(kind, fused, warmup=W, reps=K)[0]     # again, after the baselines (clock drift)
+        fused_us = float(min(t_f.mean(), t_f2.mean()))
+
+        # the timed region of the contract: W untimed, then exactly K steps between two syncs
+        for _ in range(W):
+            op.launch(kind, fused)
+        op.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(K):
+            op.launch(kind, fused)
+        op.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3 / K
+
+        b_f = op.time_batched(kind, fused, warmup=W, reps=K)
+        b_ser = op.time_batched("serial", warmup=W, reps=K)
+        b_k1 = op.time_batched("kernel1", warmup=W, reps=K)
+        b_k2 = op.time_batched("kernel2", warmup=W, reps=K)
+
+    serial_sum = float(t_a.mean() + t_b.mean())
+    back_to_back = float(t_ser.mean())
+    if pair.bound == "mfma":
+        achieved, unit = pair.flops / fused_us * 1e-6, "TFLOP/s"      # flops / us = MFLOP/s
+    else:
+        achieved, unit = (pair.bytes1 + pair.bytes2) / fused_us * 1e-3, "GB/s"
+    out = {
+        "metric": "fused-pair kernel us (speedup vs back-to-back launches; % roofline alongside)",
+        "value": round(fused_us, 3),
+        "unit": "us",
+        "n_gpus": 1,
+        "steps": K,
+        "warmup": W,
+        "ms_per_step": round(wall_ms, 6),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": pair.dtype,
+        "data": "synthetic (seeded, device-resident)",
+        "config": {"workload": f"pair {pair.number}: {pair.title}", "fused_kernel": fused.name,
+                   "grid": list(fused.grid), "block": list(fused.block), "device": dev},
+        "bit_exact_vs_unfused": bit_exact,
+        "fused_us": {"mean": round(float(t_f2.mean()), 3), "min": round(float(min(t_f.min(), t_f2.min())), 3),
+                     "std": round(float(t_f2.std()), 3), "first_pass_mean": round(float(t_f.mean()), 3)},
+        "back_to_back_us": round(back_to_back, 3),
+        "serial_sum_us": round(serial_sum, 3),
+        "kernel1_us": round(float(t_a.mean()), 3),
+        "kernel2_us": round(float(t_b.mean()), 3),
+        "parallel_streams_us": round(float(t_par.mean()), 3),
+        "speedup_vs_back_to_back": round(back_to_back / fused_us, 4),
+        "speedup_vs_serial_sum": round(serial_sum / fused_us, 4),
+        "fused_over_back_to_back": round(fused_us / back_to_back, 4),
+        "batched_fused_us": round(b_f, 3),
+        "batched_back_to_back_us": round(b_ser, 3),
+        "batched_kernel1_us": round(b_k1, 3),
+        "batched_kernel2_us": round(b_k2, 3),
+        "batched_fused_over_back_to_back": round(b_f / b_ser, 4),
+        "roofline": {"bound": pair.bound, "achieved": round(achieved, 2), "peak": pair.peak, "unit": unit,
+                     "frac": round(achieved / pair.peak, 4), "traffic": None,
+                     "kernel": fused.name, "avg_us": round(fused_us, 3),
+                     "algorithmic": {"flops": pair.flops, "bytes": pair.bytes1 + pair.bytes2}},
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(pair.number, I1, F1, I2, F2)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,208 @@
+// The three ways an operator body is instantiated, and the kernel registry.
+//
+//   single : one operator, the standalone ("unfused") kernel
+//   bfuse  : block fusion  -- fused grid = sum of grids, blockIdx.x selects operator and
+//            virtual block through a compile-time BlockPlan; LDS is a union of both sides
+//            (the reference's emitted form: horizontal-fuser/src/Matchers.cc:523-602,
+//            union layout Tools.cc:219-251)
+//   hfuse  : horizontal fusion -- one workgroup hosts both operators on disjoint wave
+//            ranges; LDS is the sum of both sides; an intra-side barrier is the LDS-counter
+//            GroupSync instead of CUDA's bar.sync id,count (Matchers.cc:288-320, 655-727)
+//
+// Every instantiation calls the same Op::run body with a virtual (block, thread) id -- the
+// counterpart of the reference rewriting blockIdx/threadIdx to locals (Matchers.cc:255-286)
+// -- so a fused kernel executes, per output element, the instruction sequence of the
+// standalone kernel and the results are bit-identical.
+//
+// Kernel ABI, as in the reference (macro_h.py:182-198): extern "C", three pointers per
+// operator (input, second operand, output), six for a fused pair (operator 1's three, then
+// operator 2's), 1-D launch, no dynamic shared memory.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "dispatch.h"
+#include "wave.h"
+
+namespace bfuse {
+
+template <class Op>
+__device__ __forceinline__ void single_body(const void* I, const void* F, void* O)
+{
+    __shared__ typename Op::Smem sm;
+    Op::run((int)blockIdx.x, (int)threadIdx.x, sm, I, F, O, BlockSync{});
+}
+
+template <class A, class B, int PATTERN, int P0, int P1>
+struct BfusePair {
+    static constexpr LaunchDims dims[2] = {{A::GRID, A::BLOCK}, {B::GRID, B::BLOCK}};
+    static constexpr BlockPlan plan() { return make_block_plan(PATTERN, 2, dims, P0, P1); }
+    static constexpr int THREADS = imax(A::THREADS, B::THREADS);
+    static constexpr int GRID = A::GRID.size() + B::GRID.size();
+    // a guarded side must be masked on whole waves, or its barrier would wait on lanes that never arrive
+    static_assert(A::THREADS % kWaveSize == 0 && B::THREADS % kWaveSize == 0, "block sizes must be whole waves");
+};
+
+template <class A, class B, int PATTERN, int P0, int P1>
+__device__ __forceinline__ void bfuse_body(const void* I1, const void* F1, void* O1, const void* I2,
+                                           const void* F2, void* O2)
+{
+    using Pair = BfusePair<A, B, PATTERN, P0, P1>;
+    union ShrdUnion {
+        typename A::Smem a;
+        typename B::Smem b;
+    };
+    __shared__ ShrdUnion su;
+    constexpr BlockPlan plan = Pair::plan();
+    int virt = 0;
+    const int kernel_id = map_block(plan, (int)blockIdx.x, &virt);
+    const int tid = (int)threadIdx.x;
+    if (kernel_id == 0 && tid < A::THREADS) {
+        A::run(virt, tid, su.a, I1, F1, O1, BlockSync{});
+    } else if (kernel_id == 1 && tid < B::THREADS) {
+        B::run(virt, tid, su.b, I2, F2, O2, BlockSync{});
+    }
+}
+
+template <class A, class B>
+struct HfusePair {
+    static constexpr LaunchDims dims[2] = {{A::GRID, A::BLOCK}, {B::GRID, B::BLOCK}};
+    static constexpr ThreadPlan plan() { return plan_threads(2, dims, kWaveSize); }
+    static constexpr int THREADS = round_up(A::THREADS, kWaveSize) + round_up(B::THREADS, kWaveSize);
+    static constexpr int GRID = imax(A::GRID.size(), B::GRID.size());
+};
+
+template <class A, class B>
+__device__ __forceinline__ void hfuse_body(const void* I1, const void* F1, void* O1, const void* I2,
+                                           const void* F2, void* O2)
+{
+    struct ShrdSum {
+        typename A::Smem a;
+        typename B::Smem b;
+        unsigned int arrive[2];
+    };
+    __shared__ ShrdSum ss;
+    constexpr ThreadPlan plan = HfusePair<A, B>::plan();
+    // the only whole-workgroup barrier: zero the per-side arrival counters before the sides diverge
+    if (threadIdx.x < 2) ss.arrive[threadIdx.x] = 0u;
+    __syncthreads();
+    int local = 0;
+    const int kernel_id = map_thread(plan, (int)blockIdx.x, (int)threadIdx.x, &local);
+    if (kernel_id == 0) {
+        A::run((int)blockIdx.x, local, ss.a, I1, F1, O1, GroupSync{&ss.arrive[0], (unsigned)(round_up(A::THREADS, kWaveSize) / kWaveSize), 0u});
+    } else if (kernel_id == 1) {
+        B::run((int)blockIdx.x, local, ss.b, I2, F2, O2, GroupSync{&ss.arrive[1], (unsigned)(round_up(B::THREADS, kWaveSize) / kWaveSize), 0u});
+    }
+}
+
+// ---- registry ---------------------------------------------------------------------------
+enum KernelKind : int { kSingle = 0, kBfuse = 1, kHfuse = 2 };
+
+struct TensorDesc {
+    int shape[4];   // padded with 1s, as the reference's macro.h tables (macro_h.py:28-42)
+    int elem_bytes;
+};
+
+struct KernelEntry {
+    std::string name;
+    const void* func;       // host-side handle of the __global__ function
+    int kind;
+    unsigned grid[3], block[3];
+    bool has_barriers;
+    TensorDesc io[3];       // single: I, F, O
+    std::string side[2];    // fused: names of the two standalone kernels
+    int pattern, p0, p1;    // bfuse: dispatch pattern and its parameters
+    unsigned (*read_sync_timeouts)();  // device counter of GroupSync give-ups in this module
+};
+
+std::vector<KernelEntry>& registry();
+
+struct Registrar {
+    explicit Registrar(const KernelEntry& e) { registry().push_back(e); }
+};
+
+template <class Op>
+KernelEntry make_single_entry(const char* name, const void* func, TensorDesc i, TensorDesc f, TensorDesc o,
+                              unsigned (*rst)())
+{
+    KernelEntry e{};
+    e.name = name;
+    e.func = func;
+    e.kind = kSingle;
+    e.grid[0] = Op::GRID.size(); e.grid[1] = 1; e.grid[2] = 1;
+    e.block[0] = Op::THREADS; e.block[1] = 1; e.block[2] = 1;
+    e.has_barriers = Op::HAS_BARRIERS;
+    e.io[0] = i; e.io[1] = f; e.io[2] = o;
+    e.read_sync_timeouts = rst;
+    return e;
+}
+
+template <class Pair>
+KernelEntry make_fused_entry(const char* name, const void* func, int kind, const char* k1, const char* k2,
+                             bool barriers, int pattern, int p0, int p1, unsigned (*rst)())
+{
+    KernelEntry e{};
+    e.name = name;
+    e.func = func;
+    e.kind = kind;
+    e.grid[0] = Pair::GRID; e.grid[1] = 1; e.grid[2] = 1;
+    e.block[0] = Pair::THREADS; e.block[1] = 1; e.block[2] = 1;
+    e.has_barriers = barriers;
+    e.side[0] = k1; e.side[1] = k2;
+    e.pattern = pattern; e.p0 = p0; e.p1 = p1;
+    e.read_sync_timeouts = rst;
+    return e;
+}
+
+}  // namespace bfuse
+
+// ---- definition macros (one extern "C" device symbol per kernel, reference naming) -----
+#define BFUSE_MODULE_PROLOGUE()                                                                     \
+    static unsigned bfuse_module_read_sync_timeouts()                                               \
+    {                                                                                               \
+        unsigned v = 0, z = 0;                                                                      \
+        if (hipMemcpyFromSymbol(&v, HIP_SYMBOL(bfuse::g_sync_timeouts), sizeof(v)) != hipSuccess) return ~0u; \
+        if (v) (void)hipMemcpyToSymbol(HIP_SYMBOL(bfuse::g_sync_timeouts), &z, sizeof(z));          \
+        return v;                                                                                   \
+    }
+
+#define BFUSE_KERNEL(NAME, OP, IDESC, FDESC, ODESC)                                                  \
+    extern "C" __global__ __launch_bounds__(OP::THREADS) void NAME(const void* __restrict__ I,       \
+                                                                   const void* __restrict__ F,       \
+                                                                   void* __restrict__ O)             \
+    {                                                                                               \
+        bfuse::single_body<OP>(I, F, O);                                                            \
+    }                                                                                               \
+    static bfuse::Registrar reg_##NAME(bfuse::make_single_entry<OP>(                                \
+        #NAME, (const void*)&NAME, bfuse::TensorDesc IDESC, bfuse::TensorDesc FDESC, bfuse::TensorDesc ODESC, \
+        &bfuse_module_read_sync_timeouts));
+
+#define BFUSE_BFUSE_KERNEL(K1, OP1, K2, OP2, SUFFIX, PATTERN, P0, P1)                                \
+    extern "C" __global__ __launch_bounds__((bfuse::BfusePair<OP1, OP2, PATTERN, P0, P1>::THREADS))  \
+    void K1##_##K2##_fused_bfuse##SUFFIX(const void* __restrict__ I1, const void* __restrict__ F1,   \
+                                         void* __restrict__ O1, const void* __restrict__ I2,         \
+                                         const void* __restrict__ F2, void* __restrict__ O2)         \
+    {                                                                                               \
+        bfuse::bfuse_body<OP1, OP2, PATTERN, P0, P1>(I1, F1, O1, I2, F2, O2);                        \
+    }                                                                                               \
+    static bfuse::Registrar reg_##K1##_##K2##_bfuse##SUFFIX(                                         \
+        bfuse::make_fused_entry<bfuse::BfusePair<OP1, OP2, PATTERN, P0, P1>>(                        \
+            #K1 "_" #K2 "_fused_bfuse" #SUFFIX, (const void*)&K1##_##K2##_fused_bfuse##SUFFIX,       \
+            bfuse::kBfuse, #K1, #K2, OP1::HAS_BARRIERS || OP2::HAS_BARRIERS, PATTERN, P0, P1,        \
+            &bfuse_module_read_sync_timeouts));
+
+#define BFUSE_HFUSE_KERNEL(K1, OP1, K2, OP2)                                                         \
+    extern "C" __global__ __launch_bounds__((bfuse::HfusePair<OP1, OP2>::THREADS))                   \
+    void K1##_##K2##_fused_hfuse(const void* __restrict__ I1, const void* __restrict__ F1,           \
+                                 void* __restrict__ O1, const void* __restrict__ I2,                 \
+                                 const void* __restrict__ F2, void* __restrict__ O2)                 \
+    {                                                                                               \
+        bfuse::hfuse_body<OP1, OP2>(I1, F1, O1, I2, F2, O2);                                         \
+    }                                                                                               \
+    static bfuse::Registrar reg_##K1##_##K2##_hfuse(                                                 \
+        bfuse::make_fused_entry<bfuse::HfusePair<OP1, OP2>>(                                         \
+            #K1 "_" #K2 "_fused_hfuse", (const void*)&K1##_##K2##_fused_hfuse, bfuse::kHfuse, #K1, #K2, \
+            OP1::HAS_BARRIERS || OP2::HAS_BARRIERS, -1, 0, 0, &bfuse_module_read_sync_timeouts));

@@ -1,0 +1,230 @@
+// fp32 GEMM side: C[M,N] = A[M,K] . B[K,N] (+ optional tanh-GELU), row-major, on the
+// gfx950 matrix cores (v_mfma_f32_16x16x4_f32).
+//
+// Replaces the TVM-generated `dense` kernels of the reference
+// (scripts/configure_kernels.py:50-58; body e.g. tests/benchmark/cuda/dense1_0_dense2_0_bfuse.cu:82+).
+// Shapes are compile-time, as in the reference's generated kernels.  B is [K,N] (the
+// reference's dense weight is (out,in) = [N,K]; values and results do not depend on it).
+//
+// Decomposition, chosen for problems that are only a few 16x16 blocks per SIMD:
+//   * one workgroup = one BM x BN tile of C; its KS waves split K (wave w owns
+//     k in [w*K/KS, (w+1)*K/KS)) and each accumulates the WHOLE tile over its k-range.
+//     No operand is shared between waves, so operands go global -> VGPR directly in MFMA
+//     layout with 128-bit loads and the main loop has no barrier at all;
+//   * at the end the KS partial tiles meet in LDS (one barrier) and are summed in wave
+//     order 0..KS-1, so the result does not depend on timing;
+//   * columns are handled in groups of 64: lane (j = lane%16, kq = lane/16) loads
+//     B[k+4kq+t][n0+4j .. n0+4j+3] (t = 0..3) with one 128-bit load each.  Component e of
+//     those vectors feeds 16x16 block e of the group, whose column j therefore is global
+//     column n0+4j+e: after the MFMAs a lane holds four consecutive columns of a row and
+//     stores them with one 128-bit store.  A trailing group of 16 columns (BN % 64 == 16)
+//     uses 32-bit loads/stores.
+//   * lane (i = lane%16, kq) loads A[m0+i][k+4kq .. k+4kq+3]; component t is the A operand of
+//     MFMA step t, matching B row k+4kq+t above (the instruction sums over kq).
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "dispatch.h"
+#include "wave.h"
+
+namespace bfuse {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+enum Epilogue : int { kEpiNone = 0, kEpiGeluTanh = 1 };
+
+// 0.5*x*(1+tanh(0.797885*(x+0.044715*x^3))) with the constants of the reference's GPT-2 dump
+// (files/gpt2.txt:67-74).
+__device__ __forceinline__ float gelu_tanh(float x)
+{
+    const float x3 = x * x * x;
+    const float u = 0.797885f * (x + 0.044715f * x3);
+    return (0.5f * x) * (tanhf(u) + 1.0f);
+}
+
+template <int M_, int N_, int K_, int BM_, int BN_, int KS_, int EPI_ = kEpiNone, int NBUF_ = 2>
+struct GemmF32 {
+    static constexpr int M = M_, N = N_, K = K_, BM = BM_, BN = BN_, KS = KS_, EPI = EPI_;
+    static constexpr int TM = BM / 16;          // 16-row blocks per tile
+    static constexpr int G4 = BN / 64;          // 64-column groups
+    static constexpr int G1 = (BN % 64) / 16;   // trailing 16-column groups
+    static constexpr int KW = K / KS;           // k-range of one wave
+    static constexpr int STAGE = 16;            // k per stage (one 128-bit A load)
+    static constexpr int NSTAGE = KW / STAGE;
+    static constexpr int NBUF = NBUF_;          // register stages in flight (>= 2)
+    static_assert(M % BM == 0 && N % BN == 0, "tile must divide the problem");
+    static_assert(BM % 16 == 0 && BN % 16 == 0 && K % (KS * STAGE) == 0, "shape/tile mismatch");
+    static_assert(N % 4 == 0 && K % 4 == 0, "rows must be 16-byte aligned");
+    static_assert(NSTAGE >= NBUF - 1, "k-range shorter than the prefetch depth");
+
+    static constexpr Dims3 GRID{N / BN, M / BM, 1};
+    static constexpr Dims3 BLOCK{64 * KS, 1, 1};
+    static constexpr int THREADS = 64 * KS;
+    static constexpr bool HAS_BARRIERS = KS > 1;
+    static constexpr int NUNIT = TM * (G4 + G1);  // reduction / store units (one column group of one row block)
+
+    // partial tiles of every wave, in accumulator layout
+    struct Smem {
+        f32x4 part[KS > 1 ? KS : 1][KS > 1 ? TM * (4 * G4 + G1) : 1][64];
+    };
+
+    struct Frag {
+        f32x4 a[TM];
+        f32x4 b4[G4 > 0 ? G4 : 1][4];  // [group][t] -> 4 columns
+        float b1[G1 > 0 ? G1 : 1][4];  // [group][t]
+    };
+
+    __device__ static __forceinline__ void load_stage(Frag& f, const float* __restrict__ A,
+                                                      const float* __restrict__ B, int m0, int n0,
+                                                      int k, int lane)
+    {
+        const int i = lane & 15, kq = lane >> 4;
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+            f.a[tm] = *reinterpret_cast<const f32x4*>(A + (size_t)(m0 + tm * 16 + i) * K + k + 4 * kq);
+#pragma unroll
+        for (int g = 0; g < G4; ++g)
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                f.b4[g][t] = *reinterpret_cast<const f32x4*>(B + (size_t)(k + 4 * kq + t) * N + n0 + g * 64 + 4 * i);
+#pragma unroll
+        for (int g = 0; g < G1; ++g)
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                f.b1[g][t] = B[(size_t)(k + 4 * kq + t) * N + n0 + G4 * 64 + g * 16 + i];
+    }
+
+    __device__ static __forceinline__ void mma_stage(f32x4 (&acc)[TM][4 * G4 + G1], const Frag& f)
+    {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm) {
+#pragma unroll
+                for (int g = 0; g < G4; ++g)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        acc[tm][4 * g + e] = __builtin_amdgcn_mfma_f32_16x16x4f32(
+                            f.a[tm][t], f.b4[g][t][e], acc[tm][4 * g + e], 0, 0, 0);
+#pragma unroll
+                for (int g = 0; g < G1; ++g)
+                    acc[tm][4 * G4 + g] = __builtin_amdgcn_mfma_f32_16x16x4f32(
+                        f.a[tm][t], f.b1[g][t], acc[tm][4 * G4 + g], 0, 0, 0);
+            }
+        }
+    }
+
+    __device__ static __forceinline__ float epilogue(float v)
+    {
+        if constexpr (EPI == kEpiGeluTanh) return gelu_tanh(v);
+        return v;
+    }
+
+    // Store one unit (row block tm, column group u) held in accumulator layout:
+    // lane (j, rg) owns rows 4*rg+v (v = 0..3).
+    __device__ static __forceinline__ void store_group4(float* __restrict__ C, int m0, int n0, int tm,
+                                                        int g, const f32x4 (&blk)[4], int lane)
+    {
+        const int j = lane & 15, rg = lane >> 4;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            f32x4 o;
+            o[0] = epilogue(blk[0][v]);
+            o[1] = epilogue(blk[1][v]);
+            o[2] = epilogue(blk[2][v]);
+            o[3] = epilogue(blk[3][v]);
+            *reinterpret_cast<f32x4*>(C + (size_t)(m0 + tm * 16 + 4 * rg + v) * N + n0 + g * 64 + 4 * j) = o;
+        }
+    }
+    __device__ static __forceinline__ void store_group1(float* __restrict__ C, int m0, int n0, int tm,
+                                                        int g, const f32x4& blk, int lane)
+    {
+        const int j = lane & 15, rg = lane >> 4;
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+            C[(size_t)(m0 + tm * 16 + 4 * rg + v) * N + n0 + G4 * 64 + g * 16 + j] = epilogue(blk[v]);
+    }
+
+    template <class Sync>
+    __device__ static __forceinline__ void run(int vblock, int tid, Smem& sm, const void* I, const void* F,
+                                               void* O, Sync sync)
+    {
+        const float* __restrict__ A = static_cast<const float*>(I);
+        const float* __restrict__ B = static_cast<const float*>(F);
+        float* __restrict__ C = static_cast<float*>(O);
+        const Dims3 vb = delinearize(vblock, GRID);
+        const int m0 = vb.y * BM, n0 = vb.x * BN;
+        const int wave = tid >> 6, lane = tid & 63;
+        const int kbeg = wave * KW;
+
+        f32x4 acc[TM][4 * G4 + G1];
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+            for (int c = 0; c < 4 * G4 + G1; ++c) acc[tm][c] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+        Frag buf[NBUF];
+#pragma unroll
+        for (int s = 0; s < NBUF - 1; ++s) load_stage(buf[s], A, B, m0, n0, kbeg + s * STAGE, lane);
+
+        // NSTAGE stages, NBUF-1 loads in flight; the loop is unrolled by NBUF so every buffer
+        // index is a compile-time constant.
+        for (int s0 = 0; s0 < NSTAGE; s0 += NBUF) {
+#pragma unroll
+            for (int u = 0; u < NBUF; ++u) {
+                const int s = s0 + u;
+                if (s < NSTAGE) {
+                    if (s + NBUF - 1 < NSTAGE)
+                        load_stage(buf[(u + NBUF - 1) % NBUF], A, B, m0, n0, kbeg + (s + NBUF - 1) * STAGE, lane);
+                    mma_stage(acc, buf[u]);
+                }
+            }
+        }
+
+        if constexpr (KS == 1) {
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm) {
+#pragma unroll
+                for (int g = 0; g < G4; ++g) {
+                    const f32x4 blk[4] = {acc[tm][4 * g], acc[tm][4 * g + 1], acc[tm][4 * g + 2], acc[tm][4 * g + 3]};
+                    store_group4(C, m0, n0, tm, g, blk, lane);
+                }
+#pragma unroll
+                for (int g = 0; g < G1; ++g) store_group1(C, m0, n0, tm, g, acc[tm][4 * G4 + g], lane);
+            }
+        } else {
+            constexpr int NB = 4 * G4 + G1;
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+                for (int c = 0; c < NB; ++c) sm.part[wave][tm * NB + c][lane] = acc[tm][c];
+            sync();
+            // unit u = (tm, group); wave w finishes units u == w (mod KS), summing waves 0..KS-1 in order
+#pragma unroll
+            for (int u0 = 0; u0 < NUNIT; u0 += KS) {
+                const int u = u0 + wave;
+                if (u < NUNIT) {
+                    const int tm = u / (G4 + G1), g = u % (G4 + G1);
+                    if (g < G4) {
+                        f32x4 blk[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            f32x4 s = sm.part[0][tm * NB + 4 * g + e][lane];
+#pragma unroll
+                            for (int w = 1; w < KS; ++w) s += sm.part[w][tm * NB + 4 * g + e][lane];
+                            blk[e] = s;
+                        }
+                        store_group4(C, m0, n0, tm, g, blk, lane);
+                    } else {
+                        f32x4 s = sm.part[0][tm * NB + 4 * G4 + (g - G4)][lane];
+#pragma unroll
+                        for (int w = 1; w < KS; ++w) s += sm.part[w][tm * NB + 4 * G4 + (g - G4)][lane];
+                        store_group1(C, m0, n0, tm, g - G4, s, lane);
+                    }
+                }
+            }
+        }
+    }
+};
+
+}  // namespace bfuse

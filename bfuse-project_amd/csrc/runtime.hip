@@ -1,0 +1,697 @@
+// libbfuse_rt: the C ABI declared in include/bfuse_rt.h over the HIP runtime.
+// Host-side counterpart of the reference's generated harness
+// (test-utils/test-suite-files/operation_cu.py, main_cc.py, utils_cc.py).
+#include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "../../include/bfuse_rt.h"
+#include "dispatch.h"
+#include "fuse.h"
+
+namespace bfuse {
+std::vector<KernelEntry>& registry()
+{
+    static std::vector<KernelEntry> r;
+    return r;
+}
+}  // namespace bfuse
+
+using namespace bfuse;
+
+static_assert(sizeof(bfuse_block_plan) == sizeof(BlockPlan), "C and C++ plan layouts must agree");
+static_assert(sizeof(bfuse_thread_plan) == sizeof(ThreadPlan), "C and C++ plan layouts must agree");
+static_assert(sizeof(bfuse_launch_dims) == sizeof(LaunchDims), "C and C++ dims layouts must agree");
+static_assert(BFUSE_MAX_KERNELS == kMaxKernels && BFUSE_MAX_SEGMENTS == kMaxSegments, "limits must agree");
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+#define HIP_TRY(call)                                                                          \
+    do {                                                                                       \
+        hipError_t st_ = (call);                                                               \
+        if (st_ != hipSuccess)                                                                 \
+            return fail(BFUSE_ERR_HIP, "HIP error (%s:%d): %s: %s", __FILE__, __LINE__, #call, \
+                        hipGetErrorString(st_));                                               \
+    } while (0)
+
+struct Side {
+    void* buf[3] = {nullptr, nullptr, nullptr};  // I, F, O on the device
+    size_t bytes[3] = {0, 0, 0};
+    int elem[3] = {4, 4, 4};
+    hipStream_t stream = nullptr;                // S1 / S2
+    bool live = false;
+};
+
+struct State {
+    bool inited = false;
+    int device = -1;
+    Side side[2];
+} g;
+
+size_t shape_bytes(const int* s, int elem) { return (size_t)s[0] * s[1] * s[2] * s[3] * (size_t)elem; }
+
+int init_side(int idx, const int* I, const int* F, const int* O)
+{
+    if (!g.inited) return fail(BFUSE_ERR_STATE, "bfuse_init has not been called");
+    if (!I || !F || !O) return fail(BFUSE_ERR_ARG, "null shape");
+    Side& s = g.side[idx];
+    if (s.live) return fail(BFUSE_ERR_STATE, "kernel%d is already initialized", idx + 1);
+    const int* shp[3] = {I, F, O};
+    for (int i = 0; i < 3; ++i) {
+        s.bytes[i] = shape_bytes(shp[i], s.elem[i]);
+        if (s.bytes[i] == 0) return fail(BFUSE_ERR_ARG, "empty tensor");
+        HIP_TRY(hipMalloc(&s.buf[i], s.bytes[i]));
+    }
+    HIP_TRY(hipStreamCreate(&s.stream));
+    s.live = true;
+    return BFUSE_OK;
+}
+
+int fini_side(int idx)
+{
+    Side& s = g.side[idx];
+    if (!s.live) return fail(BFUSE_ERR_STATE, "kernel%d is not initialized", idx + 1);
+    HIP_TRY(hipStreamDestroy(s.stream));
+    for (int i = 2; i >= 0; --i) {
+        HIP_TRY(hipFree(s.buf[i]));
+        s.buf[i] = nullptr;
+    }
+    s.live = false;
+    return BFUSE_OK;
+}
+
+int check_shapes(int idx, const int* I, const int* F, const int* O)
+{
+    Side& s = g.side[idx];
+    if (!s.live) return fail(BFUSE_ERR_STATE, "kernel%d is not initialized", idx + 1);
+    const int* shp[3] = {I, F, O};
+    for (int i = 0; i < 3; ++i)
+        if (!shp[i] || shape_bytes(shp[i], s.elem[i]) != s.bytes[i])
+            return fail(BFUSE_ERR_ARG, "shape of tensor %d does not match initialize_kernel%d", i, idx + 1);
+    return BFUSE_OK;
+}
+
+dim3 d3(const unsigned* v) { return dim3(v[0], v[1], v[2]); }
+
+const KernelEntry* entry_of(const void* func)
+{
+    for (const auto& e : registry())
+        if (e.func == func) return &e;
+    return nullptr;
+}
+
+// The grid and block a caller passes must be the ones the kernel was built for: the bodies
+// index memory from compile-time shapes, so any other launch shape would read or write out
+// of bounds.
+int check_launch(const void* func, const unsigned* grid, const unsigned* block, int want_ptrs)
+{
+    if (!func || !grid || !block) return fail(BFUSE_ERR_ARG, "null launch argument");
+    const KernelEntry* e = entry_of(func);
+    if (!e) return fail(BFUSE_ERR_ARG, "func is not a kernel of this library");
+    const int ptrs = e->kind == kSingle ? 3 : 6;
+    if (ptrs != want_ptrs) return fail(BFUSE_ERR_ARG, "%s takes %d pointers, not %d", e->name.c_str(), ptrs, want_ptrs);
+    for (int i = 0; i < 3; ++i)
+        if (grid[i] != e->grid[i] || block[i] != e->block[i])
+            return fail(BFUSE_ERR_ARG, "%s must be launched with grid (%u,%u,%u) block (%u,%u,%u)", e->name.c_str(),
+                        e->grid[0], e->grid[1], e->grid[2], e->block[0], e->block[1], e->block[2]);
+    return BFUSE_OK;
+}
+
+// Buffers a single kernel touches must be at least as large as the shapes it was built for.
+int check_side_fits(const void* func, int idx)
+{
+    const KernelEntry* e = entry_of(func);
+    if (!e || e->kind != kSingle) return BFUSE_OK;
+    const Side& s = g.side[idx];
+    if (!s.live) return fail(BFUSE_ERR_STATE, "kernel%d is not initialized", idx + 1);
+    for (int i = 0; i < 3; ++i) {
+        const size_t need = shape_bytes(e->io[i].shape, e->io[i].elem_bytes);
+        if (s.bytes[i] < need)
+            return fail(BFUSE_ERR_ARG, "%s needs %zu bytes for tensor %d, side %d holds %zu", e->name.c_str(), need, i,
+                        idx + 1, s.bytes[i]);
+    }
+    return BFUSE_OK;
+}
+
+int check_fused_fits(const void* func)
+{
+    const KernelEntry* e = entry_of(func);
+    if (!e || e->kind == kSingle) return fail(BFUSE_ERR_ARG, "not a fused kernel");
+    for (int k = 0; k < 2; ++k) {
+        const KernelEntry* sk = nullptr;
+        for (const auto& c : registry())
+            if (c.kind == kSingle && c.name == e->side[k]) sk = &c;
+        if (!sk) return fail(BFUSE_ERR_ARG, "fused kernel %s names unknown side %s", e->name.c_str(), e->side[k].c_str());
+        int rc = check_side_fits(sk->func, k);
+        if (rc) return rc;
+    }
+    return BFUSE_OK;
+}
+
+int launch3(const void* func, const unsigned* grid, const unsigned* block, int idx, hipStream_t stream,
+            hipEvent_t ev0 = nullptr, hipEvent_t ev1 = nullptr)
+{
+    Side& s = g.side[idx];
+    void* args[3] = {&s.buf[0], &s.buf[1], &s.buf[2]};
+    if (ev0 || ev1)
+        HIP_TRY(hipExtLaunchKernel(func, d3(grid), d3(block), args, 0, stream, ev0, ev1, 0));
+    else
+        HIP_TRY(hipLaunchKernel(func, d3(grid), d3(block), args, 0, stream));
+    return BFUSE_OK;
+}
+
+int launch6(const void* func, const unsigned* grid, const unsigned* block, hipStream_t stream,
+            hipEvent_t ev0 = nullptr, hipEvent_t ev1 = nullptr)
+{
+    Side &a = g.side[0], &b = g.side[1];
+    void* args[6] = {&a.buf[0], &a.buf[1], &a.buf[2], &b.buf[0], &b.buf[1], &b.buf[2]};
+    if (ev0 || ev1)
+        HIP_TRY(hipExtLaunchKernel(func, d3(grid), d3(block), args, 0, stream, ev0, ev1, 0));
+    else
+        HIP_TRY(hipLaunchKernel(func, d3(grid), d3(block), args, 0, stream));
+    return BFUSE_OK;
+}
+
+int sync_and_check(const void* fused_func)
+{
+    HIP_TRY(hipDeviceSynchronize());
+    HIP_TRY(hipGetLastError());
+    if (fused_func) {
+        const KernelEntry* e = entry_of(fused_func);
+        if (e && e->kind == kHfuse && e->read_sync_timeouts) {
+            unsigned n = e->read_sync_timeouts();
+            if (n) return fail(BFUSE_ERR_SYNC, "%s: %u side-barrier waits gave up", e->name.c_str(), n);
+        }
+    }
+    return BFUSE_OK;
+}
+
+int validate_mode(int mode, const void* fa, const unsigned* ga, const unsigned* ba, const void* fb,
+                  const unsigned* gb, const unsigned* bb)
+{
+    int rc;
+    switch (mode) {
+        case BFUSE_MODE_KERNEL1:
+            if ((rc = check_launch(fa, ga, ba, 3)) || (rc = check_side_fits(fa, 0))) return rc;
+            break;
+        case BFUSE_MODE_KERNEL2:
+            if ((rc = check_launch(fa, ga, ba, 3)) || (rc = check_side_fits(fa, 1))) return rc;
+            break;
+        case BFUSE_MODE_PARALLEL:
+        case BFUSE_MODE_SERIAL:
+            if ((rc = check_launch(fa, ga, ba, 3)) || (rc = check_side_fits(fa, 0))) return rc;
+            if ((rc = check_launch(fb, gb, bb, 3)) || (rc = check_side_fits(fb, 1))) return rc;
+            break;
+        case BFUSE_MODE_HFUSE:
+        case BFUSE_MODE_BFUSE: {
+            if ((rc = check_launch(fa, ga, ba, 6)) || (rc = check_fused_fits(fa))) return rc;
+            const KernelEntry* e = entry_of(fa);
+            if ((mode == BFUSE_MODE_HFUSE) != (e->kind == kHfuse))
+                return fail(BFUSE_ERR_ARG, "%s is not a %s kernel", e->name.c_str(), mode == BFUSE_MODE_HFUSE ? "hfuse" : "bfuse");
+            break;
+        }
+        default:
+            return fail(BFUSE_ERR_ARG, "unknown mode %d", mode);
+    }
+    return BFUSE_OK;
+}
+
+// Enqueue one repetition. ev = {start_a, stop_a, start_b, stop_b} or nullptr.
+int enqueue_mode(int mode, const void* fa, const unsigned* ga, const unsigned* ba, const void* fb,
+                 const unsigned* gb, const unsigned* bb, hipEvent_t* ev)
+{
+    hipEvent_t e0 = ev ? ev[0] : nullptr, e1 = ev ? ev[1] : nullptr, e2 = ev ? ev[2] : nullptr, e3 = ev ? ev[3] : nullptr;
+    int rc;
+    switch (mode) {
+        case BFUSE_MODE_KERNEL1: return launch3(fa, ga, ba, 0, nullptr, e0, e1);
+        case BFUSE_MODE_KERNEL2: return launch3(fa, ga, ba, 1, nullptr, e0, e1);
+        case BFUSE_MODE_PARALLEL:
+            if ((rc = launch3(fa, ga, ba, 0, g.side[0].stream, e0, e1))) return rc;
+            return launch3(fb, gb, bb, 1, g.side[1].stream, e2, e3);
+        case BFUSE_MODE_SERIAL:
+            if ((rc = launch3(fa, ga, ba, 0, nullptr, e0, e1))) return rc;
+            return launch3(fb, gb, bb, 1, nullptr, e2, e3);
+        case BFUSE_MODE_HFUSE:
+        case BFUSE_MODE_BFUSE: return launch6(fa, ga, ba, nullptr, e0, e1);
+    }
+    return fail(BFUSE_ERR_ARG, "unknown mode %d", mode);
+}
+
+__global__ void map_blocks_kernel(BlockPlan plan, int lo, int hi, int* kernel_out, int* virt_out)
+{
+    const int bid = lo + (int)(blockIdx.x * blockDim.x + threadIdx.x);
+    if (bid < hi) {
+        int v = -1;
+        const int k = map_block(plan, bid, &v);
+        kernel_out[bid - lo] = k;
+        virt_out[bid - lo] = v;
+    }
+}
+
+inline unsigned long long splitmix64(unsigned long long x)
+{
+    x += 0x9E3779B97F4A7C15ull;
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+    return x ^ (x >> 31);
+}
+inline double u01(unsigned long long seed, unsigned long long i)  // in (0,1)
+{
+    const unsigned long long r = splitmix64(seed * 0xD1342543DE82EF95ull + i);
+    return ((double)(r >> 11) + 0.5) * (1.0 / 9007199254740992.0);
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* bfuse_last_error(void) { return g_err; }
+
+int bfuse_init(int device)
+{
+    int n = 0;
+    hipError_t st = hipGetDeviceCount(&n);
+    if (st != hipSuccess || n <= 0)
+        return fail(BFUSE_ERR_HIP, "no HIP device available (%s); this library has no CPU path",
+                    st == hipSuccess ? "device count is 0" : hipGetErrorString(st));
+    if (device < 0 || device >= n) return fail(BFUSE_ERR_ARG, "device %d out of range (0..%d)", device, n - 1);
+    HIP_TRY(hipSetDevice(device));
+    g.device = device;
+    g.inited = true;
+    return BFUSE_OK;
+}
+
+int bfuse_shutdown(void)
+{
+    for (int i = 0; i < 2; ++i)
+        if (g.side[i].live) {
+            int rc = fini_side(i);
+            if (rc) return rc;
+        }
+    g.inited = false;
+    return BFUSE_OK;
+}
+
+int bfuse_device_info(char* name, size_t name_len, int* cus, int* lds, int* wave)
+{
+    if (!g.inited) return fail(BFUSE_ERR_STATE, "bfuse_init has not been called");
+    hipDeviceProp_t p;
+    HIP_TRY(hipGetDeviceProperties(&p, g.device));
+    if (name && name_len) snprintf(name, name_len, "%s%s%s", p.name, p.name[0] ? " " : "", p.gcnArchName);
+    if (cus) *cus = p.multiProcessorCount;
+    if (lds) *lds = (int)p.sharedMemPerBlock;
+    if (wave) *wave = p.warpSize;
+    return BFUSE_OK;
+}
+
+// ---- index maps -------------------------------------------------------------------------
+int bfuse_plan_threads(int n, const bfuse_launch_dims* k, int pad, bfuse_thread_plan* out)
+{
+    if (n < 1 || n > kMaxKernels || !k || !out || pad < 1) return fail(BFUSE_ERR_ARG, "bad argument");
+    for (int i = 0; i < n; ++i)
+        for (int d = 0; d < 3; ++d)
+            if (k[i].grid[d] < 1 || k[i].block[d] < 1) return fail(BFUSE_ERR_ARG, "launch dims must be positive");
+    const ThreadPlan p = plan_threads(n, reinterpret_cast<const LaunchDims*>(k), pad);
+    memcpy(out, &p, sizeof(p));
+    return BFUSE_OK;
+}
+
+int bfuse_plan_blocks(int pattern, int n, const bfuse_launch_dims* k, int p0, int p1, bfuse_block_plan* out)
+{
+    if (n < 1 || n > kMaxKernels || !k || !out) return fail(BFUSE_ERR_ARG, "bad argument");
+    if (pattern < kZigzag || pattern > kRanges) return fail(BFUSE_ERR_ARG, "unknown pattern %d", pattern);
+    for (int i = 0; i < n; ++i)
+        for (int d = 0; d < 3; ++d)
+            if (k[i].grid[d] < 1 || k[i].block[d] < 1) return fail(BFUSE_ERR_ARG, "launch dims must be positive");
+    if ((pattern == kZigzag && (p0 < 1 || p1 < 1)) || ((pattern == kProportional || pattern == kChunked) && p0 < 1))
+        return fail(BFUSE_ERR_ARG, "pattern parameters must be positive");
+    const BlockPlan p = make_block_plan(pattern, n, reinterpret_cast<const LaunchDims*>(k), p0, p1);
+    memcpy(out, &p, sizeof(p));
+    return BFUSE_OK;
+}
+
+int bfuse_map_block(const bfuse_block_plan* plan, int bid, int* virt)
+{
+    int v = -1;
+    const int k = map_block(*reinterpret_cast<const BlockPlan*>(plan), bid, &v);
+    if (virt) *virt = v;
+    return k;
+}
+
+int bfuse_map_thread(const bfuse_thread_plan* plan, int bid, int tid, int* local)
+{
+    int l = -1;
+    const int k = map_thread(*reinterpret_cast<const ThreadPlan*>(plan), bid, tid, &l);
+    if (local) *local = l;
+    return k;
+}
+
+int bfuse_map_blocks_device(const bfuse_block_plan* plan, int lo, int hi, int* kernel_out, int* virt_out)
+{
+    if (!g.inited) return fail(BFUSE_ERR_STATE, "bfuse_init has not been called");
+    if (!plan || !kernel_out || !virt_out || hi <= lo) return fail(BFUSE_ERR_ARG, "bad argument");
+    const int n = hi - lo;
+    int *dk = nullptr, *dv = nullptr;
+    HIP_TRY(hipMalloc(&dk, sizeof(int) * (size_t)n));
+    HIP_TRY(hipMalloc(&dv, sizeof(int) * (size_t)n));
+    BlockPlan p;
+    memcpy(&p, plan, sizeof(p));
+    hipLaunchKernelGGL(map_blocks_kernel, dim3((n + 255) / 256), dim3(256), 0, nullptr, p, lo, hi, dk, dv);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipMemcpy(kernel_out, dk, sizeof(int) * (size_t)n, hipMemcpyDeviceToHost));
+    HIP_TRY(hipMemcpy(virt_out, dv, sizeof(int) * (size_t)n, hipMemcpyDeviceToHost));
+    HIP_TRY(hipFree(dk));
+    HIP_TRY(hipFree(dv));
+    return BFUSE_OK;
+}
+
+// ---- registry ---------------------------------------------------------------------------
+static void fill_info(const KernelEntry& e, bfuse_kernel_info* o)
+{
+    memset(o, 0, sizeof(*o));
+    snprintf(o->name, sizeof(o->name), "%s", e.name.c_str());
+    o->func = e.func;
+    o->kind = e.kind;
+    for (int i = 0; i < 3; ++i) {
+        o->grid[i] = e.grid[i];
+        o->block[i] = e.block[i];
+        for (int d = 0; d < 4; ++d) o->shape[i][d] = e.io[i].shape[d];
+        o->elem_bytes[i] = e.io[i].elem_bytes;
+    }
+    o->has_barriers = e.has_barriers;
+    o->regs = -1;
+    o->lds_bytes = -1;
+    if (g.inited) {
+        hipFuncAttributes a;
+        if (hipFuncGetAttributes(&a, e.func) == hipSuccess) {
+            o->regs = a.numRegs;
+            o->lds_bytes = (int)a.sharedSizeBytes;
+        } else {
+            (void)hipGetLastError();
+        }
+    }
+    snprintf(o->side[0], sizeof(o->side[0]), "%s", e.side[0].c_str());
+    snprintf(o->side[1], sizeof(o->side[1]), "%s", e.side[1].c_str());
+    o->pattern = e.pattern;
+    o->p0 = e.p0;
+    o->p1 = e.p1;
+}
+
+int bfuse_kernel_count(void) { return (int)registry().size(); }
+
+int bfuse_kernel_at(int index, bfuse_kernel_info* out)
+{
+    if (index < 0 || index >= (int)registry().size() || !out) return fail(BFUSE_ERR_ARG, "index out of range");
+    fill_info(registry()[index], out);
+    return BFUSE_OK;
+}
+
+int bfuse_kernel_find(const char* name, bfuse_kernel_info* out)
+{
+    if (!name || !out) return fail(BFUSE_ERR_ARG, "null argument");
+    for (const auto& e : registry())
+        if (e.name == name) {
+            fill_info(e, out);
+            return BFUSE_OK;
+        }
+    return fail(BFUSE_ERR_ARG, "unknown kernel '%s'", name);
+}
+
+// ---- harness ----------------------------------------------------------------------------
+int bfuse_set_elem_bytes(int side, int ib, int fb, int ob)
+{
+    if (side < 1 || side > 2) return fail(BFUSE_ERR_ARG, "side must be 1 or 2");
+    if (g.side[side - 1].live) return fail(BFUSE_ERR_STATE, "set element sizes before initialize_kernel%d", side);
+    const int v[3] = {ib, fb, ob};
+    for (int i = 0; i < 3; ++i) {
+        if (v[i] != 1 && v[i] != 2 && v[i] != 4 && v[i] != 8) return fail(BFUSE_ERR_ARG, "element size must be 1, 2, 4 or 8");
+        g.side[side - 1].elem[i] = v[i];
+    }
+    return BFUSE_OK;
+}
+
+int initialize_kernel1(const int* I, const int* F, const int* O) { return init_side(0, I, F, O); }
+int initialize_kernel2(const int* I, const int* F, const int* O) { return init_side(1, I, F, O); }
+int finalize_kernel1(void) { return fini_side(0); }
+int finalize_kernel2(void) { return fini_side(1); }
+
+static int run_single(int idx, const void* I, const void* F, void* O, const int* Is, const int* Fs, const int* Os,
+                      const void* func, const unsigned* grid, const unsigned* block)
+{
+    int rc;
+    if (!I || !F || !O) return fail(BFUSE_ERR_ARG, "null host buffer");
+    if ((rc = check_shapes(idx, Is, Fs, Os))) return rc;
+    if ((rc = validate_mode(idx == 0 ? BFUSE_MODE_KERNEL1 : BFUSE_MODE_KERNEL2, func, grid, block, nullptr, nullptr, nullptr))) return rc;
+    Side& s = g.side[idx];
+    HIP_TRY(hipMemcpy(s.buf[0], I, s.bytes[0], hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(s.buf[1], F, s.bytes[1], hipMemcpyHostToDevice));
+    if ((rc = launch3(func, grid, block, idx, nullptr))) return rc;
+    if ((rc = sync_and_check(nullptr))) return rc;
+    HIP_TRY(hipMemcpy(O, s.buf[2], s.bytes[2], hipMemcpyDeviceToHost));
+    return BFUSE_OK;
+}
+
+int run_kernel1(const void* I, const void* F, void* O, const int* Is, const int* Fs, const int* Os,
+                bfuse_kernel3_fn func, const unsigned* grid, const unsigned* block, size_t)
+{
+    return run_single(0, I, F, O, Is, Fs, Os, (const void*)func, grid, block);
+}
+
+int run_kernel2(const void* I, const void* F, void* O, const int* Is, const int* Fs, const int* Os,
+                bfuse_kernel3_fn func, const unsigned* grid, const unsigned* block, size_t)
+{
+    return run_single(1, I, F, O, Is, Fs, Os, (const void*)func, grid, block);
+}
+
+static int upload_both(const void* I1, const void* F1, const void* I2, const void* F2)
+{
+    Side &a = g.side[0], &b = g.side[1];
+    HIP_TRY(hipMemcpy(a.buf[0], I1, a.bytes[0], hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(a.buf[1], F1, a.bytes[1], hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(b.buf[0], I2, b.bytes[0], hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(b.buf[1], F2, b.bytes[1], hipMemcpyHostToDevice));
+    return BFUSE_OK;
+}
+
+static int download_both(void* O1, void* O2)
+{
+    Side &a = g.side[0], &b = g.side[1];
+    HIP_TRY(hipMemcpy(O1, a.buf[2], a.bytes[2], hipMemcpyDeviceToHost));
+    HIP_TRY(hipMemcpy(O2, b.buf[2], b.bytes[2], hipMemcpyDeviceToHost));
+    return BFUSE_OK;
+}
+
+int run_parallel(const void* I1, const void* F1, void* O1, const void* I2, const void* F2, void* O2, const int* I1s,
+                 const int* F1s, const int* O1s, const int* I2s, const int* F2s, const int* O2s,
+                 bfuse_kernel3_fn func1, bfuse_kernel3_fn func2, const unsigned* g1, const unsigned* b1,
+                 const unsigned* g2, const unsigned* b2, size_t, size_t)
+{
+    int rc;
+    if (!I1 || !F1 || !O1 || !I2 || !F2 || !O2) return fail(BFUSE_ERR_ARG, "null host buffer");
+    if ((rc = check_shapes(0, I1s, F1s, O1s)) || (rc = check_shapes(1, I2s, F2s, O2s))) return rc;
+    if ((rc = validate_mode(BFUSE_MODE_PARALLEL, (const void*)func1, g1, b1, (const void*)func2, g2, b2))) return rc;
+    if ((rc = upload_both(I1, F1, I2, F2))) return rc;
+    if ((rc = enqueue_mode(BFUSE_MODE_PARALLEL, (const void*)func1, g1, b1, (const void*)func2, g2, b2, nullptr))) return rc;
+    if ((rc = sync_and_check(nullptr))) return rc;
+    return download_both(O1, O2);
+}
+
+int run_fuse(const void* I1, const void* F1, void* O1, const void* I2, const void* F2, void* O2, const int* I1s,
+             const int* F1s, const int* O1s, const int* I2s, const int* F2s, const int* O2s, bfuse_kernel6_fn func,
+             const unsigned* grid, const unsigned* block, size_t, size_t)
+{
+    int rc;
+    if (!I1 || !F1 || !O1 || !I2 || !F2 || !O2) return fail(BFUSE_ERR_ARG, "null host buffer");
+    if ((rc = check_shapes(0, I1s, F1s, O1s)) || (rc = check_shapes(1, I2s, F2s, O2s))) return rc;
+    const KernelEntry* e = entry_of((const void*)func);
+    if (!e || e->kind == kSingle) return fail(BFUSE_ERR_ARG, "func is not a fused kernel of this library");
+    const int mode = e->kind == kHfuse ? BFUSE_MODE_HFUSE : BFUSE_MODE_BFUSE;
+    if ((rc = validate_mode(mode, (const void*)func, grid, block, nullptr, nullptr, nullptr))) return rc;
+    if ((rc = upload_both(I1, F1, I2, F2))) return rc;
+    if ((rc = launch6((const void*)func, grid, block, nullptr))) return rc;
+    if ((rc = sync_and_check((const void*)func))) return rc;
+    return download_both(O1, O2);
+}
+
+// ---- device-resident operation and timing -------------------------------------------------
+int bfuse_upload(int side, const void* I, const void* F)
+{
+    if (side < 1 || side > 2) return fail(BFUSE_ERR_ARG, "side must be 1 or 2");
+    Side& s = g.side[side - 1];
+    if (!s.live) return fail(BFUSE_ERR_STATE, "kernel%d is not initialized", side);
+    if (!I || !F) return fail(BFUSE_ERR_ARG, "null host buffer");
+    HIP_TRY(hipMemcpy(s.buf[0], I, s.bytes[0], hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(s.buf[1], F, s.bytes[1], hipMemcpyHostToDevice));
+    return BFUSE_OK;
+}
+
+int bfuse_zero_output(int side)
+{
+    if (side < 1 || side > 2) return fail(BFUSE_ERR_ARG, "side must be 1 or 2");
+    Side& s = g.side[side - 1];
+    if (!s.live) return fail(BFUSE_ERR_STATE, "kernel%d is not initialized", side);
+    HIP_TRY(hipMemset(s.buf[2], 0, s.bytes[2]));
+    return BFUSE_OK;
+}
+
+int bfuse_download(int side, void* O)
+{
+    if (side < 1 || side > 2) return fail(BFUSE_ERR_ARG, "side must be 1 or 2");
+    Side& s = g.side[side - 1];
+    if (!s.live) return fail(BFUSE_ERR_STATE, "kernel%d is not initialized", side);
+    if (!O) return fail(BFUSE_ERR_ARG, "null host buffer");
+    HIP_TRY(hipDeviceSynchronize());
+    HIP_TRY(hipMemcpy(O, s.buf[2], s.bytes[2], hipMemcpyDeviceToHost));
+    return BFUSE_OK;
+}
+
+int bfuse_synchronize(void)
+{
+    if (!g.inited) return fail(BFUSE_ERR_STATE, "bfuse_init has not been called");
+    return sync_and_check(nullptr);
+}
+
+int bfuse_launch(int mode, const void* fa, const unsigned* ga, const unsigned* ba, const void* fb, const unsigned* gb,
+                 const unsigned* bb)
+{
+    int rc;
+    if ((rc = validate_mode(mode, fa, ga, ba, fb, gb, bb))) return rc;
+    return enqueue_mode(mode, fa, ga, ba, fb, gb, bb, nullptr);
+}
+
+int bfuse_time(int mode, const void* fa, const unsigned* ga, const unsigned* ba, const void* fb, const unsigned* gb,
+               const unsigned* bb, int warmup, int reps, float* us_total, float* us_a, float* us_b)
+{
+    int rc;
+    if (warmup < 0 || reps < 1 || reps > 100000 || !us_total) return fail(BFUSE_ERR_ARG, "bad repetition count or null output");
+    if ((rc = validate_mode(mode, fa, ga, ba, fb, gb, bb))) return rc;
+    const bool two = (mode == BFUSE_MODE_PARALLEL || mode == BFUSE_MODE_SERIAL);
+    for (int i = 0; i < warmup; ++i)
+        if ((rc = enqueue_mode(mode, fa, ga, ba, fb, gb, bb, nullptr))) return rc;
+    HIP_TRY(hipDeviceSynchronize());
+    std::vector<hipEvent_t> ev((size_t)reps * 4, nullptr);
+    const int per = two ? 4 : 2;
+    for (int r = 0; r < reps; ++r)
+        for (int j = 0; j < per; ++j) HIP_TRY(hipEventCreate(&ev[(size_t)r * 4 + j]));
+    for (int r = 0; r < reps; ++r)
+        if ((rc = enqueue_mode(mode, fa, ga, ba, fb, gb, bb, &ev[(size_t)r * 4]))) return rc;
+    if ((rc = sync_and_check(mode == BFUSE_MODE_HFUSE ? fa : nullptr))) return rc;
+    for (int r = 0; r < reps; ++r) {
+        hipEvent_t* e = &ev[(size_t)r * 4];
+        float ms_a = 0.f;
+        HIP_TRY(hipEventElapsedTime(&ms_a, e[0], e[1]));
+        if (us_a) us_a[r] = ms_a * 1000.f;
+        if (!two) {
+            us_total[r] = ms_a * 1000.f;
+            if (us_b) us_b[r] = 0.f;
+        } else {
+            float ms_b = 0.f, s_ab = 0.f;
+            HIP_TRY(hipEventElapsedTime(&ms_b, e[2], e[3]));
+            HIP_TRY(hipEventElapsedTime(&s_ab, e[0], e[2]));  // start_b - start_a (may be negative)
+            if (us_b) us_b[r] = ms_b * 1000.f;
+            // first start -> last end (scripts/analyze_test_suite.py:142-154)
+            const float first = s_ab < 0.f ? s_ab : 0.f;
+            const float end_a = ms_a, end_b = s_ab + ms_b;
+            us_total[r] = ((end_a > end_b ? end_a : end_b) - first) * 1000.f;
+        }
+    }
+    for (auto e : ev)
+        if (e) HIP_TRY(hipEventDestroy(e));
+    return BFUSE_OK;
+}
+
+int bfuse_time_batched(int mode, const void* fa, const unsigned* ga, const unsigned* ba, const void* fb,
+                       const unsigned* gb, const unsigned* bb, int warmup, int reps, float* us_per_launch)
+{
+    int rc;
+    if (warmup < 0 || reps < 1 || !us_per_launch) return fail(BFUSE_ERR_ARG, "bad repetition count or null output");
+    if (mode == BFUSE_MODE_PARALLEL) return fail(BFUSE_ERR_ARG, "batched timing is single-stream");
+    if ((rc = validate_mode(mode, fa, ga, ba, fb, gb, bb))) return rc;
+    for (int i = 0; i < warmup; ++i)
+        if ((rc = enqueue_mode(mode, fa, ga, ba, fb, gb, bb, nullptr))) return rc;
+    HIP_TRY(hipDeviceSynchronize());
+    hipEvent_t e0, e1;
+    HIP_TRY(hipEventCreate(&e0));
+    HIP_TRY(hipEventCreate(&e1));
+    HIP_TRY(hipEventRecord(e0, nullptr));
+    for (int r = 0; r < reps; ++r)
+        if ((rc = enqueue_mode(mode, fa, ga, ba, fb, gb, bb, nullptr))) return rc;
+    HIP_TRY(hipEventRecord(e1, nullptr));
+    if ((rc = sync_and_check(mode == BFUSE_MODE_HFUSE ? fa : nullptr))) return rc;
+    float ms = 0.f;
+    HIP_TRY(hipEventElapsedTime(&ms, e0, e1));
+    *us_per_launch = ms * 1000.f / (float)reps;
+    HIP_TRY(hipEventDestroy(e0));
+    HIP_TRY(hipEventDestroy(e1));
+    return BFUSE_OK;
+}
+
+// ---- synthetic inputs and checks ------------------------------------------------------------
+void bfuse_fill_uniform(unsigned long long seed, size_t n, float lo, float hi, float* out)
+{
+    for (size_t i = 0; i < n; ++i) out[i] = (float)((double)lo + ((double)hi - (double)lo) * u01(seed, i));
+}
+
+void bfuse_fill_normal(unsigned long long seed, size_t n, float mean, float std, float* out)
+{
+    const double two_pi = 6.283185307179586476925;
+    for (size_t i = 0; i < n; ++i) {
+        const double u1 = u01(seed, 2 * (unsigned long long)i), u2 = u01(seed, 2 * (unsigned long long)i + 1);
+        out[i] = (float)((double)mean + (double)std * std::sqrt(-2.0 * std::log(u1)) * std::cos(two_pi * u2));
+    }
+}
+
+void bfuse_f32_to_bf16(size_t n, const float* in, unsigned short* out)
+{
+    for (size_t i = 0; i < n; ++i) {
+        unsigned u;
+        memcpy(&u, &in[i], 4);
+        if ((u & 0x7fffffffu) > 0x7f800000u) {
+            out[i] = (unsigned short)((u >> 16) | 0x0040u);
+        } else {
+            u += 0x7fffu + ((u >> 16) & 1u);
+            out[i] = (unsigned short)(u >> 16);
+        }
+    }
+}
+
+void bfuse_bf16_to_f32(size_t n, const unsigned short* in, float* out)
+{
+    for (size_t i = 0; i < n; ++i) {
+        const unsigned u = (unsigned)in[i] << 16;
+        memcpy(&out[i], &u, 4);
+    }
+}
+
+long bfuse_check_matrix(const float* O, const float* A, size_t count, float eps)
+{
+    long bad = 0;
+    for (size_t i = 0; i < count; ++i) {
+        const float o = O[i], a = A[i];
+        if (std::isnan(o) || std::isnan(a)) {
+            bad += !(std::isnan(o) && std::isnan(a));
+            continue;
+        }
+        if (std::fabs(o - a) > eps && (a == 0.f || std::fabs((o - a) / a) > eps)) ++bad;
+    }
+    return bad;
+}
+
+}  // extern "C"

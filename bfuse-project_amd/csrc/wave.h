@@ -1,0 +1,89 @@
+// Wave64 primitives for gfx950: DPP reductions and the two synchronisation policies an
+// operator body can be instantiated with.
+#pragma once
+#include <hip/hip_runtime.h>
+
+namespace bfuse {
+
+// ---- DPP cross-lane moves -------------------------------------------------------------
+// dpp_ctrl encodings (GCN3+/CDNA): quad_perm 0x00-0xff, row_mirror 0x140, row_half_mirror 0x141.
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v)
+{
+    const int i = __builtin_bit_cast(int, v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(i, i, CTRL, 0xf, 0xf, false));
+}
+
+struct SumOp {
+    __device__ __forceinline__ float operator()(float a, float b) const { return a + b; }
+};
+struct MaxOp {
+    __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); }
+};
+
+// All 64 lanes end up holding the reduction over the wave.  Inside each row of 16 lanes the
+// reduction is a butterfly on DPP (no LDS traffic); the four row results are combined in
+// lane order 0,16,32,48 through scalar registers, so the operation order is fixed and is
+// the same in every kernel the body is instantiated in.
+template <class Op>
+__device__ __forceinline__ float wave_reduce(float v, Op op)
+{
+    v = op(v, dpp_mov<0xB1>(v));   // quad_perm [1,0,3,2]
+    v = op(v, dpp_mov<0x4E>(v));   // quad_perm [2,3,0,1]
+    v = op(v, dpp_mov<0x141>(v));  // row_half_mirror
+    v = op(v, dpp_mov<0x140>(v));  // row_mirror
+    const int i = __builtin_bit_cast(int, v);
+    const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(i, 0));
+    const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(i, 16));
+    const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(i, 32));
+    const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(i, 48));
+    return op(op(r0, r1), op(r2, r3));
+}
+
+__device__ __forceinline__ float wave_sum(float v) { return wave_reduce(v, SumOp{}); }
+__device__ __forceinline__ float wave_max(float v) { return wave_reduce(v, MaxOp{}); }
+
+// ---- synchronisation policies ---------------------------------------------------------
+// Counts waits that gave up (see GroupSync); read back by the host after a fused launch.
+static __device__ unsigned int g_sync_timeouts;
+
+// Whole-workgroup barrier: standalone kernels and block-fused kernels (each workgroup runs
+// one operator; waves outside the operator's thread range have already exited, and the
+// hardware barrier only counts waves that are still alive).
+struct BlockSync {
+    __device__ __forceinline__ void operator()() const { __syncthreads(); }
+};
+
+// Barrier over the waves of ONE side of a horizontally fused workgroup.  gfx950 has no
+// partial-workgroup barrier (s_barrier always spans the workgroup), so the side's waves
+// meet on an LDS counter: lane 0 of each wave adds 1, then the wave polls until the counter
+// reaches waves * epoch.  All waves of a workgroup are resident on one CU for the whole
+// kernel, so the wait cannot depend on a wave that has not been scheduled.  The poll is
+// bounded: a side whose waves disagree on the number of barriers gives up after
+// kSpinLimit polls, records it in g_sync_timeouts and carries on, so the grid always drains.
+struct GroupSync {
+    unsigned int* counter;  // in LDS, zeroed before the sides diverge
+    unsigned int waves;
+    unsigned int epoch;
+    static constexpr unsigned int kSpinLimit = 1u << 22;
+
+    __device__ __forceinline__ void operator()()
+    {
+        ++epoch;
+        const unsigned int target = waves * epoch;
+        // order this wave's earlier LDS writes before its arrival
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        if ((threadIdx.x & 63) == 0) atomicAdd(counter, 1u);
+        unsigned int spins = 0;
+        while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < target) {
+            __builtin_amdgcn_s_sleep(1);
+            if (++spins == kSpinLimit) {
+                if ((threadIdx.x & 63) == 0) atomicAdd(&g_sync_timeouts, 1u);
+                break;
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    }
+};
+
+}  // namespace bfuse

@@ -1,0 +1,230 @@
+"""Host-side mirror of the reference harness (test-utils/test-suite-files/operation_h.py:9-27,
+operation_cu.py:123-256): initialize / run_kernel1 / run_kernel2 / run_parallel / run_fuse /
+finalize over numpy buffers, plus the device-resident launch and GPU-side timing entry points.
+"""
+import ctypes as C
+from dataclasses import dataclass
+from typing import List, Optional, Sequence
+
+import numpy as np
+
+from . import _lib
+
+MODES = {"kernel1": 0, "kernel2": 1, "parallel": 2, "hfuse": 3, "bfuse": 4, "serial": 5}
+
+
+@dataclass
+class KernelHandle:
+    name: str
+    func: int
+    kind: int                 # 0 single, 1 bfuse, 2 hfuse
+    grid: tuple
+    block: tuple
+    has_barriers: bool
+    regs: int
+    lds_bytes: int
+    shapes: tuple             # ((4 ints) x 3) for single kernels
+    elem_bytes: tuple
+    sides: tuple
+    pattern: int
+    p0: int
+    p1: int
+
+
+def _handle(ci: "_lib.KernelInfoC") -> KernelHandle:
+    return KernelHandle(ci.name.decode(), ci.func, ci.kind, tuple(ci.grid), tuple(ci.block), bool(ci.has_barriers),
+                        ci.regs, ci.lds_bytes, tuple(tuple(s) for s in ci.shape), tuple(ci.elem_bytes),
+                        (ci.side[0].value.decode(), ci.side[1].value.decode()), ci.pattern, ci.p0, ci.p1)
+
+
+def kernel_info(name: str) -> KernelHandle:
+    ci = _lib.KernelInfoC()
+    _lib.check(_lib.lib().bfuse_kernel_find(name.encode(), C.byref(ci)))
+    return _handle(ci)
+
+
+def list_kernels() -> List[KernelHandle]:
+    l = _lib.lib()
+    out = []
+    for i in range(l.bfuse_kernel_count()):
+        ci = _lib.KernelInfoC()
+        _lib.check(l.bfuse_kernel_at(i, C.byref(ci)))
+        out.append(_handle(ci))
+    return out
+
+
+def _i4(shape):
+    s = list(shape) + [1] * (4 - len(shape))
+    return (C.c_int * 4)(*s)
+
+
+def _u3(v):
+    return (C.c_uint * 3)(*v)
+
+
+_DT = {4: np.float32, 2: np.uint16}
+
+
+class Operation:
+    """One pair of sides with their device buffers (the reference keeps them in file-scope
+    globals; so does the library -- one Operation may be live at a time)."""
+
+    def __init__(self, k1: str, k2: str, device: int = 0):
+        self.l = _lib.lib()
+        _lib.check(self.l.bfuse_init(device))
+        self.k = [kernel_info(k1), kernel_info(k2)]
+        for side, k in enumerate(self.k, 1):
+            if k.kind != 0:
+                raise ValueError(f"{k.name} is a fused kernel; sides must be standalone kernels")
+            _lib.check(self.l.bfuse_set_elem_bytes(side, *k.elem_bytes))
+        self.shapes = [[_i4(s) for s in k.shapes] for k in self.k]
+        _lib.check(self.l.initialize_kernel1(*self.shapes[0]))
+        try:
+            _lib.check(self.l.initialize_kernel2(*self.shapes[1]))
+        except Exception:
+            self.l.finalize_kernel1()
+            raise
+        self.live = True
+
+    # -- context management ------------------------------------------------------------
+    def close(self):
+        if self.live:
+            self.live = False
+            _lib.check(self.l.finalize_kernel1())
+            _lib.check(self.l.finalize_kernel2())
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    # -- helpers -----------------------------------------------------------------------
+    def _host(self, side, idx, arr):
+        k = self.k[side]
+        dt = _DT[k.elem_bytes[idx]]
+        a = np.ascontiguousarray(arr, dtype=dt)
+        want = int(np.prod(k.shapes[idx]))
+        if a.size != want:
+            raise ValueError(f"{k.name}: tensor {idx} has {a.size} elements, kernel expects {want}")
+        return a
+
+    def empty_output(self, side):
+        k = self.k[side]
+        return np.empty(tuple(d for d in k.shapes[2]), _DT[k.elem_bytes[2]])
+
+    def fused(self, kind: str, suffix: str = "") -> KernelHandle:
+        return kernel_info(f"{self.k[0].name}_{self.k[1].name}_fused_{kind}{suffix}")
+
+    # -- operation.h mirror (H2D, launch, sync, D2H) ---------------------------------------
+    def run_kernel(self, side: int, I, F) -> np.ndarray:
+        k = self.k[side]
+        I, F = self._host(side, 0, I), self._host(side, 1, F)
+        O = self.empty_output(side)
+        fn = self.l.run_kernel1 if side == 0 else self.l.run_kernel2
+        _lib.check(fn(I.ctypes.data, F.ctypes.data, O.ctypes.data, *self.shapes[side], k.func, _u3(k.grid), _u3(k.block), side))
+        return O
+
+    def run_parallel(self, I1, F1, I2, F2):
+        a, b = self.k
+        I1, F1, I2, F2 = self._host(0, 0, I1), self._host(0, 1, F1), self._host(1, 0, I2), self._host(1, 1, F2)
+        O1, O2 = self.empty_output(0), self.empty_output(1)
+        _lib.check(self.l.run_parallel(I1.ctypes.data, F1.ctypes.data, O1.ctypes.data, I2.ctypes.data, F2.ctypes.data,
+                                       O2.ctypes.data, *self.shapes[0], *self.shapes[1], a.func, b.func,
+                                       _u3(a.grid), _u3(a.block), _u3(b.grid), _u3(b.block), 0, 0))
+        return O1, O2
+
+    def run_fuse(self, fused: KernelHandle, I1, F1, I2, F2):
+        I1, F1, I2, F2 = self._host(0, 0, I1), self._host(0, 1, F1), self._host(1, 0, I2), self._host(1, 1, F2)
+        O1, O2 = self.empty_output(0), self.empty_output(1)
+        _lib.check(self.l.run_fuse(I1.ctypes.data, F1.ctypes.data, O1.ctypes.data, I2.ctypes.data, F2.ctypes.data,
+                                   O2.ctypes.data, *self.shapes[0], *self.shapes[1], fused.func,
+                                   _u3(fused.grid), _u3(fused.block), 0, 0))
+        return O1, O2
+
+    # -- device-resident ---------------------------------------------------------------
+    def upload(self, side: int, I, F):
+        I, F = self._host(side, 0, I), self._host(side, 1, F)
+        _lib.check(self.l.bfuse_upload(side + 1, I.ctypes.data, F.ctypes.data))
+
+    def zero_outputs(self):
+        _lib.check(self.l.bfuse_zero_output(1))
+        _lib.check(self.l.bfuse_zero_output(2))
+
+    def download(self, side: int) -> np.ndarray:
+        O = self.empty_output(side)
+        _lib.check(self.l.bfuse_download(side + 1, O.ctypes.data))
+        return O
+
+    def _mode_args(self, mode: str, fused: Optional[KernelHandle]):
+        a, b = self.k
+        if mode == "kernel1":
+            return (a.func, _u3(a.grid), _u3(a.block), None, None, None)
+        if mode == "kernel2":
+            return (b.func, _u3(b.grid), _u3(b.block), None, None, None)
+        if mode in ("parallel", "serial"):
+            return (a.func, _u3(a.grid), _u3(a.block), b.func, _u3(b.grid), _u3(b.block))
+        if fused is None:
+            raise ValueError("fused kernel handle required")
+        return (fused.func, _u3(fused.grid), _u3(fused.block), None, None, None)
+
+    def launch(self, mode: str, fused: Optional[KernelHandle] = None):
+        _lib.check(self.l.bfuse_launch(MODES[mode], *self._mode_args(mode, fused)))
+
+    def synchronize(self):
+        _lib.check(self.l.bfuse_synchronize())
+
+    def time(self, mode: str, fused: Optional[KernelHandle] = None, warmup: int = 3, reps: int = 30):
+        """GPU-side microseconds per repetition: (total, kernel_a, kernel_b) arrays.  The default
+        3 + 30 is the reference's sampling (scripts/profile_test_suite.py:10-11)."""
+        tot, ta, tb = (np.zeros(reps, np.float32) for _ in range(3))
+        fp = C.POINTER(C.c_float)
+        _lib.check(self.l.bfuse_time(MODES[mode], *self._mode_args(mode, fused), warmup, reps,
+                                     tot.ctypes.data_as(fp), ta.ctypes.data_as(fp), tb.ctypes.data_as(fp)))
+        return tot, ta, tb
+
+    def time_batched(self, mode: str, fused: Optional[KernelHandle] = None, warmup: int = 3, reps: int = 30) -> float:
+        us = C.c_float()
+        _lib.check(self.l.bfuse_time_batched(MODES[mode], *self._mode_args(mode, fused), warmup, reps, C.byref(us)))
+        return us.value
+
+
+# ---- synthetic inputs ---------------------------------------------------------------------
+def fill_uniform(seed: int, n: int, lo: float, hi: float) -> np.ndarray:
+    out = np.empty(n, np.float32)
+    _lib.lib().bfuse_fill_uniform(seed, n, lo, hi, out.ctypes.data)
+    return out
+
+
+def fill_normal(seed: int, n: int, mean: float, std: float) -> np.ndarray:
+    out = np.empty(n, np.float32)
+    _lib.lib().bfuse_fill_normal(seed, n, mean, std, out.ctypes.data)
+    return out
+
+
+def f32_to_bf16(x: np.ndarray) -> np.ndarray:
+    x = np.ascontiguousarray(x, np.float32)
+    out = np.empty(x.shape, np.uint16)
+    _lib.lib().bfuse_f32_to_bf16(x.size, x.ctypes.data, out.ctypes.data)
+    return out
+
+
+def bf16_to_f32(x: np.ndarray) -> np.ndarray:
+    x = np.ascontiguousarray(x, np.uint16)
+    out = np.empty(x.shape, np.float32)
+    _lib.lib().bfuse_bf16_to_f32(x.size, x.ctypes.data, out.ctypes.data)
+    return out
+
+
+def check_matrix(o: np.ndarray, o_ans: np.ndarray, eps: float = 1e-3) -> int:
+    """check_matrix of the reference (utils_cc.py:52-85): number of wrong elements."""
+    o, a = np.ascontiguousarray(o, np.float32), np.ascontiguousarray(o_ans, np.float32)
+    assert o.size == a.size
+    return _lib.lib().bfuse_check_matrix(o.ctypes.data, a.ctypes.data, o.size, eps)
+
+
+def device_name() -> str:
+    buf = C.create_string_buffer(256)
+    cus, lds, wave = C.c_int(), C.c_int(), C.c_int()
+    _lib.check(_lib.lib().bfuse_device_info(buf, 256, C.byref(cus), C.byref(lds), C.byref(wave)))
+    return f"{buf.value.decode()} CUs={cus.value} wave={wave.value}"

@@ -1,0 +1,207 @@
+/*
+ * libbfuse_rt -- C ABI of the MI355X fused-pair runtime.
+ *
+ * Plain C: pointers, ints and POD structs only.  Every function returns 0 on success and a
+ * negative code on failure (bfuse_last_error() holds the text) unless stated otherwise.
+ * The library is not re-entrant: like the reference harness it keeps one set of device
+ * buffers and two streams in file-scope state (operation_cu.py:123-126).
+ *
+ * Citations are paths in the reference repository (jiny0ung97/bfuse-project).
+ */
+#ifndef BFUSE_RT_H
+#define BFUSE_RT_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------------------------------
+ * Status
+ * ---------------------------------------------------------------------------------------- */
+enum {
+    BFUSE_OK = 0,
+    BFUSE_ERR_ARG = -1,      /* bad argument (null pointer, unknown name, shape mismatch) */
+    BFUSE_ERR_HIP = -2,      /* a HIP runtime call failed; replaces CHECK_CUDA's exit(EXIT_FAILURE),
+                                operation_cu.py:111-121 */
+    BFUSE_ERR_STATE = -3,    /* called before bfuse_init / initialize_kernelN */
+    BFUSE_ERR_SYNC = -4      /* a horizontally fused side gave up waiting on its LDS barrier */
+};
+const char* bfuse_last_error(void);
+
+/* Selects the device and creates the two streams the harness uses (S1, S2 of
+ * operation_cu.py:126).  Fails if no HIP device is present: there is no CPU fallback. */
+int bfuse_init(int device);
+int bfuse_shutdown(void);
+/* name, CU count, LDS bytes per workgroup, wavefront size of the selected device */
+int bfuse_device_info(char* name, size_t name_len, int* compute_units, int* lds_bytes, int* wave_size);
+
+/* ------------------------------------------------------------------------------------------
+ * Fusion index maps -- horizontal-fuser/src/Algorithms.cc.  Pure host arithmetic, usable
+ * without a GPU.  The same code is compiled into the fused kernels.
+ * ---------------------------------------------------------------------------------------- */
+#define BFUSE_MAX_KERNELS 4
+#define BFUSE_MAX_SEGMENTS 8
+
+/* GridDim / BlockDim of one kernel -- horizontal-fuser/include/fuse/Contexts.h:13-26 */
+typedef struct { int grid[3]; int block[3]; } bfuse_launch_dims;
+
+typedef struct { int kern, off, width, base; } bfuse_slot;
+typedef struct { int lo, hi, period, n_slot; bfuse_slot slot[BFUSE_MAX_KERNELS]; } bfuse_segment;
+/* Block-fusion dispatch table: fused block `bid` in segment [lo,hi) belongs to the slot that
+ * owns (bid-lo) % period; virt = base + ((bid-lo)/period)*width + ((bid-lo)%period - off). */
+typedef struct {
+    int n_kernels, n_seg;
+    bfuse_segment seg[BFUSE_MAX_SEGMENTS];
+    int fused_grid, fused_block;
+    int threads[BFUSE_MAX_KERNELS];
+} bfuse_block_plan;
+
+typedef struct {
+    int n_kernels;
+    int thr_lo[BFUSE_MAX_KERNELS], thr_hi[BFUSE_MAX_KERNELS];
+    int blocks[BFUSE_MAX_KERNELS];
+    int fused_grid, fused_block;
+} bfuse_thread_plan;
+
+enum {
+    BFUSE_PATTERN_ZIGZAG = 0,        /* coarseInterleaveWithoutSMPattern2, Algorithms.cc:528-739; p0 = M, p1 = N */
+    BFUSE_PATTERN_PROPORTIONAL = 1,  /* coarseInterleaveWithoutSMPattern,  Algorithms.cc:319-526; p0 = MinOption */
+    BFUSE_PATTERN_CHUNKED = 2,       /* coarseInterleavePattern,           Algorithms.cc:118-317; p0 = TotalSM */
+    BFUSE_PATTERN_RANGES = 3         /* blockIdx ranges only (the tail branches, Algorithms.cc:661-685) */
+};
+
+/* hfusePattern, Algorithms.cc:19-116.  pad = 32 reproduces the reference, 64 is what the
+ * gfx950 kernels use (one wavefront never holds threads of two operators). */
+int bfuse_plan_threads(int n, const bfuse_launch_dims* kernels, int pad, bfuse_thread_plan* out);
+int bfuse_plan_blocks(int pattern, int n, const bfuse_launch_dims* kernels, int p0, int p1,
+                      bfuse_block_plan* out);
+/* Return the kernel index owning the id (or -1 if none) */
+int bfuse_map_block(const bfuse_block_plan* plan, int bid, int* virt_block);
+int bfuse_map_thread(const bfuse_thread_plan* plan, int bid, int tid, int* local_tid);
+/* Evaluates bfuse_map_block for bid in [lo,hi) ON THE GPU with the device build of the map
+ * (one thread per fused block) and copies the tables back. */
+int bfuse_map_blocks_device(const bfuse_block_plan* plan, int lo, int hi, int* kernel_out, int* virt_out);
+
+/* ------------------------------------------------------------------------------------------
+ * Kernel registry -- the role of the reference's generated macro.h tables
+ * (test-utils/test-suite-files/macro_h.py:79-198) and of kernels.yaml / {b,h}fuse_kernels.yaml
+ * (horizontal-fuser/include/fuse/Utils.h:70-112).
+ * ---------------------------------------------------------------------------------------- */
+enum { BFUSE_KIND_SINGLE = 0, BFUSE_KIND_BFUSE = 1, BFUSE_KIND_HFUSE = 2 };
+
+typedef struct {
+    char name[128];          /* KernelName; fused: <K1>_<K2>_fused_{bfuse,hfuse} (Contexts.cc:56-92) */
+    const void* func;        /* launch handle: pass as `func` to run_kernelN / run_fuse */
+    int kind;
+    unsigned grid[3], block[3];
+    int has_barriers;        /* KernelInfo.HasBarriers */
+    int regs;                /* KernelInfo.Reg: VGPRs per lane from the code object (-1 without a GPU) */
+    int lds_bytes;           /* static LDS of the kernel (-1 without a GPU) */
+    int shape[3][4];         /* single kernels: I, F, O shapes, padded with 1s */
+    int elem_bytes[3];
+    char side[2][64];        /* fused kernels: the two standalone kernels */
+    int pattern, p0, p1;     /* bfuse kernels: dispatch pattern */
+} bfuse_kernel_info;
+
+int bfuse_kernel_count(void);
+int bfuse_kernel_at(int index, bfuse_kernel_info* out);
+int bfuse_kernel_find(const char* name, bfuse_kernel_info* out);
+
+/* ------------------------------------------------------------------------------------------
+ * Harness functions -- test-utils/test-suite-files/operation_h.py:9-27.  Same names and
+ * argument meaning.  Differences: data pointers are void* (bf16 sides), an int status is
+ * returned instead of exit(), and `func` is the registry handle of a kernel with the
+ * reference's three- / six-pointer ABI.  K / K1 / K2 (the reference's switch index into the
+ * fusion sets) are accepted and ignored.
+ * ---------------------------------------------------------------------------------------- */
+typedef void (*bfuse_kernel3_fn)(const void*, const void*, void*);
+typedef void (*bfuse_kernel6_fn)(const void*, const void*, void*, const void*, const void*, void*);
+
+/* element sizes of side 1 / side 2 buffers (default 4 = float, as in the reference) */
+int bfuse_set_elem_bytes(int side, int i_bytes, int f_bytes, int o_bytes);
+
+/* device alloc of I/F/O for one side + stream create -- operation_cu.py:128-144 */
+int initialize_kernel1(const int* I_shape, const int* F_shape, const int* O_shape);
+int initialize_kernel2(const int* I_shape, const int* F_shape, const int* O_shape);
+/* operation_cu.py:146-162 */
+int finalize_kernel1(void);
+int finalize_kernel2(void);
+/* H2D of I,F; launch on the default stream; device sync; D2H of O -- operation_cu.py:164-201 */
+int run_kernel1(const void* I, const void* F, void* O, const int* I_shape, const int* F_shape,
+                const int* O_shape, bfuse_kernel3_fn func, const unsigned* gridDim,
+                const unsigned* blockDim, size_t K);
+int run_kernel2(const void* I, const void* F, void* O, const int* I_shape, const int* F_shape,
+                const int* O_shape, bfuse_kernel3_fn func, const unsigned* gridDim,
+                const unsigned* blockDim, size_t K);
+/* both kernels, one per stream -- operation_cu.py:203-229 */
+int run_parallel(const void* I1, const void* F1, void* O1, const void* I2, const void* F2, void* O2,
+                 const int* I1_shape, const int* F1_shape, const int* O1_shape, const int* I2_shape,
+                 const int* F2_shape, const int* O2_shape, bfuse_kernel3_fn func1, bfuse_kernel3_fn func2,
+                 const unsigned* gridDim1, const unsigned* blockDim1, const unsigned* gridDim2,
+                 const unsigned* blockDim2, size_t K1, size_t K2);
+/* one fused kernel over both sides' buffers -- operation_cu.py:231-256 */
+int run_fuse(const void* I1, const void* F1, void* O1, const void* I2, const void* F2, void* O2,
+             const int* I1_shape, const int* F1_shape, const int* O1_shape, const int* I2_shape,
+             const int* F2_shape, const int* O2_shape, bfuse_kernel6_fn func, const unsigned* gridDim,
+             const unsigned* blockDim, size_t K1, size_t K2);
+
+/* ------------------------------------------------------------------------------------------
+ * Device-resident operation and GPU-side timing.  The reference copies H2D/D2H around every
+ * launch but reports only the profiler's GPU-side kernel durations
+ * (scripts/profile_test_suite.py:10-11,106-109; scripts/analyze_test_suite.py:103-161);
+ * these entry points keep the operands in HBM and return those durations directly.
+ * ---------------------------------------------------------------------------------------- */
+int bfuse_upload(int side, const void* I, const void* F);   /* side 1 or 2 */
+int bfuse_zero_output(int side);
+int bfuse_download(int side, void* O);
+int bfuse_synchronize(void);
+
+enum {
+    BFUSE_MODE_KERNEL1 = 0,   /* the reference CLI's T = 0..4 (main_cc.py:22-36) */
+    BFUSE_MODE_KERNEL2 = 1,
+    BFUSE_MODE_PARALLEL = 2,  /* two streams */
+    BFUSE_MODE_HFUSE = 3,
+    BFUSE_MODE_BFUSE = 4,
+    BFUSE_MODE_SERIAL = 5     /* kernel 1 then kernel 2 on one stream, no host sync in between */
+};
+
+/* One asynchronous launch of `mode` over the resident buffers (no copies, no sync).
+ * func_a/grid_a/block_a: kernel 1 (modes 0,2,5) or the fused kernel (modes 3,4) or kernel 2 (mode 1);
+ * func_b/...: kernel 2 (modes 2,5). */
+int bfuse_launch(int mode, const void* func_a, const unsigned* grid_a, const unsigned* block_a,
+                 const void* func_b, const unsigned* grid_b, const unsigned* block_b);
+
+/* `warmup` untimed + `reps` timed launches of `mode`; GPU timestamps of each kernel's own
+ * start and end.  us_total[r] = first kernel start -> last kernel end of repetition r;
+ * us_a[r], us_b[r] = duration of each kernel (us_b only for modes 2 and 5; may be NULL). */
+int bfuse_time(int mode, const void* func_a, const unsigned* grid_a, const unsigned* block_a,
+               const void* func_b, const unsigned* grid_b, const unsigned* block_b, int warmup, int reps,
+               float* us_total, float* us_a, float* us_b);
+
+/* Wall-clock throughput: `reps` launches of `mode` enqueued back to back between two stream
+ * events; returns the mean microseconds per launch (includes dispatch gaps). */
+int bfuse_time_batched(int mode, const void* func_a, const unsigned* grid_a, const unsigned* block_a,
+                       const void* func_b, const unsigned* grid_b, const unsigned* block_b, int warmup,
+                       int reps, float* us_per_launch);
+
+/* ------------------------------------------------------------------------------------------
+ * Seeded synthetic inputs (host side): splitmix64 counter stream -> U[lo,hi) or Box-Muller
+ * N(mean,std).  Element i depends only on (seed, i).
+ * ---------------------------------------------------------------------------------------- */
+void bfuse_fill_uniform(unsigned long long seed, size_t n, float lo, float hi, float* out);
+void bfuse_fill_normal(unsigned long long seed, size_t n, float mean, float std, float* out);
+/* round-to-nearest-even conversions for bf16 buffers */
+void bfuse_f32_to_bf16(size_t n, const float* in, unsigned short* out);
+void bfuse_bf16_to_f32(size_t n, const unsigned short* in, float* out);
+
+/* The reference's acceptance rule, check_matrix (test-utils/test-suite-files/utils_cc.py:52-85):
+ * element wrong iff |o-a| > eps and (a == 0 or |o-a|/|a| > eps).  Returns the number of wrong
+ * elements (NaN mismatches count as wrong). */
+long bfuse_check_matrix(const float* O, const float* O_ans, size_t count, float eps);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BFUSE_RT_H */
