@@ -29,6 +29,11 @@
 
 namespace bfuse {
 
+// Every kernel is compiled to fit two waves per SIMD (at most 256 of the 512 VGPRs): a fused
+// kernel allocates the larger side's registers for BOTH sides' waves, and with more than
+// 256 a memory-bound workgroup could never be resident next to a GEMM workgroup.
+constexpr int kMinWavesPerEu = 2;
+
 template <class Op>
 __device__ __forceinline__ void single_body(const void* I, const void* F, void* O)
 {
@@ -170,7 +175,7 @@ KernelEntry make_fused_entry(const char* name, const void* func, int kind, const
     }
 
 #define BFUSE_KERNEL(NAME, OP, IDESC, FDESC, ODESC)                                                  \
-    extern "C" __global__ __launch_bounds__(OP::THREADS) void NAME(const void* __restrict__ I,       \
+    extern "C" __global__ __launch_bounds__(OP::THREADS, bfuse::kMinWavesPerEu) void NAME(const void* __restrict__ I,       \
                                                                    const void* __restrict__ F,       \
                                                                    void* __restrict__ O)             \
     {                                                                                               \
@@ -181,7 +186,7 @@ KernelEntry make_fused_entry(const char* name, const void* func, int kind, const
         &bfuse_module_read_sync_timeouts));
 
 #define BFUSE_BFUSE_KERNEL(K1, OP1, K2, OP2, SUFFIX, PATTERN, P0, P1)                                \
-    extern "C" __global__ __launch_bounds__((bfuse::BfusePair<OP1, OP2, PATTERN, P0, P1>::THREADS))  \
+    extern "C" __global__ __launch_bounds__((bfuse::BfusePair<OP1, OP2, PATTERN, P0, P1>::THREADS), bfuse::kMinWavesPerEu)  \
     void K1##_##K2##_fused_bfuse##SUFFIX(const void* __restrict__ I1, const void* __restrict__ F1,   \
                                          void* __restrict__ O1, const void* __restrict__ I2,         \
                                          const void* __restrict__ F2, void* __restrict__ O2)         \
@@ -195,7 +200,7 @@ KernelEntry make_fused_entry(const char* name, const void* func, int kind, const
             &bfuse_module_read_sync_timeouts));
 
 #define BFUSE_HFUSE_KERNEL(K1, OP1, K2, OP2)                                                         \
-    extern "C" __global__ __launch_bounds__((bfuse::HfusePair<OP1, OP2>::THREADS))                   \
+    extern "C" __global__ __launch_bounds__((bfuse::HfusePair<OP1, OP2>::THREADS), bfuse::kMinWavesPerEu)                  \
     void K1##_##K2##_fused_hfuse(const void* __restrict__ I1, const void* __restrict__ F1,           \
                                  void* __restrict__ O1, const void* __restrict__ I2,                 \
                                  const void* __restrict__ F2, void* __restrict__ O2)                 \

@@ -1,0 +1,22 @@
+// Pair 5 (Llama-3-8B shapes, seq 512): bf16 gate-projection GEMM [512x4096].[4096x14336]
+// (fp32 accumulate) block-fused with RMSNorm over [512x4096] bf16 followed by RoPE on
+// 32 heads x 128.
+#include "fuse.h"
+#include "ops_gemm_bf16.h"
+#include "ops_rowwise.h"
+
+using namespace bfuse;
+
+BFUSE_MODULE_PROLOGUE()
+
+using GemmGate = GemmBf16NT<512, 14336, 4096, 128, 224>;    // 4 x 64 = 256 workgroups
+using NormRope1 = RmsNormRope<512, 32, 128, 1>;             // 512 one-wave workgroups
+using NormRope4 = RmsNormRope<512, 32, 128, 4>;             // 128 four-wave workgroups
+
+BFUSE_KERNEL(gemm_bf16_512x4096x14336, GemmGate, ({{512, 4096, 1, 1}, 2}), ({{14336, 4096, 1, 1}, 2}), ({{512, 14336, 1, 1}, 2}))
+BFUSE_KERNEL(rmsnorm_rope_bf16_512x4096, NormRope1, ({{512, 4096, 1, 1}, 2}), ({{(int)NormRope1::F_BYTES, 1, 1, 1}, 1}), ({{512, 4096, 1, 1}, 2}))
+BFUSE_KERNEL(rmsnorm_rope_bf16_512x4096_w4, NormRope4, ({{512, 4096, 1, 1}, 2}), ({{(int)NormRope4::F_BYTES, 1, 1, 1}, 1}), ({{512, 4096, 1, 1}, 2}))
+
+BFUSE_BFUSE_KERNEL(gemm_bf16_512x4096x14336, GemmGate, rmsnorm_rope_bf16_512x4096, NormRope1, , bfuse::kZigzag, 1, 1)
+BFUSE_BFUSE_KERNEL(gemm_bf16_512x4096x14336, GemmGate, rmsnorm_rope_bf16_512x4096, NormRope1, _c256, bfuse::kChunked, 256, 1)
+BFUSE_BFUSE_KERNEL(gemm_bf16_512x4096x14336, GemmGate, rmsnorm_rope_bf16_512x4096_w4, NormRope4, _c256, bfuse::kChunked, 256, 1)

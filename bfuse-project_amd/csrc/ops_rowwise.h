@@ -112,53 +112,154 @@ struct LayerNorm {
 // softmax over the last axis of x[HEADS, S, S] with the causal mask: column j > row i is
 // masked to -inf before the softmax, so its probability is exactly 0
 // (files/gpt2.txt:35-36).  One wave per row; only the visible prefix is read.
-template <int HEADS_, int S_, int WAVES_>
+template <int HEADS_, int S_, int WAVES_, int RPW_ = 1, int RB_ = 1>
 struct SoftmaxCausal {
-    static constexpr int HEADS = HEADS_, S = S_, WAVES = WAVES_;
+    // RPW rows per wave, processed RB at a time (RB rows' loads are in flight together)
+    static constexpr int HEADS = HEADS_, S = S_, WAVES = WAVES_, RPW = RPW_, RB = RB_;
     static constexpr int THREADS = 64 * WAVES;
     static constexpr int ROWS = HEADS * S;
-    static constexpr Dims3 GRID{ROWS / WAVES, 1, 1};
+    static constexpr Dims3 GRID{ROWS / (WAVES * RPW), 1, 1};
     static constexpr Dims3 BLOCK{THREADS, 1, 1};
     static constexpr bool HAS_BARRIERS = false;
     static constexpr int VEC = S / 256;
-    static_assert(ROWS % WAVES == 0 && S % 256 == 0, "one wave per row, whole vectors per lane");
+    static_assert(ROWS % (WAVES * RPW) == 0 && S % 256 == 0 && RPW % RB == 0, "whole rows per wave, whole vectors per lane");
     using Smem = NoSmem;
+
+    // rows row0 + b*stride, b = 0..RB-1; every row is reduced on its own, in the same order
+    // whatever RB is
+    __device__ static __forceinline__ void rows(int row0, int stride, int lane, const void* I, void* O)
+    {
+        const float ninf = -__builtin_inff();
+        f32x4 v[RB][VEC];
+#pragma unroll
+        for (int b = 0; b < RB; ++b) {
+            const int row = row0 + b * stride;
+            const int i = row % S;  // query position: columns 0..i are visible
+            const f32x4* __restrict__ x = static_cast<const f32x4*>(I) + (size_t)row * (S / 4);
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) {
+                const int col = (c * 64 + lane) * 4;
+                v[b][c] = f32x4{ninf, ninf, ninf, ninf};
+                if (col <= i) {
+                    const f32x4 t = x[c * 64 + lane];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[b][c][e] = (col + e <= i) ? t[e] : ninf;
+                }
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < RB; ++b) {
+            const int row = row0 + b * stride;
+            f32x4* __restrict__ y = static_cast<f32x4*>(O) + (size_t)row * (S / 4);
+            float m = ninf;
+#pragma unroll
+            for (int c = 0; c < VEC; ++c)
+                m = fmaxf(m, fmaxf(fmaxf(v[b][c][0], v[b][c][1]), fmaxf(v[b][c][2], v[b][c][3])));
+            m = wave_max(m);
+            float s = 0.f;
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[b][c][e] = expf(v[b][c][e] - m);  // exp(-inf) == 0 for masked columns
+                s += (v[b][c][0] + v[b][c][1]) + (v[b][c][2] + v[b][c][3]);
+            }
+            s = wave_sum(s);
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) y[c * 64 + lane] = v[b][c] / s;
+        }
+    }
 
     template <class Sync>
     __device__ static __forceinline__ void run(int vblock, int tid, Smem&, const void* I, const void*,
                                                void* O, Sync)
     {
         const int wave = tid >> 6, lane = tid & 63;
-        const int row = vblock * WAVES + wave;
-        const int i = row % S;  // query position: columns 0..i are visible
-        const f32x4* __restrict__ x = static_cast<const f32x4*>(I) + (size_t)row * (S / 4);
-        f32x4* __restrict__ y = static_cast<f32x4*>(O) + (size_t)row * (S / 4);
-        const float ninf = -__builtin_inff();
+        // consecutive waves take consecutive rows; a wave's RPW rows are WAVES*GRID apart so
+        // that every pass over the grid touches one contiguous slab of the matrix
+        constexpr int stride = GRID.size() * WAVES;
+        for (int r = 0; r < RPW; r += RB)
+            rows((r * GRID.size() + vblock) * WAVES + wave, stride, lane, I, O);
+    }
+};
 
-        f32x4 v[VEC];
-        float m = ninf;
+// RMSNorm over x[S, HEADS*HD] (bf16) followed by rotate-half RoPE per head, bf16 out:
+//   t = w * (x * (1/sqrt(mean(x^2) + 1e-5)))                     files/Meta-Llama-3-8B.txt:5-14
+//   out = t*cos + concat(-t[HD/2:], t[:HD/2])*sin                 files/Meta-Llama-3-8B.txt:19-26
+// evaluated in fp32 from the bf16 inputs, rounded once (to nearest even) to bf16.
+// F holds w[HEADS*HD] (bf16), then cos[S,HD] and sin[S,HD] (fp32), as the dump holds them
+// as (1,1,S,HD) constants.  One wave per row (sequence position); a lane owns, for each of
+// its (head, octet) slots, the eight elements j..j+7 AND their rotation partners j+HD/2.., so
+// the rotation needs no cross-lane traffic and every load/store is 128 bits.
+template <int S_, int HEADS_, int HD_, int WAVES_>
+struct RmsNormRope {
+    static constexpr int S = S_, HEADS = HEADS_, HD = HD_, WAVES = WAVES_;
+    static constexpr int D = HEADS * HD, HALF = HD / 2;
+    static constexpr int THREADS = 64 * WAVES;
+    static constexpr Dims3 GRID{S / WAVES, 1, 1};
+    static constexpr Dims3 BLOCK{THREADS, 1, 1};
+    static constexpr bool HAS_BARRIERS = false;
+    static constexpr int OCT = HALF / 8;                 // octets per half head
+    static constexpr int SLOTS = HEADS * OCT / 64;       // (head, octet) slots per lane
+    static_assert(S % WAVES == 0 && HALF % 8 == 0 && (HEADS * OCT) % 64 == 0, "whole slots per lane");
+    static constexpr size_t COS_OFFSET = (size_t)D * 2;                 // bytes into F
+    static constexpr size_t SIN_OFFSET = COS_OFFSET + (size_t)S * HD * 4;
+    static constexpr size_t F_BYTES = SIN_OFFSET + (size_t)S * HD * 4;
+    using Smem = NoSmem;
+
+    __device__ static __forceinline__ void unpack(const u16x8& h, float (&f)[8])
+    {
 #pragma unroll
-        for (int c = 0; c < VEC; ++c) {
-            const int col = (c * 64 + lane) * 4;
-            v[c] = f32x4{ninf, ninf, ninf, ninf};
-            if (col <= i) {
-                const f32x4 t = x[c * 64 + lane];
+        for (int e = 0; e < 8; ++e) f[e] = __builtin_bit_cast(float, (unsigned int)h[e] << 16);
+    }
+    __device__ static __forceinline__ unsigned short to_bf16(float f)
+    {
+        unsigned int u = __builtin_bit_cast(unsigned int, f);
+        u += 0x7fffu + ((u >> 16) & 1u);
+        return (unsigned short)(u >> 16);
+    }
+
+    template <class Sync>
+    __device__ static __forceinline__ void run(int vblock, int tid, Smem&, const void* I, const void* F,
+                                               void* O, Sync)
+    {
+        const int wave = tid >> 6, lane = tid & 63;
+        const int pos = vblock * WAVES + wave;
+        const unsigned short* __restrict__ x = static_cast<const unsigned short*>(I) + (size_t)pos * D;
+        const unsigned short* __restrict__ w = static_cast<const unsigned short*>(F);
+        const float* __restrict__ cosv = reinterpret_cast<const float*>(static_cast<const char*>(F) + COS_OFFSET) + (size_t)pos * HD;
+        const float* __restrict__ sinv = reinterpret_cast<const float*>(static_cast<const char*>(F) + SIN_OFFSET) + (size_t)pos * HD;
+        unsigned short* __restrict__ y = static_cast<unsigned short*>(O) + (size_t)pos * D;
+
+        float lo[SLOTS][8], hi[SLOTS][8];
+        float ss = 0.f;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) v[c][e] = (col + e <= i) ? t[e] : ninf;
+        for (int s = 0; s < SLOTS; ++s) {
+            const int slot = s * 64 + lane;
+            const int base = (slot / OCT) * HD + (slot % OCT) * 8;
+            unpack(*reinterpret_cast<const u16x8*>(x + base), lo[s]);
+            unpack(*reinterpret_cast<const u16x8*>(x + base + HALF), hi[s]);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) ss += lo[s][e] * lo[s][e] + hi[s][e] * hi[s][e];
+        }
+        const float r = 1.0f / sqrtf(wave_sum(ss) / (float)D + 1e-5f);
+#pragma unroll
+        for (int s = 0; s < SLOTS; ++s) {
+            const int slot = s * 64 + lane;
+            const int j = (slot % OCT) * 8;
+            const int base = (slot / OCT) * HD + j;
+            float wl[8], wh[8];
+            unpack(*reinterpret_cast<const u16x8*>(w + base), wl);
+            unpack(*reinterpret_cast<const u16x8*>(w + base + HALF), wh);
+            u16x8 ol, oh;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float tl = wl[e] * (lo[s][e] * r), th = wh[e] * (hi[s][e] * r);
+                ol[e] = to_bf16(tl * cosv[j + e] + (-th) * sinv[j + e]);
+                oh[e] = to_bf16(th * cosv[j + HALF + e] + tl * sinv[j + HALF + e]);
             }
-            m = fmaxf(m, fmaxf(fmaxf(v[c][0], v[c][1]), fmaxf(v[c][2], v[c][3])));
+            *reinterpret_cast<u16x8*>(y + base) = ol;
+            *reinterpret_cast<u16x8*>(y + base + HALF) = oh;
         }
-        m = wave_max(m);
-        float s = 0.f;
-#pragma unroll
-        for (int c = 0; c < VEC; ++c) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) v[c][e] = expf(v[c][e] - m);  // exp(-inf) == 0 for masked columns
-            s += (v[c][0] + v[c][1]) + (v[c][2] + v[c][3]);
-        }
-        s = wave_sum(s);
-#pragma unroll
-        for (int c = 0; c < VEC; ++c) y[c * 64 + lane] = v[c] / s;
     }
 };
 

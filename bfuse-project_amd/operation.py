@@ -62,7 +62,7 @@ def _u3(v):
     return (C.c_uint * 3)(*v)
 
 
-_DT = {4: np.float32, 2: np.uint16}
+_DT = {4: np.float32, 2: np.uint16, 1: np.uint8}
 
 
 class Operation:

@@ -52,6 +52,53 @@ def _pair2_inputs():
     return a, w, x, gb
 
 
+def _pair3_inputs():
+    x = np.maximum(fill_normal(_seed(3, 0), 64 * 56 * 56, 0.0, 1.0), np.float32(0.0))
+    w = fill_normal(_seed(3, 1), 64 * 64 * 9, 0.0, 0.05)
+    p = fill_normal(_seed(3, 2), 64 * 112 * 112, 0.0, 1.0)
+    unused = np.zeros(1, np.float32)
+    return x, w, p, unused
+
+
+def _pair4_inputs():
+    scores = fill_normal(_seed(4, 0), 12 * 512 * 512, 0.0, 1.0) / np.float32(8.0)
+    unused = np.zeros(1, np.float32)
+    a = fill_normal(_seed(4, 2), 512 * 768, 0.0, 1.0)
+    w = fill_normal(_seed(4, 3), 768 * 3072, 0.0, 0.02)
+    return scores, unused, a, w
+
+
+def rope_tables(S: int, hd: int, theta: float):
+    """cos/sin tables [S, hd] of rotate-half RoPE: angle(p, j) = p * theta^(-2*(j mod hd/2)/hd),
+    evaluated in double, stored fp32 (the Llama dump holds them as (1,1,S,hd) constants)."""
+    j = np.arange(hd) % (hd // 2)
+    inv = np.power(float(theta), -2.0 * j / hd)
+    ang = np.arange(S, dtype=np.float64)[:, None] * inv[None, :]
+    return np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+
+
+def pack_norm_rope_operand(w_bf16: np.ndarray, cosv: np.ndarray, sinv: np.ndarray) -> np.ndarray:
+    """Second operand of the RMSNorm+RoPE kernel: weight (bf16), cos table, sin table (fp32), as bytes."""
+    return np.concatenate([w_bf16.view(np.uint8).ravel(), cosv.view(np.uint8).ravel(), sinv.view(np.uint8).ravel()])
+
+
+def unpack_norm_rope_operand(F: np.ndarray, S: int, d: int, hd: int):
+    F = np.ascontiguousarray(F, np.uint8)
+    w = F[: 2 * d].view(np.uint16)
+    cosv = F[2 * d: 2 * d + 4 * S * hd].view(np.float32).reshape(S, hd)
+    sinv = F[2 * d + 4 * S * hd:].view(np.float32).reshape(S, hd)
+    return w, cosv, sinv
+
+
+def _pair5_inputs():
+    a = f32_to_bf16(fill_normal(_seed(5, 0), 512 * 4096, 0.0, 1.0))
+    w = f32_to_bf16(fill_normal(_seed(5, 1), 14336 * 4096, 0.0, 0.02))       # [N, K] = (out, in)
+    x = f32_to_bf16(fill_normal(_seed(5, 2), 512 * 4096, 0.0, 1.0))
+    cosv, sinv = rope_tables(512, 128, 500000.0)
+    f2 = pack_norm_rope_operand(f32_to_bf16(np.ones(4096, np.float32)), cosv, sinv)
+    return a, w, x, f2
+
+
 PAIRS: Dict[int, Pair] = {
     1: Pair(1, "GEMM fp32 512x512x512 || ReLU(x+b) over 1Mi fp32, hfuse 128/128",
             "gemm_f32_512x512x512", "bias_relu_1048576", "hfuse",
@@ -68,6 +115,32 @@ PAIRS: Dict[int, Pair] = {
              ("gemm_f32_512x768x2304_p3", "layernorm_512x768_w2", "bfuse", "_r")], _pair2_inputs,
             bytes1=(512 * 768 + 768 * 2304 + 512 * 2304) * 4, bytes2=(2 * 512 * 768 + 2 * 768) * 4,
             flops=2 * 512 * 768 * 2304, bound="mfma", peak=157.3, dtype="f32", tol=1e-5),
+    3: Pair(3, "conv 3x3 s1 p1 [1,64,56,56]->64 fp32 || max-pool 3x3 s2 p1 [1,64,112,112], zig-zag bfuse",
+            "conv3x3_f32_64x56x56_64", "maxpool3x3s2_f32_64x112x112", "bfuse",
+            [("bfuse", ""), ("bfuse", "_c8"), ("bfuse", "_c256"), ("hfuse", "")],
+            [("conv3x3_f32_64x56x56_64_h", "maxpool3x3s2_f32_64x112x112", "bfuse", ""),
+             ("conv3x3_f32_64x56x56_64_h", "maxpool3x3s2_f32_64x112x112", "bfuse", "_c8")], _pair3_inputs,
+            bytes1=(64 * 56 * 56 * 2 + 64 * 64 * 9) * 4, bytes2=(64 * 112 * 112 + 64 * 56 * 56) * 4,
+            flops=2 * 64 * 64 * 9 * 56 * 56, bound="mfma", peak=157.3, dtype="f32", tol=1e-5),
+    4: Pair(4, "causal softmax 12x[512x512] fp32 || GEMM fp32 [512x768].[768x3072] + tanh-GELU, bfuse",
+            "softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072", "bfuse",
+            [("bfuse", ""), ("bfuse", "_c256")],
+            [("softmax_causal_12x512x512_w1", "gemm_gelu_f32_512x768x3072", "bfuse", "_c256"),
+             ("softmax_causal_12x512x512_w1", "gemm_gelu_f32_512x768x3072_t32", "bfuse", "_c256"),
+             ("softmax_causal_12x512x512_b4", "gemm_gelu_f32_512x768x3072", "bfuse", "_c256"),
+             ("softmax_causal_12x512x512_b4", "gemm_gelu_f32_512x768x3072_h", "bfuse", "_c256"),
+             ("softmax_causal_12x512x512_b4", "gemm_gelu_f32_512x768x3072_h", "bfuse", "_c512"),
+             ("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072_h", "bfuse", "_c512"),
+             ("softmax_causal_12x512x512_r6", "gemm_gelu_f32_512x768x3072", "hfuse", ""),
+             ("softmax_causal_12x512x512_r6", "gemm_gelu_f32_512x768x3072_t32", "hfuse", "")], _pair4_inputs,
+            bytes1=2 * 12 * 512 * 512 * 4, bytes2=(512 * 768 + 768 * 3072 + 512 * 3072) * 4,
+            flops=2 * 512 * 768 * 3072, bound="mfma", peak=157.3, dtype="f32", tol=1e-5),
+    5: Pair(5, "GEMM bf16 [512x4096].[14336x4096]^T (fp32 acc) || RMSNorm+RoPE [512x4096] bf16, bfuse",
+            "gemm_bf16_512x4096x14336", "rmsnorm_rope_bf16_512x4096", "bfuse",
+            [("bfuse", ""), ("bfuse", "_c256")],
+            [("gemm_bf16_512x4096x14336", "rmsnorm_rope_bf16_512x4096_w4", "bfuse", "_c256")], _pair5_inputs,
+            bytes1=(512 * 4096 + 4096 * 14336 + 512 * 14336) * 2, bytes2=2 * 512 * 4096 * 2 + 4096 * 2,
+            flops=2 * 512 * 4096 * 14336, bound="mfma", peak=2500.0, dtype="bf16", tol=1e-2),
 }
 
 
@@ -84,4 +157,7 @@ def fusions(pair: Pair):
 HEADLINE = {
     1: ("gemm_f32_512x512x512", "bias_relu_1048576", "hfuse", ""),
     2: ("gemm_f32_512x768x2304", "layernorm_512x768_w1", "bfuse", "_r"),
+    3: ("conv3x3_f32_64x56x56_64", "maxpool3x3s2_f32_64x112x112", "bfuse", "_c8"),
+    4: ("softmax_causal_12x512x512_b4", "gemm_gelu_f32_512x768x3072_h", "bfuse", "_c512"),
+    5: ("gemm_bf16_512x4096x14336", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
 }
