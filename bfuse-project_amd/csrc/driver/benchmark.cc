@@ -1,0 +1,255 @@
+// benchmark -- command-line driver over libbfuse_rt, the counterpart of the reference's
+// generated main.cc (test-utils/test-suite-files/main_cc.py:22-36,139-299):
+//
+//     benchmark [-vh] [-n num_iterations] [-s seed] [-x suffix] T K1 K2
+//
+//      T : type of operation: 0 kernel1, 1 kernel2, 2 parallel (two streams), 3 hfuse, 4 bfuse,
+//          5 serial (kernel1 then kernel2 on one stream; not in the reference)
+//  K1,K2 : index into the first / second fusion set, or a kernel name.  The sets are the
+//          distinct first / second sides of the fused kernels the library was built with.
+//     -v : validate: run the variant, then each unfused kernel on the same inputs, and compare
+//          (the reference's check, main_cc.py:82-122,246-268).  Fused and parallel outputs
+//          must be bit-identical to the unfused ones; check_matrix (eps 1e-3) is reported too.
+//          Exit status 1 on mismatch (main_cc.py:288-292).
+//     -x : variant suffix of a bfuse kernel (e.g. _c256); default is the plain name.
+//
+// Inputs are seeded U(-0.5, 0.5) (the reference uses rand()/RAND_MAX - 0.5, utils_cc.py:28-31).
+// Prints the GPU-side duration of every timed launch set (3 warm-up launches are discarded,
+// scripts/profile_test_suite.py:10-11).
+#include <getopt.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "../../../include/bfuse_rt.h"
+
+static bool validation = false;
+static size_t num_iterations = 1;
+static unsigned long long seed = 0xB5F05E;
+static std::string suffix;
+static const char* operation_type_string[] = {"kernel1", "kernel2", "parallel", "hfuse", "bfuse", "serial"};
+
+static void print_help(const char* prog)
+{
+    printf("Usage: %s [-vh] [-n num_iterations] [-s seed] [-x suffix] T K1 K2\n", prog);
+    printf("Options:\n");
+    printf("     -v : validate test.                (default: off)\n");
+    printf("     -h : print this page.\n");
+    printf("     -n : number of iterations.         (default: 1)\n");
+    printf("     -s : seed of the synthetic inputs.\n");
+    printf("     -x : suffix of the bfuse variant.   (default: none)\n");
+    printf("      T : type of operation (0 kernel1, 1 kernel2, 2 parallel, 3 hfuse, 4 bfuse, 5 serial).\n");
+    printf("     K1 : idx or name of kernel1.\n");
+    printf("     K2 : idx or name of kernel2.\n");
+}
+
+#define CHECK(call)                                                                \
+    do {                                                                           \
+        int rc_ = (call);                                                          \
+        if (rc_ != 0) {                                                            \
+            fprintf(stderr, "bfuse error %d (%s:%d): %s\n", rc_, __FILE__, __LINE__, bfuse_last_error()); \
+            exit(EXIT_FAILURE);                                                    \
+        }                                                                          \
+    } while (0)
+
+static std::vector<std::string> fusion_set(int which)
+{
+    std::vector<std::string> out;
+    for (int i = 0; i < bfuse_kernel_count(); ++i) {
+        bfuse_kernel_info ki;
+        CHECK(bfuse_kernel_at(i, &ki));
+        if (ki.kind == BFUSE_KIND_SINGLE) continue;
+        std::string s = ki.side[which];
+        bool seen = false;
+        for (auto& o : out) seen |= (o == s);
+        if (!seen) out.push_back(s);
+    }
+    return out;
+}
+
+static std::string resolve(const char* arg, int which)
+{
+    char* end = nullptr;
+    long idx = strtol(arg, &end, 10);
+    if (end && *end == '\0') {
+        auto set = fusion_set(which);
+        if (idx < 0 || idx >= (long)set.size()) {
+            fprintf(stderr, "K%d index %ld out of range (set has %zu kernels)\n", which + 1, idx, set.size());
+            exit(EXIT_FAILURE);
+        }
+        return set[idx];
+    }
+    return arg;
+}
+
+struct HostSide {
+    std::vector<unsigned char> I, F, O, O_ans;
+    bfuse_kernel_info ki;
+};
+
+static size_t nelem(const int* s) { return (size_t)s[0] * s[1] * s[2] * s[3]; }
+
+static void fill(std::vector<unsigned char>& buf, const int* shape, int elem, unsigned long long sd)
+{
+    const size_t n = nelem(shape);
+    buf.assign(n * elem, 0);
+    if (elem == 4) {
+        bfuse_fill_uniform(sd, n, -0.5f, 0.5f, reinterpret_cast<float*>(buf.data()));
+    } else if (elem == 2) {
+        std::vector<float> tmp(n);
+        bfuse_fill_uniform(sd, n, -0.5f, 0.5f, tmp.data());
+        bfuse_f32_to_bf16(n, tmp.data(), reinterpret_cast<unsigned short*>(buf.data()));
+    } else {
+        // packed byte operand: finite fp32 values in every 4-byte word and finite bf16 in every
+        // half word (high halves of small floats), so both views of the bytes stay finite
+        const size_t words = n / 4;
+        std::vector<float> tmp(words);
+        bfuse_fill_uniform(sd, words, 0.25f, 0.5f, tmp.data());
+        for (size_t i = 0; i < words; ++i) {
+            unsigned u;
+            memcpy(&u, &tmp[i], 4);
+            u = (u & 0xffff0000u) | (u >> 16);
+            memcpy(buf.data() + 4 * i, &u, 4);
+        }
+    }
+}
+
+static void setup(HostSide& h, const std::string& name, int side)
+{
+    CHECK(bfuse_kernel_find(name.c_str(), &h.ki));
+    if (h.ki.kind != BFUSE_KIND_SINGLE) {
+        fprintf(stderr, "%s is a fused kernel; K%d must name a standalone kernel\n", name.c_str(), side);
+        exit(EXIT_FAILURE);
+    }
+    fill(h.I, h.ki.shape[0], h.ki.elem_bytes[0], seed * 16 + 4 * side);
+    fill(h.F, h.ki.shape[1], h.ki.elem_bytes[1], seed * 16 + 4 * side + 1);
+    h.O.assign(nelem(h.ki.shape[2]) * h.ki.elem_bytes[2], 0);
+    h.O_ans = h.O;
+    CHECK(bfuse_set_elem_bytes(side, h.ki.elem_bytes[0], h.ki.elem_bytes[1], h.ki.elem_bytes[2]));
+}
+
+static bool compare(const HostSide& h, const char* what)
+{
+    const bool same = memcmp(h.O.data(), h.O_ans.data(), h.O.size()) == 0;
+    long bad = -1;
+    if (h.ki.elem_bytes[2] == 4)
+        bad = bfuse_check_matrix(reinterpret_cast<const float*>(h.O.data()), reinterpret_cast<const float*>(h.O_ans.data()),
+                                 h.O.size() / 4, 1e-3f);
+    printf("Validation %s: %s (bit-exact: %s", what, same ? "VALID" : "INVALID", same ? "yes" : "no");
+    if (bad >= 0) printf(", check_matrix eps 1e-3: %ld wrong", bad);
+    printf(")\n");
+    return same;
+}
+
+static void stats(const char* label, const std::vector<float>& v)
+{
+    double s = 0, mn = 1e30, sq = 0;
+    for (float x : v) { s += x; mn = x < mn ? x : mn; }
+    const double mean = s / v.size();
+    for (float x : v) sq += (x - mean) * (x - mean);
+    printf("%-10s mean %9.3f us  min %9.3f us  std %7.3f us  (n=%zu)\n", label, mean, mn, std::sqrt(sq / v.size()), v.size());
+}
+
+int main(int argc, char** argv)
+{
+    int c;
+    while ((c = getopt(argc, argv, "vhn:s:x:")) != -1) {
+        switch (c) {
+            case 'v': validation = true; break;
+            case 'n': num_iterations = (size_t)atoi(optarg); break;
+            case 's': seed = strtoull(optarg, nullptr, 0); break;
+            case 'x': suffix = optarg; break;
+            case 'h':
+            default: print_help(argv[0]); exit(0);
+        }
+    }
+    if (argc - optind < 3) {
+        print_help(argv[0]);
+        exit(0);
+    }
+    const size_t T = (size_t)atoi(argv[optind]);
+    if (T > 5 || num_iterations < 1) {
+        fprintf(stderr, "T must be 0..5 and -n at least 1\n");
+        return EXIT_FAILURE;
+    }
+    CHECK(bfuse_init(0));
+    const std::string k1 = resolve(argv[optind + 1], 0), k2 = resolve(argv[optind + 2], 1);
+
+    HostSide a, b;
+    setup(a, k1, 1);
+    setup(b, k2, 2);
+    CHECK(initialize_kernel1(a.ki.shape[0], a.ki.shape[1], a.ki.shape[2]));
+    CHECK(initialize_kernel2(b.ki.shape[0], b.ki.shape[1], b.ki.shape[2]));
+
+    bfuse_kernel_info fused;
+    memset(&fused, 0, sizeof(fused));
+    if (T == BFUSE_MODE_HFUSE || T == BFUSE_MODE_BFUSE) {
+        const std::string fname = k1 + "_" + k2 + (T == BFUSE_MODE_HFUSE ? "_fused_hfuse" : "_fused_bfuse" + suffix);
+        CHECK(bfuse_kernel_find(fname.c_str(), &fused));
+    }
+    printf("============= Benchmark =============\n");
+    printf("- Number of iterations: %zu\n- Type of operation: %s\n- Kernel1: %s\n- Kernel2: %s\n", num_iterations,
+           operation_type_string[T], k1.c_str(), k2.c_str());
+    if (fused.func) printf("- Fused kernel: %s  grid %u block %u regs %d lds %d\n", fused.name, fused.grid[0], fused.block[0], fused.regs, fused.lds_bytes);
+
+    // one run through the reference's copy-in / launch / copy-out entry points
+    switch (T) {
+        case BFUSE_MODE_KERNEL1:
+            CHECK(run_kernel1(a.I.data(), a.F.data(), a.O.data(), a.ki.shape[0], a.ki.shape[1], a.ki.shape[2],
+                              (bfuse_kernel3_fn)a.ki.func, a.ki.grid, a.ki.block, 0));
+            break;
+        case BFUSE_MODE_KERNEL2:
+            CHECK(run_kernel2(b.I.data(), b.F.data(), b.O.data(), b.ki.shape[0], b.ki.shape[1], b.ki.shape[2],
+                              (bfuse_kernel3_fn)b.ki.func, b.ki.grid, b.ki.block, 0));
+            break;
+        case BFUSE_MODE_PARALLEL:
+        case BFUSE_MODE_SERIAL:
+            CHECK(run_parallel(a.I.data(), a.F.data(), a.O.data(), b.I.data(), b.F.data(), b.O.data(), a.ki.shape[0],
+                               a.ki.shape[1], a.ki.shape[2], b.ki.shape[0], b.ki.shape[1], b.ki.shape[2],
+                               (bfuse_kernel3_fn)a.ki.func, (bfuse_kernel3_fn)b.ki.func, a.ki.grid, a.ki.block,
+                               b.ki.grid, b.ki.block, 0, 0));
+            break;
+        default:
+            CHECK(run_fuse(a.I.data(), a.F.data(), a.O.data(), b.I.data(), b.F.data(), b.O.data(), a.ki.shape[0],
+                           a.ki.shape[1], a.ki.shape[2], b.ki.shape[0], b.ki.shape[1], b.ki.shape[2],
+                           (bfuse_kernel6_fn)fused.func, fused.grid, fused.block, 0, 0));
+    }
+
+    bool is_valid = true;
+    if (validation) {
+        if (T != BFUSE_MODE_KERNEL2) {
+            CHECK(run_kernel1(a.I.data(), a.F.data(), a.O_ans.data(), a.ki.shape[0], a.ki.shape[1], a.ki.shape[2],
+                              (bfuse_kernel3_fn)a.ki.func, a.ki.grid, a.ki.block, 0));
+            is_valid &= compare(a, "kernel1");
+        }
+        if (T != BFUSE_MODE_KERNEL1) {
+            CHECK(run_kernel2(b.I.data(), b.F.data(), b.O_ans.data(), b.ki.shape[0], b.ki.shape[1], b.ki.shape[2],
+                              (bfuse_kernel3_fn)b.ki.func, b.ki.grid, b.ki.block, 0));
+            is_valid &= compare(b, "kernel2");
+        }
+    }
+
+    // GPU-side durations over device-resident operands
+    const void* fa = T == 1 ? b.ki.func : (T >= 3 && T <= 4 ? fused.func : a.ki.func);
+    const unsigned* ga = T == 1 ? b.ki.grid : (T >= 3 && T <= 4 ? fused.grid : a.ki.grid);
+    const unsigned* ba = T == 1 ? b.ki.block : (T >= 3 && T <= 4 ? fused.block : a.ki.block);
+    std::vector<float> tot(num_iterations), ta(num_iterations), tb(num_iterations);
+    CHECK(bfuse_time((int)T, fa, ga, ba, b.ki.func, b.ki.grid, b.ki.block, 3, (int)num_iterations, tot.data(), ta.data(), tb.data()));
+    stats(operation_type_string[T], tot);
+    if (T == BFUSE_MODE_PARALLEL || T == BFUSE_MODE_SERIAL) {
+        stats("  kernel1", ta);
+        stats("  kernel2", tb);
+    }
+
+    CHECK(finalize_kernel1());
+    CHECK(finalize_kernel2());
+    if (!is_valid) {
+        printf("Validation: INVALID\n");
+        exit(1);
+    }
+    return 0;
+}

@@ -1,0 +1,54 @@
+// Small instances of every operator body and fusion form.  They exist for the parity tests:
+// shapes the CPU oracle evaluates in full, tile configurations the five headline pairs do
+// not reach (single-wave GEMM without LDS reduction, 16-column groups only, deeper
+// prefetch, multi-group convolution, several K-steps / M-tiles of the bf16 GEMM), sides with
+// different grid sizes under horizontal fusion, and the ratio / proportional block patterns.
+#include "fuse.h"
+#include "ops_conv.h"
+#include "ops_gemm_bf16.h"
+#include "ops_gemm_f32.h"
+#include "ops_rowwise.h"
+
+using namespace bfuse;
+
+BFUSE_MODULE_PROLOGUE()
+
+using GemmS1 = GemmF32<64, 48, 32, 16, 48, 1>;                        // one wave, 16-column groups only
+using GemmS2 = GemmF32<96, 192, 128, 32, 64, 2, kEpiGeluTanh, 3>;     // 2 waves, GELU, 3 register stages
+using GemmS3 = GemmF32<32, 144, 256, 32, 144, 4>;                     // the 64+64+16 column split, one tile
+using BiasReluS = BiasRelu<4096, 64, 4>;
+using LayerNormS = LayerNorm<8, 256, 2, 1>;
+using SoftmaxS = SoftmaxCausal<2, 256, 2, 2, 2>;
+using ConvS1 = Conv3x3F32<16, 16, 8, 8, 16, 1, 1>;                     // one channel group, one wave
+using ConvS2 = Conv3x3F32<32, 32, 12, 12, 16, 1, 2>;                   // two channel groups on two waves
+using ConvS3 = Conv3x3F32<64, 16, 8, 16, 16, 2, 2>;                    // two groups per wave, two pixel blocks
+using PoolS = MaxPool3x3S2<4, 16, 16, 64>;
+using GemmB1 = GemmBf16NT<128, 1792, 64, 128, 224>;                   // one K-step
+using GemmB2 = GemmBf16NT<256, 1792, 192, 128, 224>;                  // two M-tiles, three K-steps
+using NormRopeS = RmsNormRope<6, 8, 128, 2>;
+
+BFUSE_KERNEL(gemm_f32_64x32x48, GemmS1, ({{64, 32, 1, 1}, 4}), ({{32, 48, 1, 1}, 4}), ({{64, 48, 1, 1}, 4}))
+BFUSE_KERNEL(gemm_gelu_f32_96x128x192, GemmS2, ({{96, 128, 1, 1}, 4}), ({{128, 192, 1, 1}, 4}), ({{96, 192, 1, 1}, 4}))
+BFUSE_KERNEL(gemm_f32_32x256x144, GemmS3, ({{32, 256, 1, 1}, 4}), ({{256, 144, 1, 1}, 4}), ({{32, 144, 1, 1}, 4}))
+BFUSE_KERNEL(bias_relu_4096, BiasReluS, ({{4096, 1, 1, 1}, 4}), ({{4096, 1, 1, 1}, 4}), ({{4096, 1, 1, 1}, 4}))
+BFUSE_KERNEL(layernorm_8x256, LayerNormS, ({{8, 256, 1, 1}, 4}), ({{2, 256, 1, 1}, 4}), ({{8, 256, 1, 1}, 4}))
+BFUSE_KERNEL(softmax_causal_2x256x256, SoftmaxS, ({{2, 256, 256, 1}, 4}), ({{1, 1, 1, 1}, 4}), ({{2, 256, 256, 1}, 4}))
+BFUSE_KERNEL(conv3x3_f32_16x8x8_16, ConvS1, ({{1, 16, 8, 8}, 4}), ({{16, 16, 3, 3}, 4}), ({{1, 16, 8, 8}, 4}))
+BFUSE_KERNEL(conv3x3_f32_32x12x12_32, ConvS2, ({{1, 32, 12, 12}, 4}), ({{32, 32, 3, 3}, 4}), ({{1, 32, 12, 12}, 4}))
+BFUSE_KERNEL(conv3x3_f32_64x8x16_16, ConvS3, ({{1, 64, 8, 16}, 4}), ({{16, 64, 3, 3}, 4}), ({{1, 16, 8, 16}, 4}))
+BFUSE_KERNEL(maxpool3x3s2_f32_4x16x16, PoolS, ({{1, 4, 16, 16}, 4}), ({{1, 1, 1, 1}, 4}), ({{1, 4, 8, 8}, 4}))
+BFUSE_KERNEL(gemm_bf16_128x64x1792, GemmB1, ({{128, 64, 1, 1}, 2}), ({{1792, 64, 1, 1}, 2}), ({{128, 1792, 1, 1}, 2}))
+BFUSE_KERNEL(gemm_bf16_256x192x1792, GemmB2, ({{256, 192, 1, 1}, 2}), ({{1792, 192, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
+BFUSE_KERNEL(rmsnorm_rope_bf16_6x1024, NormRopeS, ({{6, 1024, 1, 1}, 2}), ({{(int)NormRopeS::F_BYTES, 1, 1, 1}, 1}), ({{6, 1024, 1, 1}, 2}))
+
+// horizontal fusion with unequal grids (9 GEMM tiles, 4 element-wise blocks) and a barrier side
+BFUSE_HFUSE_KERNEL(gemm_gelu_f32_96x128x192, GemmS2, bias_relu_4096, BiasReluS)
+// both sides carry a barrier: two LDS-counter barriers in one workgroup
+BFUSE_HFUSE_KERNEL(gemm_gelu_f32_96x128x192, GemmS2, conv3x3_f32_32x12x12_32, ConvS2)
+// ratio 2:1 zig-zag (18 conv tiles, 9 GEMM tiles), proportional, chunked with a remainder
+BFUSE_BFUSE_KERNEL(conv3x3_f32_32x12x12_32, ConvS2, gemm_gelu_f32_96x128x192, GemmS2, , bfuse::kZigzag, 2, 1)
+BFUSE_BFUSE_KERNEL(conv3x3_f32_32x12x12_32, ConvS2, gemm_gelu_f32_96x128x192, GemmS2, _p1, bfuse::kProportional, 1, 1)
+BFUSE_BFUSE_KERNEL(conv3x3_f32_32x12x12_32, ConvS2, gemm_gelu_f32_96x128x192, GemmS2, _c4, bfuse::kChunked, 4, 1)
+BFUSE_BFUSE_KERNEL(layernorm_8x256, LayerNormS, softmax_causal_2x256x256, SoftmaxS, , bfuse::kZigzag, 1, 1)
+BFUSE_BFUSE_KERNEL(gemm_bf16_256x192x1792, GemmB2, rmsnorm_rope_bf16_6x1024, NormRopeS, _c8, bfuse::kChunked, 8, 1)
+BFUSE_HFUSE_KERNEL(maxpool3x3s2_f32_4x16x16, PoolS, layernorm_8x256, LayerNormS)

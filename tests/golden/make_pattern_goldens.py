@@ -19,7 +19,10 @@ Inputs are *outputs of the reference's fuser* that the reference checked in:
   * guards and `bar.sync` lines of emitted *_hfuse.cu / hfuse_kernels.cu files
         -> hfuse_ranges.json : thread range / block bound per side, barrier id+count.
 
-Only numbers are stored; no kernel body text is copied.
+  * config/*.yaml of legacy/tests/single_bgemm_conv2d/case-0_4/M_diff/case-2 (copied as is
+    into config_sample/: they are the fuser's input/output data files).
+
+Only numbers and config data are stored; no kernel body text is copied.
 """
 import glob
 import json
@@ -214,7 +217,20 @@ def make_fused_dims():
     print("fused_dims.json:", n_rows, "rows read,", len(out), "unique")
 
 
+def copy_config_sample():
+    """The four small YAML configs of one legacy case (two kernels, 152-thread conv block): data
+    files in the fuser's wire format, one written by PyYAML and two by llvm::yaml."""
+    import shutil
+    src = f"{REF}/legacy/tests/single_bgemm_conv2d/case-0_4/M_diff/case-2/config"
+    dst = f"{OUT}/config_sample"
+    os.makedirs(dst, exist_ok=True)
+    for n in ("kernels.yaml", "fusions.yaml", "bfuse_kernels.yaml", "hfuse_kernels.yaml"):
+        shutil.copyfile(f"{src}/{n}", f"{dst}/{n}")
+    print("config_sample/: 4 yaml files")
+
+
 if __name__ == "__main__":
+    copy_config_sample()
     make_fused_dims()
     make_bfuse_maps()
     make_hfuse_ranges()

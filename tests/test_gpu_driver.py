@@ -1,0 +1,35 @@
+"""The C++ command-line driver (the reference's `benchmark [-v] [-n N] T K1 K2`) end to end on
+the GPU: every mode validates, and a mismatch would exit with status 1 as the reference's does."""
+import os
+import subprocess
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+EXE = os.path.join(ROOT, "bfuse-project_amd", "benchmark")
+
+
+def _run(*args):
+    print("benchmark", *args, flush=True)
+    return subprocess.run([EXE, *args], capture_output=True, text=True, timeout=120)
+
+
+def test_driver_modes_validate():
+    if not os.path.exists(EXE):
+        pytest.fail(f"{EXE} has not been built")
+    k1, k2 = "gemm_f32_512x768x2304", "layernorm_512x768_w1"
+    for mode, extra in (("0", []), ("1", []), ("2", []), ("5", []), ("4", ["-x", "_r"])):
+        r = _run("-v", "-n", "5", *extra, mode, k1, k2)
+        assert r.returncode == 0, r.stdout + r.stderr
+        assert "INVALID" not in r.stdout and "VALID" in r.stdout
+    r = _run("-v", "-n", "3", "3", "gemm_f32_512x512x512", "bias_relu_1048576")
+    assert r.returncode == 0 and "bit-exact: yes" in r.stdout, r.stdout + r.stderr
+    # bf16 pair with the packed byte operand, by index into the fusion sets
+    r = _run("-v", "-n", "2", "-x", "_c256", "4", "gemm_bf16_512x4096x14336", "rmsnorm_rope_bf16_512x4096")
+    assert r.returncode == 0 and "bit-exact: yes" in r.stdout, r.stdout + r.stderr
+
+
+def test_driver_rejects_unknown_kernels():
+    r = _run("4", "no_such_kernel", "layernorm_512x768")
+    assert r.returncode != 0 and "unknown kernel" in r.stderr
