@@ -59,7 +59,7 @@ def main():
                  "this build launches nothing on a second GPU; run with --gpus 1")
 
     import bfuse_project_amd as bf
-    from bfuse_project_amd.workloads import PAIRS, HEADLINE
+    from bfuse_project_amd.workloads import PAIRS, HEADLINE, MEASURED_TRAFFIC
 
     pair = PAIRS[args.pair]
     k1, k2, kind, suffix = HEADLINE[args.pair]
@@ -147,7 +147,7 @@ def main():
         "batched_kernel2_us": round(b_k2, 3),
         "batched_fused_over_back_to_back": round(b_f / b_ser, 4),
         "roofline": {"bound": pair.bound, "achieved": round(achieved, 2), "peak": pair.peak, "unit": unit,
-                     "frac": round(achieved / pair.peak, 4), "traffic": None,
+                     "frac": round(achieved / pair.peak, 4), "traffic": MEASURED_TRAFFIC.get(fused.name),
                      "kernel": fused.name, "avg_us": round(fused_us, 3),
                      "algorithmic": {"flops": pair.flops, "bytes": pair.bytes1 + pair.bytes2}},
     }

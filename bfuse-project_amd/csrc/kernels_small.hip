@@ -41,6 +41,10 @@ BFUSE_KERNEL(gemm_bf16_128x64x1792, GemmB1, ({{128, 64, 1, 1}, 2}), ({{1792, 64,
 BFUSE_KERNEL(gemm_bf16_256x192x1792, GemmB2, ({{256, 192, 1, 1}, 2}), ({{1792, 192, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
 BFUSE_KERNEL(rmsnorm_rope_bf16_6x1024, NormRopeS, ({{6, 1024, 1, 1}, 2}), ({{(int)NormRopeS::F_BYTES, 1, 1, 1}, 1}), ({{6, 1024, 1, 1}, 2}))
 
+// calibration kernel for the memory counters: 64 MiB read, 64 MiB written
+using Copy64M = CopyF32<16777216, 256>;
+BFUSE_KERNEL(copy_f32_16777216, Copy64M, ({{16777216, 1, 1, 1}, 4}), ({{1, 1, 1, 1}, 4}), ({{16777216, 1, 1, 1}, 4}))
+
 // horizontal fusion with unequal grids (9 GEMM tiles, 4 element-wise blocks) and a barrier side
 BFUSE_HFUSE_KERNEL(gemm_gelu_f32_96x128x192, GemmS2, bias_relu_4096, BiasReluS)
 // both sides carry a barrier: two LDS-counter barriers in one workgroup

@@ -59,6 +59,31 @@ struct BiasRelu {
     }
 };
 
+// y = x over COUNT floats: a plain copy of known size, the calibration kernel for memory
+// counters (COUNT*4 bytes read, COUNT*4 bytes written).
+template <int COUNT_, int THREADS_>
+struct CopyF32 {
+    static constexpr int COUNT = COUNT_, THREADS = THREADS_;
+    static constexpr int PER_BLOCK = 4 * THREADS * 4;  // four 128-bit vectors per thread
+    static_assert(COUNT % PER_BLOCK == 0, "whole workgroups");
+    static constexpr Dims3 GRID{COUNT / PER_BLOCK, 1, 1};
+    static constexpr Dims3 BLOCK{THREADS_, 1, 1};
+    static constexpr bool HAS_BARRIERS = false;
+    using Smem = NoSmem;
+
+    template <class Sync>
+    __device__ static __forceinline__ void run(int vblock, int tid, Smem&, const void* I, const void*, void* O, Sync)
+    {
+        const f32x4* __restrict__ x = static_cast<const f32x4*>(I) + (size_t)vblock * (PER_BLOCK / 4);
+        f32x4* __restrict__ y = static_cast<f32x4*>(O) + (size_t)vblock * (PER_BLOCK / 4);
+        f32x4 v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = x[i * THREADS + tid];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) y[i * THREADS + tid] = v[i];
+    }
+};
+
 // LayerNorm over the last axis of x[ROWS, D]; F holds gamma[D] then beta[D].
 //   y = (x - mean) * (1 / sqrt(var + eps)) * gamma + beta, biased variance
 // (files/bert-base-uncased.txt:8-16).  One wave per row, the row lives in registers

@@ -161,3 +161,11 @@ HEADLINE = {
     4: ("softmax_causal_12x512x512_b4", "gemm_gelu_f32_512x768x3072_h", "bfuse", "_c512"),
     5: ("gemm_bf16_512x4096x14336", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
 }
+
+
+# HBM-side bytes per launch of a fused kernel, measured with rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE and scaled by what the same counters read for a 64 MiB copy kernel (the
+# derivation and commands are in the profile summaries shipped with the repository).
+MEASURED_TRAFFIC = {
+    "gemm_f32_512x768x2304_layernorm_512x768_w1_fused_bfuse_r": 28_460_000,
+}
