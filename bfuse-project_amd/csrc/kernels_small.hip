@@ -25,6 +25,8 @@ using ConvS3 = Conv3x3F32<64, 16, 8, 16, 16, 2, 2>;                    // two gr
 using PoolS = MaxPool3x3S2<4, 16, 16, 64>;
 using GemmB1 = GemmBf16NT<128, 1792, 64, 128, 224>;                   // one K-step
 using GemmB2 = GemmBf16NT<256, 1792, 192, 128, 224>;                  // two M-tiles, three K-steps
+using GemmB3 = GemmBf16NTDma<256, 1792, 320, 128, 224, 3>;             // direct-to-LDS ring, five K-steps
+using GemmB4 = GemmBf16NTDma<128, 1792, 192, 128, 224, 2>;             // two stages, three K-steps
 using NormRopeS = RmsNormRope<6, 8, 128, 2>;
 
 BFUSE_KERNEL(gemm_f32_64x32x48, GemmS1, ({{64, 32, 1, 1}, 4}), ({{32, 48, 1, 1}, 4}), ({{64, 48, 1, 1}, 4}))
@@ -39,6 +41,8 @@ BFUSE_KERNEL(conv3x3_f32_64x8x16_16, ConvS3, ({{1, 64, 8, 16}, 4}), ({{16, 64, 3
 BFUSE_KERNEL(maxpool3x3s2_f32_4x16x16, PoolS, ({{1, 4, 16, 16}, 4}), ({{1, 1, 1, 1}, 4}), ({{1, 4, 8, 8}, 4}))
 BFUSE_KERNEL(gemm_bf16_128x64x1792, GemmB1, ({{128, 64, 1, 1}, 2}), ({{1792, 64, 1, 1}, 2}), ({{128, 1792, 1, 1}, 2}))
 BFUSE_KERNEL(gemm_bf16_256x192x1792, GemmB2, ({{256, 192, 1, 1}, 2}), ({{1792, 192, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
+BFUSE_KERNEL(gemm_bf16_256x320x1792_d, GemmB3, ({{256, 320, 1, 1}, 2}), ({{1792, 320, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
+BFUSE_KERNEL(gemm_bf16_128x192x1792_d4, GemmB4, ({{128, 192, 1, 1}, 2}), ({{1792, 192, 1, 1}, 2}), ({{128, 1792, 1, 1}, 2}))
 BFUSE_KERNEL(rmsnorm_rope_bf16_6x1024, NormRopeS, ({{6, 1024, 1, 1}, 2}), ({{(int)NormRopeS::F_BYTES, 1, 1, 1}, 1}), ({{6, 1024, 1, 1}, 2}))
 
 // calibration kernel for the memory counters: 64 MiB read, 64 MiB written
@@ -56,3 +60,5 @@ BFUSE_BFUSE_KERNEL(conv3x3_f32_32x12x12_32, ConvS2, gemm_gelu_f32_96x128x192, Ge
 BFUSE_BFUSE_KERNEL(layernorm_8x256, LayerNormS, softmax_causal_2x256x256, SoftmaxS, , bfuse::kZigzag, 1, 1)
 BFUSE_BFUSE_KERNEL(gemm_bf16_256x192x1792, GemmB2, rmsnorm_rope_bf16_6x1024, NormRopeS, _c8, bfuse::kChunked, 8, 1)
 BFUSE_HFUSE_KERNEL(maxpool3x3s2_f32_4x16x16, PoolS, layernorm_8x256, LayerNormS)
+// the direct-to-LDS GEMM under horizontal fusion: its fence-free barrier becomes the LDS-counter one
+BFUSE_HFUSE_KERNEL(gemm_bf16_256x320x1792_d, GemmB3, rmsnorm_rope_bf16_6x1024, NormRopeS)

@@ -162,4 +162,230 @@ struct GemmBf16NT {
     }
 };
 
+// Same GEMM with the K-pipeline rebuilt around direct global->LDS loads
+// (global_load_lds_dwordx4): no staging registers, NSTG LDS stages in a ring, NSTG-1
+// K-steps of loads in flight while one is multiplied.  A wave-level load writes 64 lanes x
+// 16 bytes contiguously (8 rows of 128 bytes), so rows cannot be padded; instead the
+// 16-byte chunk c of row r is stored at chunk position c ^ ((r >> 1) & 7), which makes the
+// 128-bit operand reads of 16 consecutive rows hit 16 different bank groups.
+template <int M_, int N_, int K_, int BM_, int BN_, int NSTG_ = 3>
+struct GemmBf16NTDma {
+    static constexpr int M = M_, N = N_, K = K_, BM = BM_, BN = BN_, NSTG = NSTG_;
+    static constexpr int BK = 64;
+    static constexpr int THREADS = 256;
+    static constexpr int WM = BM / 2, WN = BN / 2;
+    static constexpr int TM = WM / 16, TN = WN / 16;
+    static constexpr int NKT = K / BK;
+    static constexpr int ROWS = BM + BN;
+    static constexpr int GROUPS = ROWS / 8;             // wave-level loads per stage
+    static constexpr int GPW = GROUPS / 4;              // per wave
+    static constexpr int STAGE_BYTES = ROWS * 128;
+    static constexpr int CPITCH = BN + 8;
+    static constexpr int OCHUNKS = BM * (BN / 8);
+    static_assert(M % BM == 0 && N % BN == 0 && K % BK == 0, "tile must divide the problem");
+    static_assert(WM % 16 == 0 && WN % 16 == 0 && BM % 8 == 0 && GROUPS % 4 == 0, "tile shape");
+    static_assert(OCHUNKS % THREADS == 0 && NSTG >= 2 && NSTG <= 4 && NKT >= NSTG - 1, "pipeline shape");
+    static constexpr int MT = M / BM, NT = N / BN;
+    static_assert((MT * NT) % 8 == 0 && NT % 8 == 0, "tiles are dealt to 8 XCDs");
+
+    static constexpr Dims3 GRID{MT * NT, 1, 1};
+    static constexpr Dims3 BLOCK{THREADS, 1, 1};
+    static constexpr bool HAS_BARRIERS = true;
+    static constexpr int EPI_BYTES = BM * CPITCH * 2;
+    struct Smem {
+        __attribute__((aligned(1024))) unsigned char t[(NSTG * STAGE_BYTES > EPI_BYTES) ? NSTG * STAGE_BYTES : EPI_BYTES];
+    };
+
+    // s_waitcnt vmcnt(n), other counters untouched (gfx9 encoding: vmcnt in bits 3:0 and 15:14)
+    template <int N_OUT>
+    __device__ static __forceinline__ void wait_vm()
+    {
+        __builtin_amdgcn_s_waitcnt((N_OUT & 0xF) | ((N_OUT >> 4) << 14) | 0x0F70);
+    }
+
+    typedef __attribute__((address_space(3))) unsigned char lds_u8;
+
+    // this wave's GPW wave-level loads of K-step kt into LDS stage `stage`
+    __device__ static __forceinline__ void issue(const unsigned short* const (&src)[GPW], lds_u8* wave_base, int stage, int kt)
+    {
+#if defined(__HIP_DEVICE_COMPILE__)
+#pragma unroll
+        for (int i = 0; i < GPW; ++i)
+            __builtin_amdgcn_global_load_lds(src[i] + kt * BK, wave_base + stage * STAGE_BYTES + i * 1024, 16, 0, 0);
+#endif
+    }
+
+    // ---- operand reads are issued and waited for by hand ------------------------------------
+    // The compiler waits for ALL outstanding LDS reads (lgkmcnt(0)) before the first MFMA
+    // that needs one of them, which throws away the read-ahead; written as asm it cannot see
+    // them, and each MFMA group waits only for the fragments it uses (LDS reads of a wave
+    // return in order, so "at most n outstanding" identifies which have landed).
+    template <int OFF>
+    __device__ static __forceinline__ bf16x8 lds_read(int addr)
+    {
+        bf16x8 r;
+#if defined(__HIP_DEVICE_COMPILE__)
+        if constexpr (OFF < 65536) {
+            asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
+        } else {
+            asm volatile("ds_read_b128 %0, %1" : "=v"(r) : "v"(addr + OFF));
+        }
+#else
+        r = bf16x8{};
+#endif
+        return r;
+    }
+    template <int N_OUT>
+    __device__ static __forceinline__ void wait_lds(bf16x8& b, bf16x8 (&a)[TM])
+    {
+#if defined(__HIP_DEVICE_COMPILE__)
+        static_assert(TM == 4, "the dependency list below names four A fragments");
+        asm volatile("s_waitcnt lgkmcnt(%5)" : "+v"(b), "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]) : "n"(N_OUT));
+#endif
+    }
+
+    static constexpr int STEPS = (BK / 32) * TN;
+    // reads still allowed in flight when MFMA group `st` starts: the B fragment one ahead, and
+    // the next K-substep's A fragments if they were issued after B[st]
+    static constexpr int allowed(int st)
+    {
+        int n = st + 1 < STEPS ? 1 : 0;
+        for (int ks = 0; ks + 1 < BK / 32; ++ks)
+            if (st == ks * TN + 2 || st == ks * TN + 3) n += TM;
+        return n;
+    }
+
+    template <int U, int ST>
+    __device__ static __forceinline__ void step_chain(f32x4 (&acc)[TM][TN], bf16x8 (&af)[BK / 32][TM], bf16x8 (&bq)[3],
+                                                      const int (&a_ad)[BK / 32][TM], const int (&b_ad)[BK / 32][TN])
+    {
+        if constexpr (ST < STEPS) {
+            constexpr int ks = ST / TN, b = ST % TN;
+            constexpr int OFF = U * STAGE_BYTES;
+            wait_lds<allowed(ST)>(bq[ST % 3], af[ks]);
+#pragma unroll
+            for (int a = 0; a < TM; ++a)
+                acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[ks][a], bq[ST % 3], acc[a][b], 0, 0, 0);
+            if constexpr (ST + 2 < STEPS) bq[(ST + 2) % 3] = lds_read<OFF>(b_ad[(ST + 2) / TN][(ST + 2) % TN]);
+            if constexpr (b == 1 && ks + 1 < BK / 32) {
+#pragma unroll
+                for (int a = 0; a < TM; ++a) af[ks + 1][a] = lds_read<OFF>(a_ad[ks + 1][a]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            step_chain<U, ST + 1>(acc, af, bq, a_ad, b_ad);
+        }
+    }
+
+    // one K-step out of LDS stage U
+    template <int U, class Sync>
+    __device__ static __forceinline__ void k_step(int kt, f32x4 (&acc)[TM][TN], const int (&a_ad)[BK / 32][TM],
+                                                  const int (&b_ad)[BK / 32][TN], const unsigned short* const (&src)[GPW],
+                                                  lds_u8* lds, Sync& sync)
+    {
+        if (kt >= NKT) return;
+        // loads of K-step kt have landed once at most the newer steps' loads are outstanding
+        if (kt + NSTG - 2 < NKT) wait_vm<GPW * (NSTG - 2)>();
+        else wait_vm<0>();
+        sync.raw();  // everyone's part of step kt is in LDS; everyone is done reading step kt-1
+        if (kt + NSTG - 1 < NKT) issue(src, lds, (U + NSTG - 1) % NSTG, kt + NSTG - 1);
+        constexpr int OFF = U * STAGE_BYTES;
+        bf16x8 af[BK / 32][TM], bq[3];
+#pragma unroll
+        for (int a = 0; a < TM; ++a) af[0][a] = lds_read<OFF>(a_ad[0][a]);
+        bq[0] = lds_read<OFF>(b_ad[0][0]);
+        bq[1] = lds_read<OFF>(b_ad[1 / TN][1 % TN]);
+        __builtin_amdgcn_sched_barrier(0);
+        step_chain<U, 0>(acc, af, bq, a_ad, b_ad);
+    }
+
+    template <class Sync>
+    __device__ static __forceinline__ void run(int vblock, int tid, Smem& sm, const void* I, const void* F,
+                                               void* O, Sync sync)
+    {
+        const unsigned short* __restrict__ A = static_cast<const unsigned short*>(I);
+        const unsigned short* __restrict__ Wt = static_cast<const unsigned short*>(F);
+        unsigned short* __restrict__ C = static_cast<unsigned short*>(O);
+        const int xcd = vblock & 7, slot = vblock >> 3;
+        const int nt = xcd * (NT / 8) + slot / MT, mt = slot % MT;
+        const int m0 = mt * BM, n0 = nt * BN;
+        const int wave = tid >> 6, lane = tid & 63;
+        const int wm = wave >> 1, wn = wave & 1;
+        const int li = lane & 15, kq = lane >> 4;
+
+        // per-lane source of each of this wave's GPW loads (K-step 0); swizzled chunk
+        const unsigned short* src[GPW];
+#pragma unroll
+        for (int i = 0; i < GPW; ++i) {
+            const int row = 8 * (wave * GPW + i) + (lane >> 3);
+            const int gc = (lane & 7) ^ ((row >> 1) & 7);
+            src[i] = (row < BM ? A + (size_t)(m0 + row) * K : Wt + (size_t)(n0 + row - BM) * K) + gc * 8;
+        }
+        lds_u8* const lds = (lds_u8*)sm.t + wave * GPW * 1024;
+
+        f32x4 acc[TM][TN];
+#pragma unroll
+        for (int a = 0; a < TM; ++a)
+#pragma unroll
+            for (int b = 0; b < TN; ++b) acc[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll
+        for (int s = 0; s < NSTG - 1; ++s) issue(src, lds, s, s);
+
+        // byte offset inside a stage of every operand fragment this lane reads (K-substep ks,
+        // block a / b), with the chunk swizzle folded in: loop invariant
+        int a_rd[BK / 32][TM], b_rd[BK / 32][TN];
+#pragma unroll
+        for (int ks = 0; ks < BK / 32; ++ks) {
+            const int c = ks * 4 + kq;
+#pragma unroll
+            for (int a = 0; a < TM; ++a) {
+                const int row = wm * WM + a * 16 + li;
+                a_rd[ks][a] = row * 128 + ((c ^ ((row >> 1) & 7)) << 4);
+            }
+#pragma unroll
+            for (int b = 0; b < TN; ++b) {
+                const int row = BM + wn * WN + b * 16 + li;
+                b_rd[ks][b] = row * 128 + ((c ^ ((row >> 1) & 7)) << 4);
+            }
+        }
+
+        const unsigned lds_base = (unsigned)(unsigned long long)(lds_u8*)sm.t;
+        int a_ad[BK / 32][TM], b_ad[BK / 32][TN];  // absolute LDS byte addresses in stage 0
+#pragma unroll
+        for (int ks = 0; ks < BK / 32; ++ks) {
+#pragma unroll
+            for (int a = 0; a < TM; ++a) a_ad[ks][a] = a_rd[ks][a] + (int)lds_base;
+#pragma unroll
+            for (int b = 0; b < TN; ++b) b_ad[ks][b] = b_rd[ks][b] + (int)lds_base;
+        }
+
+        // K-steps are taken NSTG at a time so that the LDS stage of each is a compile-time constant
+        for (int kt0 = 0; kt0 < NKT; kt0 += NSTG) {
+            k_step<0>(kt0, acc, a_ad, b_ad, src, lds, sync);
+            if constexpr (NSTG > 1) k_step<1>(kt0 + 1, acc, a_ad, b_ad, src, lds, sync);
+            if constexpr (NSTG > 2) k_step<2>(kt0 + 2, acc, a_ad, b_ad, src, lds, sync);
+            if constexpr (NSTG > 3) k_step<3>(kt0 + 3, acc, a_ad, b_ad, src, lds, sync);
+        }
+        sync();  // all waves are done reading the last stage before the tile buffer overwrites it
+
+        unsigned short* ct = reinterpret_cast<unsigned short*>(sm.t);
+#pragma unroll
+        for (int a = 0; a < TM; ++a)
+#pragma unroll
+            for (int b = 0; b < TN; ++b)
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    ct[(wm * WM + a * 16 + 4 * kq + v) * CPITCH + wn * WN + b * 16 + li] =
+                        (unsigned short)f32_to_bf16_bits(acc[a][b][v]);
+        sync();
+#pragma unroll
+        for (int i = 0; i < OCHUNKS / THREADS; ++i) {
+            const int c = tid + i * THREADS;
+            const int row = c / (BN / 8), col = (c % (BN / 8)) * 8;
+            *reinterpret_cast<u32x4*>(C + (size_t)(m0 + row) * N + n0 + col) =
+                *reinterpret_cast<const u32x4*>(ct + row * CPITCH + col);
+        }
+    }
+};
+
 }  // namespace bfuse

@@ -42,7 +42,7 @@ __device__ __forceinline__ float gelu_tanh(float x)
     return (0.5f * x) * (tanhf(u) + 1.0f);
 }
 
-template <int M_, int N_, int K_, int BM_, int BN_, int KS_, int EPI_ = kEpiNone, int NBUF_ = 2>
+template <int M_, int N_, int K_, int BM_, int BN_, int KS_, int EPI_ = kEpiNone, int NBUF_ = 2, int SCHED_ = 1>
 struct GemmF32 {
     static constexpr int M = M_, N = N_, K = K_, BM = BM_, BN = BN_, KS = KS_, EPI = EPI_;
     static constexpr int TM = BM / 16;          // 16-row blocks per tile
@@ -176,6 +176,9 @@ struct GemmF32 {
                 if (s < NSTAGE) {
                     if (s + NBUF - 1 < NSTAGE)
                         load_stage(buf[(u + NBUF - 1) % NBUF], A, B, m0, n0, kbeg + (s + NBUF - 1) * STAGE, lane);
+                    // keep the loads ahead of this stage's MFMAs: the scheduler otherwise sinks
+                    // them to the end of the stage and the next stage waits on them at once
+                    if constexpr (SCHED_ == 1) __builtin_amdgcn_sched_barrier(0);
                     mma_stage(acc, buf[u]);
                 }
             }

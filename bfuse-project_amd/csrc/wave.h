@@ -52,6 +52,15 @@ static __device__ unsigned int g_sync_timeouts;
 // hardware barrier only counts waves that are still alive).
 struct BlockSync {
     __device__ __forceinline__ void operator()() const { __syncthreads(); }
+    // Barrier WITHOUT a memory fence: only this wave's LDS accesses are drained.  For
+    // pipelines that keep global->LDS loads in flight across the barrier and account for
+    // them with explicit s_waitcnt vmcnt(n) (a fence would wait for all of them).
+    __device__ __forceinline__ void raw() const
+    {
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    }
 };
 
 // Barrier over the waves of ONE side of a horizontally fused workgroup.  gfx950 has no
@@ -83,6 +92,26 @@ struct GroupSync {
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    }
+
+    // Same meeting point without fences (see BlockSync::raw): the caller has already waited
+    // for the loads the other waves depend on; LDS operations of one wave execute in order,
+    // so reads issued after the poll see what the other waves wrote before they arrived.
+    __device__ __forceinline__ void raw()
+    {
+        ++epoch;
+        const unsigned int target = waves * epoch;
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if ((threadIdx.x & 63) == 0) atomicAdd(counter, 1u);
+        unsigned int spins = 0;
+        while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < target) {
+            __builtin_amdgcn_s_sleep(1);
+            if (++spins == kSpinLimit) {
+                if ((threadIdx.x & 63) == 0) atomicAdd(&g_sync_timeouts, 1u);
+                break;
+            }
+        }
+        asm volatile("" ::: "memory");
     }
 };
 

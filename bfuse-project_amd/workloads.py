@@ -138,7 +138,8 @@ PAIRS: Dict[int, Pair] = {
     5: Pair(5, "GEMM bf16 [512x4096].[14336x4096]^T (fp32 acc) || RMSNorm+RoPE [512x4096] bf16, bfuse",
             "gemm_bf16_512x4096x14336", "rmsnorm_rope_bf16_512x4096", "bfuse",
             [("bfuse", ""), ("bfuse", "_c256")],
-            [("gemm_bf16_512x4096x14336", "rmsnorm_rope_bf16_512x4096_w4", "bfuse", "_c256")], _pair5_inputs,
+            [("gemm_bf16_512x4096x14336", "rmsnorm_rope_bf16_512x4096_w4", "bfuse", "_c256"),
+             ("gemm_bf16_512x4096x14336_d", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256")], _pair5_inputs,
             bytes1=(512 * 4096 + 4096 * 14336 + 512 * 14336) * 2, bytes2=2 * 512 * 4096 * 2 + 4096 * 2,
             flops=2 * 512 * 4096 * 14336, bound="mfma", peak=2500.0, dtype="bf16", tol=1e-2),
 }

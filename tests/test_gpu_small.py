@@ -57,6 +57,10 @@ def _cases():
                                   lambda I, F: orf.gemm_bf16(I.reshape(128, 64), F.reshape(1792, 64), b_is_nk=True), 1e-2, True),
         "gemm_bf16_256x192x1792": (lambda s: (f32_to_bf16(fill_normal(s, 256 * 192, 0, 1)), f32_to_bf16(fill_normal(s + 1, 1792 * 192, 0, 0.1))),
                                    lambda I, F: orf.gemm_bf16(I.reshape(256, 192), F.reshape(1792, 192), b_is_nk=True), 1e-2, True),
+        "gemm_bf16_256x320x1792_d": (lambda s: (f32_to_bf16(fill_normal(s, 256 * 320, 0, 1)), f32_to_bf16(fill_normal(s + 1, 1792 * 320, 0, 0.1))),
+                                     lambda I, F: orf.gemm_bf16(I.reshape(256, 320), F.reshape(1792, 320), b_is_nk=True), 1e-2, True),
+        "gemm_bf16_128x192x1792_d4": (lambda s: (f32_to_bf16(fill_normal(s, 128 * 192, 0, 1)), f32_to_bf16(fill_normal(s + 1, 1792 * 192, 0, 0.1))),
+                                      lambda I, F: orf.gemm_bf16(I.reshape(128, 192), F.reshape(1792, 192), b_is_nk=True), 1e-2, True),
         "rmsnorm_rope_bf16_6x1024": (lambda s: (f32_to_bf16(fill_normal(s, 6 * 1024, 0, 1.5)), _norm_rope_operand(6, 1024, 128, s + 1)),
                                      lambda I, F: orf.rmsnorm_rope_bf16(I.reshape(6, 1024), *wl.unpack_norm_rope_operand(F, 6, 1024, 128), heads=8, eps=1e-5), 1e-2, True),
     }
@@ -71,6 +75,7 @@ FUSIONS = [
     ("layernorm_8x256", "softmax_causal_2x256x256", "bfuse", ""),
     ("gemm_bf16_256x192x1792", "rmsnorm_rope_bf16_6x1024", "bfuse", "_c8"),
     ("maxpool3x3s2_f32_4x16x16", "layernorm_8x256", "hfuse", ""),
+    ("gemm_bf16_256x320x1792_d", "rmsnorm_rope_bf16_6x1024", "hfuse", ""),
 ]
 
 
