@@ -15,9 +15,9 @@ using Softmax1 = SoftmaxCausal<12, 512, 1, 1>;
 using Softmax4x6 = SoftmaxCausal<12, 512, 4, 6, 3>;
 using Softmax4b = SoftmaxCausal<12, 512, 4, 4, 4>;   // 384 workgroups, 4 rows in flight per wave
 // GEMM + GELU: 256 workgroups, four waves split K = 768
-using GemmFc = GemmF32<512, 3072, 768, 64, 96, 4, kEpiGeluTanh>;     // 8 x 32 tiles of 64x96
-using GemmFcH = GemmF32<512, 3072, 768, 32, 96, 4, kEpiGeluTanh>;    // 32 x 16 tiles of 32x96, two per CU
-using GemmFcW = GemmF32<512, 3072, 768, 32, 192, 4, kEpiGeluTanh>;   // 16 x 16 tiles of 32x192
+using GemmFc = GemmF32<512, 3072, 768, 64, 96, 4, kEpiGeluTanh, 2, 0>;     // 8 x 32 tiles of 64x96
+using GemmFcH = GemmF32<512, 3072, 768, 32, 96, 4, kEpiGeluTanh, 2, 0>;    // 32 x 16 tiles of 32x96, two per CU
+using GemmFcW = GemmF32<512, 3072, 768, 32, 192, 4, kEpiGeluTanh, 2, 0>;   // 16 x 16 tiles of 32x192
 
 
 BFUSE_KERNEL(softmax_causal_12x512x512, Softmax4, ({{12, 512, 512, 1}, 4}), ({{1, 1, 1, 1}, 4}), ({{12, 512, 512, 1}, 4}))
@@ -38,3 +38,11 @@ BFUSE_BFUSE_KERNEL(softmax_causal_12x512x512_b4, Softmax4b, gemm_gelu_f32_512x76
 BFUSE_BFUSE_KERNEL(softmax_causal_12x512x512_b4, Softmax4b, gemm_gelu_f32_512x768x3072_h, GemmFcH, _c256, bfuse::kChunked, 256, 1)
 BFUSE_BFUSE_KERNEL(softmax_causal_12x512x512_b4, Softmax4b, gemm_gelu_f32_512x768x3072_h, GemmFcH, _c512, bfuse::kChunked, 512, 1)
 BFUSE_BFUSE_KERNEL(softmax_causal_12x512x512, Softmax4, gemm_gelu_f32_512x768x3072_h, GemmFcH, _c512, bfuse::kChunked, 512, 1)
+// 32x96 tiles with three register stages; softmax as 512 workgroups (4 waves x 3 rows, all in flight)
+using GemmFcH3 = GemmF32<512, 3072, 768, 32, 96, 4, kEpiGeluTanh, 3, 0>;
+using Softmax4x3 = SoftmaxCausal<12, 512, 4, 3, 3>;
+BFUSE_KERNEL(gemm_gelu_f32_512x768x3072_h3, GemmFcH3, ({{512, 768, 1, 1}, 4}), ({{768, 3072, 1, 1}, 4}), ({{512, 3072, 1, 1}, 4}))
+BFUSE_KERNEL(softmax_causal_12x512x512_r3, Softmax4x3, ({{12, 512, 512, 1}, 4}), ({{1, 1, 1, 1}, 4}), ({{12, 512, 512, 1}, 4}))
+BFUSE_BFUSE_KERNEL(softmax_causal_12x512x512_b4, Softmax4b, gemm_gelu_f32_512x768x3072_h3, GemmFcH3, _c512, bfuse::kChunked, 512, 1)
+BFUSE_HFUSE_KERNEL(softmax_causal_12x512x512_r3, Softmax4x3, gemm_gelu_f32_512x768x3072_h, GemmFcH)
+BFUSE_HFUSE_KERNEL(softmax_causal_12x512x512_r3, Softmax4x3, gemm_gelu_f32_512x768x3072_h3, GemmFcH3)

@@ -9,17 +9,17 @@ using namespace bfuse;
 
 BFUSE_MODULE_PROLOGUE()
 
-using GemmGate = GemmBf16NT<512, 14336, 4096, 128, 224>;    // 4 x 64 = 256 workgroups
-using GemmGateD = GemmBf16NTDma<512, 14336, 4096, 128, 224, 3>;
+using GemmGate = GemmBf16NTDma<512, 14336, 4096, 128, 224, 3, 4>;   // 4 x 64 = 256 workgroups, direct-to-LDS ring
+using GemmGateV = GemmBf16NT<512, 14336, 4096, 128, 224>;           // same tiles, operands staged through VGPRs
 using NormRope1 = RmsNormRope<512, 32, 128, 1>;             // 512 one-wave workgroups
 using NormRope4 = RmsNormRope<512, 32, 128, 4>;             // 128 four-wave workgroups
 
 BFUSE_KERNEL(gemm_bf16_512x4096x14336, GemmGate, ({{512, 4096, 1, 1}, 2}), ({{14336, 4096, 1, 1}, 2}), ({{512, 14336, 1, 1}, 2}))
-BFUSE_KERNEL(gemm_bf16_512x4096x14336_d, GemmGateD, ({{512, 4096, 1, 1}, 2}), ({{14336, 4096, 1, 1}, 2}), ({{512, 14336, 1, 1}, 2}))
+BFUSE_KERNEL(gemm_bf16_512x4096x14336_v, GemmGateV, ({{512, 4096, 1, 1}, 2}), ({{14336, 4096, 1, 1}, 2}), ({{512, 14336, 1, 1}, 2}))
 BFUSE_KERNEL(rmsnorm_rope_bf16_512x4096, NormRope1, ({{512, 4096, 1, 1}, 2}), ({{(int)NormRope1::F_BYTES, 1, 1, 1}, 1}), ({{512, 4096, 1, 1}, 2}))
 BFUSE_KERNEL(rmsnorm_rope_bf16_512x4096_w4, NormRope4, ({{512, 4096, 1, 1}, 2}), ({{(int)NormRope4::F_BYTES, 1, 1, 1}, 1}), ({{512, 4096, 1, 1}, 2}))
 
 BFUSE_BFUSE_KERNEL(gemm_bf16_512x4096x14336, GemmGate, rmsnorm_rope_bf16_512x4096, NormRope1, , bfuse::kZigzag, 1, 1)
 BFUSE_BFUSE_KERNEL(gemm_bf16_512x4096x14336, GemmGate, rmsnorm_rope_bf16_512x4096, NormRope1, _c256, bfuse::kChunked, 256, 1)
 BFUSE_BFUSE_KERNEL(gemm_bf16_512x4096x14336, GemmGate, rmsnorm_rope_bf16_512x4096_w4, NormRope4, _c256, bfuse::kChunked, 256, 1)
-BFUSE_BFUSE_KERNEL(gemm_bf16_512x4096x14336_d, GemmGateD, rmsnorm_rope_bf16_512x4096, NormRope1, _c256, bfuse::kChunked, 256, 1)
+BFUSE_BFUSE_KERNEL(gemm_bf16_512x4096x14336_v, GemmGateV, rmsnorm_rope_bf16_512x4096, NormRope1, _c256, bfuse::kChunked, 256, 1)

@@ -168,7 +168,7 @@ struct GemmBf16NT {
 // 16 bytes contiguously (8 rows of 128 bytes), so rows cannot be padded; instead the
 // 16-byte chunk c of row r is stored at chunk position c ^ ((r >> 1) & 7), which makes the
 // 128-bit operand reads of 16 consecutive rows hit 16 different bank groups.
-template <int M_, int N_, int K_, int BM_, int BN_, int NSTG_ = 3>
+template <int M_, int N_, int K_, int BM_, int BN_, int NSTG_ = 3, int PD_ = 4>
 struct GemmBf16NTDma {
     static constexpr int M = M_, N = N_, K = K_, BM = BM_, BN = BN_, NSTG = NSTG_;
     static constexpr int BK = 64;
@@ -185,6 +185,7 @@ struct GemmBf16NTDma {
     static_assert(M % BM == 0 && N % BN == 0 && K % BK == 0, "tile must divide the problem");
     static_assert(WM % 16 == 0 && WN % 16 == 0 && BM % 8 == 0 && GROUPS % 4 == 0, "tile shape");
     static_assert(OCHUNKS % THREADS == 0 && NSTG >= 2 && NSTG <= 4 && NKT >= NSTG - 1, "pipeline shape");
+    static_assert(PD_ >= 1 && PD_ < (BK / 32) * (BN / 32), "read-ahead distance");
     static constexpr int MT = M / BM, NT = N / BN;
     static_assert((MT * NT) % 8 == 0 && NT % 8 == 0, "tiles are dealt to 8 XCDs");
 
@@ -245,28 +246,33 @@ struct GemmBf16NTDma {
     }
 
     static constexpr int STEPS = (BK / 32) * TN;
-    // reads still allowed in flight when MFMA group `st` starts: the B fragment one ahead, and
-    // the next K-substep's A fragments if they were issued after B[st]
+    static constexpr int PD = PD_;      // B fragments are read PD MFMA groups ahead
+    static constexpr int RING = PD + 1;
+    // reads still allowed in flight when MFMA group `st` starts: the B fragments ahead of it,
+    // and the next K-substep's A fragments (issued after group ks*TN+1) if they came after B[st]
     static constexpr int allowed(int st)
     {
-        int n = st + 1 < STEPS ? 1 : 0;
-        for (int ks = 0; ks + 1 < BK / 32; ++ks)
-            if (st == ks * TN + 2 || st == ks * TN + 3) n += TM;
+        int n = (STEPS - 1 - st) < (PD - 1) ? (STEPS - 1 - st) : (PD - 1);
+        for (int ks = 0; ks + 1 < BK / 32; ++ks) {
+            const int s_af = ks * TN + 1;
+            const int lo = st - PD > 0 ? st - PD : 0;
+            if (s_af >= lo && s_af <= st - 1) n += TM;
+        }
         return n;
     }
 
     template <int U, int ST>
-    __device__ static __forceinline__ void step_chain(f32x4 (&acc)[TM][TN], bf16x8 (&af)[BK / 32][TM], bf16x8 (&bq)[3],
+    __device__ static __forceinline__ void step_chain(f32x4 (&acc)[TM][TN], bf16x8 (&af)[BK / 32][TM], bf16x8 (&bq)[RING],
                                                       const int (&a_ad)[BK / 32][TM], const int (&b_ad)[BK / 32][TN])
     {
         if constexpr (ST < STEPS) {
             constexpr int ks = ST / TN, b = ST % TN;
             constexpr int OFF = U * STAGE_BYTES;
-            wait_lds<allowed(ST)>(bq[ST % 3], af[ks]);
+            wait_lds<allowed(ST)>(bq[ST % RING], af[ks]);
 #pragma unroll
             for (int a = 0; a < TM; ++a)
-                acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[ks][a], bq[ST % 3], acc[a][b], 0, 0, 0);
-            if constexpr (ST + 2 < STEPS) bq[(ST + 2) % 3] = lds_read<OFF>(b_ad[(ST + 2) / TN][(ST + 2) % TN]);
+                acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[ks][a], bq[ST % RING], acc[a][b], 0, 0, 0);
+            if constexpr (ST + PD < STEPS) bq[(ST + PD) % RING] = lds_read<OFF>(b_ad[(ST + PD) / TN][(ST + PD) % TN]);
             if constexpr (b == 1 && ks + 1 < BK / 32) {
 #pragma unroll
                 for (int a = 0; a < TM; ++a) af[ks + 1][a] = lds_read<OFF>(a_ad[ks + 1][a]);
@@ -289,11 +295,11 @@ struct GemmBf16NTDma {
         sync.raw();  // everyone's part of step kt is in LDS; everyone is done reading step kt-1
         if (kt + NSTG - 1 < NKT) issue(src, lds, (U + NSTG - 1) % NSTG, kt + NSTG - 1);
         constexpr int OFF = U * STAGE_BYTES;
-        bf16x8 af[BK / 32][TM], bq[3];
+        bf16x8 af[BK / 32][TM], bq[RING];
 #pragma unroll
         for (int a = 0; a < TM; ++a) af[0][a] = lds_read<OFF>(a_ad[0][a]);
-        bq[0] = lds_read<OFF>(b_ad[0][0]);
-        bq[1] = lds_read<OFF>(b_ad[1 / TN][1 % TN]);
+#pragma unroll
+        for (int p = 0; p < PD; ++p) bq[p] = lds_read<OFF>(b_ad[p / TN][p % TN]);
         __builtin_amdgcn_sched_barrier(0);
         step_chain<U, 0>(acc, af, bq, a_ad, b_ad);
     }
