@@ -2,6 +2,7 @@
 // block-fused with the MLP up-projection GEMM [512x768].[768x3072] fp32 + tanh-GELU.
 #include "fuse.h"
 #include "ops_gemm_f32.h"
+#include "ops_gemm_f32_lds.h"
 #include "ops_rowwise.h"
 
 using namespace bfuse;
@@ -46,3 +47,10 @@ BFUSE_KERNEL(softmax_causal_12x512x512_r3, Softmax4x3, ({{12, 512, 512, 1}, 4}),
 BFUSE_BFUSE_KERNEL(softmax_causal_12x512x512_b4, Softmax4b, gemm_gelu_f32_512x768x3072_h3, GemmFcH3, _c512, bfuse::kChunked, 512, 1)
 BFUSE_HFUSE_KERNEL(softmax_causal_12x512x512_r3, Softmax4x3, gemm_gelu_f32_512x768x3072_h, GemmFcH)
 BFUSE_HFUSE_KERNEL(softmax_causal_12x512x512_r3, Softmax4x3, gemm_gelu_f32_512x768x3072_h3, GemmFcH3)
+// LDS-staged GEMM: 64x96 tiles, eight waves of 16x48, no K split; softmax as 256 workgroups of 4 waves x 6 rows
+using GemmFcL = GemmF32Lds<512, 3072, 768, 64, 96, 48, kEpiGeluTanh, 4>;
+using Softmax4x6b = SoftmaxCausal<12, 512, 4, 6, 3>;
+BFUSE_KERNEL(gemm_gelu_f32_512x768x3072_l, GemmFcL, ({{512, 768, 1, 1}, 4}), ({{768, 3072, 1, 1}, 4}), ({{512, 3072, 1, 1}, 4}))
+BFUSE_HFUSE_KERNEL(softmax_causal_12x512x512_r6, Softmax4x6, gemm_gelu_f32_512x768x3072_l, GemmFcL)
+BFUSE_BFUSE_KERNEL(softmax_causal_12x512x512_b4, Softmax4b, gemm_gelu_f32_512x768x3072_l, GemmFcL, _c256, bfuse::kChunked, 256, 1)
+BFUSE_BFUSE_KERNEL(softmax_causal_12x512x512, Softmax4, gemm_gelu_f32_512x768x3072_l, GemmFcL, _c256, bfuse::kChunked, 256, 1)

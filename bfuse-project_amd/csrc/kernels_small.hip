@@ -7,6 +7,7 @@
 #include "ops_conv.h"
 #include "ops_gemm_bf16.h"
 #include "ops_gemm_f32.h"
+#include "ops_gemm_f32_lds.h"
 #include "ops_rowwise.h"
 
 using namespace bfuse;
@@ -16,6 +17,7 @@ BFUSE_MODULE_PROLOGUE()
 using GemmS1 = GemmF32<64, 48, 32, 16, 48, 1>;                        // one wave, 16-column groups only
 using GemmS2 = GemmF32<96, 192, 128, 32, 64, 2, kEpiGeluTanh, 3>;     // 2 waves, GELU, 3 register stages
 using GemmS3 = GemmF32<32, 144, 256, 32, 144, 4>;                     // the 64+64+16 column split, one tile
+using GemmS4 = GemmF32Lds<128, 192, 160, 64, 96, 48, kEpiNone, 3>;          // LDS-staged, 2x2 tiles, five K-steps
 using BiasReluS = BiasRelu<4096, 64, 4>;
 using LayerNormS = LayerNorm<8, 256, 2, 1>;
 using SoftmaxS = SoftmaxCausal<2, 256, 2, 2, 2>;
@@ -32,6 +34,7 @@ using NormRopeS = RmsNormRope<6, 8, 128, 2>;
 BFUSE_KERNEL(gemm_f32_64x32x48, GemmS1, ({{64, 32, 1, 1}, 4}), ({{32, 48, 1, 1}, 4}), ({{64, 48, 1, 1}, 4}))
 BFUSE_KERNEL(gemm_gelu_f32_96x128x192, GemmS2, ({{96, 128, 1, 1}, 4}), ({{128, 192, 1, 1}, 4}), ({{96, 192, 1, 1}, 4}))
 BFUSE_KERNEL(gemm_f32_32x256x144, GemmS3, ({{32, 256, 1, 1}, 4}), ({{256, 144, 1, 1}, 4}), ({{32, 144, 1, 1}, 4}))
+BFUSE_KERNEL(gemm_f32_128x160x192_l, GemmS4, ({{128, 160, 1, 1}, 4}), ({{160, 192, 1, 1}, 4}), ({{128, 192, 1, 1}, 4}))
 BFUSE_KERNEL(bias_relu_4096, BiasReluS, ({{4096, 1, 1, 1}, 4}), ({{4096, 1, 1, 1}, 4}), ({{4096, 1, 1, 1}, 4}))
 BFUSE_KERNEL(layernorm_8x256, LayerNormS, ({{8, 256, 1, 1}, 4}), ({{2, 256, 1, 1}, 4}), ({{8, 256, 1, 1}, 4}))
 BFUSE_KERNEL(softmax_causal_2x256x256, SoftmaxS, ({{2, 256, 256, 1}, 4}), ({{1, 1, 1, 1}, 4}), ({{2, 256, 256, 1}, 4}))
@@ -62,3 +65,4 @@ BFUSE_BFUSE_KERNEL(gemm_bf16_256x192x1792, GemmB2, rmsnorm_rope_bf16_6x1024, Nor
 BFUSE_HFUSE_KERNEL(maxpool3x3s2_f32_4x16x16, PoolS, layernorm_8x256, LayerNormS)
 // the direct-to-LDS GEMM under horizontal fusion: its fence-free barrier becomes the LDS-counter one
 BFUSE_HFUSE_KERNEL(gemm_bf16_256x320x1792_d, GemmB3, rmsnorm_rope_bf16_6x1024, NormRopeS)
+BFUSE_HFUSE_KERNEL(gemm_f32_128x160x192_l, GemmS4, bias_relu_4096, BiasReluS)
