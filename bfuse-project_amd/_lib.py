@@ -56,7 +56,7 @@ EXPORTS = [
     "bfuse_set_elem_bytes", "initialize_kernel1", "initialize_kernel2", "finalize_kernel1", "finalize_kernel2",
     "run_kernel1", "run_kernel2", "run_parallel", "run_fuse",
     "bfuse_upload", "bfuse_zero_output", "bfuse_download", "bfuse_synchronize", "bfuse_launch",
-    "bfuse_time", "bfuse_time_batched",
+    "bfuse_time", "bfuse_time_batched", "bfuse_module_load", "bfuse_module_unload", "bfuse_module_launch",
     "bfuse_fill_uniform", "bfuse_fill_normal", "bfuse_f32_to_bf16", "bfuse_bf16_to_f32", "bfuse_check_matrix",
 ]
 
@@ -104,6 +104,8 @@ def lib():
         fp = C.POINTER(C.c_float)
         l.bfuse_time.argtypes = [C.c_int, vp, up, up, vp, up, up, C.c_int, C.c_int, fp, fp, fp]
         l.bfuse_time_batched.argtypes = [C.c_int, vp, up, up, vp, up, up, C.c_int, C.c_int, fp]
+        l.bfuse_module_load.argtypes = [C.c_char_p, ip]
+        l.bfuse_module_launch.argtypes = [C.c_int, C.c_char_p, up, up, C.c_int, C.c_int, fp]
         _LIB = l
     return _LIB
 

@@ -643,6 +643,94 @@ int bfuse_time_batched(int mode, const void* fa, const unsigned* ga, const unsig
     return BFUSE_OK;
 }
 
+// ---- kernels from a code object -------------------------------------------------------------
+static std::vector<hipModule_t>& modules()
+{
+    static std::vector<hipModule_t> m;
+    return m;
+}
+
+int bfuse_module_load(const char* path, int* module_id)
+{
+    if (!g.inited) return fail(BFUSE_ERR_STATE, "bfuse_init has not been called");
+    if (!path || !module_id) return fail(BFUSE_ERR_ARG, "null argument");
+    hipModule_t mod = nullptr;
+    hipError_t st = hipModuleLoad(&mod, path);
+    if (st != hipSuccess) {
+        (void)hipGetLastError();  // do not leave the failure for the next call to find
+        return fail(BFUSE_ERR_HIP, "hipModuleLoad(%s): %s", path, hipGetErrorString(st));
+    }
+    auto& ms = modules();
+    for (size_t i = 0; i < ms.size(); ++i)
+        if (!ms[i]) {
+            ms[i] = mod;
+            *module_id = (int)i;
+            return BFUSE_OK;
+        }
+    ms.push_back(mod);
+    *module_id = (int)ms.size() - 1;
+    return BFUSE_OK;
+}
+
+int bfuse_module_unload(int id)
+{
+    auto& ms = modules();
+    if (id < 0 || id >= (int)ms.size() || !ms[id]) return fail(BFUSE_ERR_ARG, "unknown module %d", id);
+    HIP_TRY(hipModuleUnload(ms[id]));
+    ms[id] = nullptr;
+    return BFUSE_OK;
+}
+
+int bfuse_module_launch(int id, const char* name, const unsigned* grid, const unsigned* block, int n_ptrs, int side,
+                        float* us_out)
+{
+    auto& ms = modules();
+    if (id < 0 || id >= (int)ms.size() || !ms[id]) return fail(BFUSE_ERR_ARG, "unknown module %d", id);
+    if (!name || !grid || !block) return fail(BFUSE_ERR_ARG, "null argument");
+    if (n_ptrs != 3 && n_ptrs != 6) return fail(BFUSE_ERR_ARG, "n_ptrs must be 3 or 6");
+    if (n_ptrs == 3 && side != 1 && side != 2) return fail(BFUSE_ERR_ARG, "side must be 1 or 2");
+    for (int i = 0; i < 3; ++i)
+        if (grid[i] == 0 || block[i] == 0) return fail(BFUSE_ERR_ARG, "empty launch shape");
+    if ((size_t)block[0] * block[1] * block[2] > 1024) return fail(BFUSE_ERR_ARG, "more than 1024 threads per workgroup");
+    hipFunction_t fn = nullptr;
+    hipError_t st = hipModuleGetFunction(&fn, ms[id], name);
+    if (st != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(BFUSE_ERR_ARG, "kernel '%s' is not in module %d: %s", name, id, hipGetErrorString(st));
+    }
+    void* ptrs[6];
+    if (n_ptrs == 3) {
+        Side& s = g.side[side - 1];
+        if (!s.live) return fail(BFUSE_ERR_STATE, "kernel%d is not initialized", side);
+        for (int i = 0; i < 3; ++i) ptrs[i] = s.buf[i];
+    } else {
+        if (!g.side[0].live || !g.side[1].live) return fail(BFUSE_ERR_STATE, "both sides must be initialized");
+        for (int i = 0; i < 3; ++i) {
+            ptrs[i] = g.side[0].buf[i];
+            ptrs[3 + i] = g.side[1].buf[i];
+        }
+    }
+    void* args[6];
+    for (int i = 0; i < n_ptrs; ++i) args[i] = &ptrs[i];
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    if (us_out) {
+        HIP_TRY(hipEventCreate(&e0));
+        HIP_TRY(hipEventCreate(&e1));
+    }
+    HIP_TRY(hipExtModuleLaunchKernel(fn, grid[0] * block[0], grid[1] * block[1], grid[2] * block[2], block[0], block[1],
+                                     block[2], 0, nullptr, args, nullptr, e0, e1, 0));
+    if (us_out) {
+        HIP_TRY(hipDeviceSynchronize());
+        HIP_TRY(hipGetLastError());
+        float ms_ = 0.f;
+        HIP_TRY(hipEventElapsedTime(&ms_, e0, e1));
+        *us_out = ms_ * 1000.f;
+        HIP_TRY(hipEventDestroy(e0));
+        HIP_TRY(hipEventDestroy(e1));
+    }
+    return BFUSE_OK;
+}
+
 // ---- synthetic inputs and checks ------------------------------------------------------------
 void bfuse_fill_uniform(unsigned long long seed, size_t n, float lo, float hi, float* out)
 {

@@ -189,6 +189,60 @@ class Operation:
         return us.value
 
 
+class GenericOperation:
+    """Two sides with caller-given shapes, for kernels that come from a code object (the
+    front end's output) rather than from the library's registry."""
+
+    def __init__(self, shapes1, shapes2, device: int = 0):
+        self.l = _lib.lib()
+        _lib.check(self.l.bfuse_init(device))
+        for side in (1, 2):
+            _lib.check(self.l.bfuse_set_elem_bytes(side, 4, 4, 4))
+        self.shapes = [[_i4(s) for s in shapes1], [_i4(s) for s in shapes2]]
+        self.nelem = [[int(np.prod(s)) for s in shapes1], [int(np.prod(s)) for s in shapes2]]
+        _lib.check(self.l.initialize_kernel1(*self.shapes[0]))
+        _lib.check(self.l.initialize_kernel2(*self.shapes[1]))
+        self.modules = []
+
+    def close(self):
+        for m in self.modules:
+            self.l.bfuse_module_unload(m)
+        _lib.check(self.l.finalize_kernel1())
+        _lib.check(self.l.finalize_kernel2())
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def load(self, path: str) -> int:
+        mid = C.c_int(-1)
+        _lib.check(self.l.bfuse_module_load(path.encode(), C.byref(mid)))
+        self.modules.append(mid.value)
+        return mid.value
+
+    def upload(self, side: int, I, F):
+        I, F = np.ascontiguousarray(I, np.float32), np.ascontiguousarray(F, np.float32)
+        assert I.size == self.nelem[side][0] and F.size == self.nelem[side][1]
+        _lib.check(self.l.bfuse_upload(side + 1, I.ctypes.data, F.ctypes.data))
+
+    def zero_outputs(self):
+        _lib.check(self.l.bfuse_zero_output(1))
+        _lib.check(self.l.bfuse_zero_output(2))
+
+    def download(self, side: int) -> np.ndarray:
+        O = np.empty(self.nelem[side][2], np.float32)
+        _lib.check(self.l.bfuse_download(side + 1, O.ctypes.data))
+        return O
+
+    def launch(self, module: int, name: str, grid, block, n_ptrs: int, side: int = 0) -> float:
+        us = C.c_float()
+        _lib.check(self.l.bfuse_module_launch(module, name.encode(), _u3(grid), _u3(block), n_ptrs, side + 1 if n_ptrs == 3 else 0,
+                                              C.byref(us)))
+        return us.value
+
+
 # ---- synthetic inputs ---------------------------------------------------------------------
 def fill_uniform(seed: int, n: int, lo: float, hi: float) -> np.ndarray:
     out = np.empty(n, np.float32)

@@ -187,6 +187,21 @@ int bfuse_time_batched(int mode, const void* func_a, const unsigned* grid_a, con
                        int reps, float* us_per_launch);
 
 /* ------------------------------------------------------------------------------------------
+ * Kernels from a code object: what the horizontal-fuser front end emits (one fused HIP kernel
+ * per fusion, compiled with `hipcc --genco`), or any kernel with the reference's three- /
+ * six-pointer ABI (macro_h.py:182-198).  Launched over the same resident buffers as the
+ * built-in kernels; the caller vouches for the launch shape (it comes from the
+ * {b,h}fuse_kernels.yaml the front end wrote).
+ * ---------------------------------------------------------------------------------------- */
+int bfuse_module_load(const char* code_object_path, int* module_id);
+int bfuse_module_unload(int module_id);
+/* n_ptrs = 3: launch `kernel_name` over side `side` (1 or 2); n_ptrs = 6: over both sides.
+ * Asynchronous on the default stream; if us_out is not NULL the call synchronises and returns
+ * the kernel's GPU-side duration in microseconds. */
+int bfuse_module_launch(int module_id, const char* kernel_name, const unsigned* gridDim, const unsigned* blockDim,
+                        int n_ptrs, int side, float* us_out);
+
+/* ------------------------------------------------------------------------------------------
  * Seeded synthetic inputs (host side): splitmix64 counter stream -> U[lo,hi) or Box-Muller
  * N(mean,std).  Element i depends only on (seed, i).
  * ---------------------------------------------------------------------------------------- */

@@ -1,0 +1,174 @@
+"""Front end (`horizontal-fuser`): command line, YAML outputs and the text it emits.
+
+The command line follows the reference tool (horizontal-fuser/tools/main.cc:38-135:
+`[-b] [-o dir] [-y dir] fusion_config kernel_config [compile_commands_dir]`), the output
+files follow Fuse.cc:120-213 (`<K1>_<K2>_{b,h}fuse.*`, `{b,h}fuse_kernels.yaml`).  The
+prologue the tool prints is C that is also an arithmetic expression language Python can
+evaluate after a token swap, so the emitted index map is executed here, block by block, and
+compared with the library's plan for the same pattern (itself pinned to the oracle and to the
+reference's generated prologues).
+"""
+import os
+import re
+import subprocess
+
+import pytest
+import yaml
+
+from bfuse_project_amd import config, patterns
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+FUSER = os.path.join(ROOT, "bfuse-project_amd", "horizontal-fuser")
+FE = os.path.join(ROOT, "tests", "frontend")
+
+pytestmark = pytest.mark.skipif(not os.path.exists(FUSER), reason="front end not built (python -c 'import __graft_entry__ as g; g.build()')")
+
+
+def run_fuser(tmp_path, *opts, fusions=None, kernels=None, src=None, check=True):
+    out = tmp_path / "out"
+    cmd = [FUSER, *opts, "-o", str(out), "-y", str(out), fusions or os.path.join(FE, "fusions.yaml"),
+           kernels or os.path.join(FE, "kernels.yaml"), src or FE]
+    r = subprocess.run(cmd, capture_output=True, text=True, timeout=60)
+    if check:
+        assert r.returncode == 0, r.stderr
+    return r, out
+
+
+def test_help_and_usage():
+    # fewer than two positional arguments prints the help page (main.cc:114-118)
+    r = subprocess.run([FUSER], capture_output=True, text=True, timeout=60)
+    assert "fusion_config" in r.stdout and "-b" in r.stdout
+    r = subprocess.run([FUSER, "-h", "a", "b"], capture_output=True, text=True, timeout=60)
+    assert "Options:" in r.stdout
+
+
+@pytest.mark.parametrize("bfuse", [True, False])
+def test_outputs_and_yaml_match_fusion_context(tmp_path, bfuse):
+    r, out = run_fuser(tmp_path, *(["-b"] if bfuse else []))
+    kind = "bfuse" if bfuse else "hfuse"
+    kmap = config.load_kernels_yaml(os.path.join(FE, "kernels.yaml"))
+    fusions = config.load_fusions_yaml(os.path.join(FE, "fusions.yaml"))
+    written = config.load_kernels_yaml(str(out / f"{kind}_kernels.yaml"))
+    assert len(written) == len(fusions)
+    for f in fusions:
+        ctx = config.FusionContext.create(f, kmap, bfuse)
+        info = written[ctx.FusedKernelName]
+        assert (info.GridDim, info.BlockDim) == (ctx.FusedGridDim, ctx.FusedBlockDim)
+        assert info.HasBarriers is True and info.Reg == 32  # Fuse.cc:204-209
+        text = (out / ("_".join(f.Kernels) + f"_{kind}.hip")).read_text()
+        assert f'extern "C" __global__ __launch_bounds__({ctx.FusedBlockDim[0]}) void {ctx.FusedKernelName}(' in text
+        assert f"Start to {kind} \"{ctx.FusedKernelName}\"" in r.stdout
+    assert (out / "kernels.hip").exists()
+
+
+def c_to_py(expr):
+    expr = expr.replace("(int)blockIdx.x", "b").replace("&&", " and ").replace("||", " or ")
+    expr = re.sub(r"\bint\(", "(", expr)
+    return expr.replace("/", "//")
+
+
+def eval_prologue(text, bid):
+    """Executes the if / else-if chain of an emitted bfuse kernel for one physical block."""
+    chain = re.findall(r"(?:else )?if \((.*)\)\n  \{\n    NewBlockIdx_ = (.*);\n    KernelID_  = (\d+);", text)
+    assert chain
+    for cond, virt, kid in chain:
+        if eval(c_to_py(cond), {"b": bid}):
+            return int(kid), eval(c_to_py(virt), {"b": bid})
+    return -1, -1
+
+
+@pytest.mark.parametrize("opts,pattern,p0,p1", [
+    ([], "zigzag", 1, 1),
+    (["-M", "2", "-N", "3"], "zigzag", 2, 3),
+    (["-M", "8", "-N", "2"], "zigzag", 8, 2),
+    (["-p", "chunked", "-c", "8"], "chunked", 8, 1),
+    (["-p", "chunked", "-c", "84"], "chunked", 84, 1),
+    (["-p", "proportional", "-c", "1"], "proportional", 1, 1),
+    (["-p", "ranges"], "ranges", 1, 1),
+])
+def test_emitted_prologue_is_the_library_plan(tmp_path, opts, pattern, p0, p1):
+    _, out = run_fuser(tmp_path, "-b", *opts)
+    kmap = config.load_kernels_yaml(os.path.join(FE, "kernels.yaml"))
+    for f in config.load_fusions_yaml(os.path.join(FE, "fusions.yaml")):
+        plan = patterns.plan_blocks(pattern, [kmap[k].dims for k in f.Kernels], p0, p1)
+        text = (out / ("_".join(f.Kernels) + "_bfuse.hip")).read_text()
+        seen = [set(), set()]
+        for bid in range(plan.fused_grid):
+            k, v = eval_prologue(text, bid)
+            assert (k, v) == plan.map(bid), (pattern, bid)
+            if k >= 0:
+                seen[k].add(v)
+        for side, name in enumerate(f.Kernels):
+            g = kmap[name].GridDim
+            assert seen[side] == set(range(g[0] * g[1] * g[2]))
+        assert eval_prologue(text, plan.fused_grid) == (-1, -1)
+
+
+def test_body_rewrite(tmp_path):
+    _, out = run_fuser(tmp_path, "-b")
+    text = (out / "mm_tiled_row_scale_bfuse.hip").read_text()
+    body = text[text.index("switch") if "switch" in text else 0:]
+    # parameters are renamed `<kernel>_<param>_`, builtins become the prologue's variables,
+    # LDS arrays live in one union, and no bare builtin is left in a kernel body
+    assert "mm_tiled_A_[" in text and "row_scale_X_[" in text
+    assert "union" in text and ".mm_tiled.A_shared" in text and ".row_scale.S_shared" in text
+    tail = text[text.index("KernelID_ == 0") if "KernelID_ == 0" in text else text.rindex("else"):]
+    assert not re.search(r"\b(threadIdx|blockDim|gridDim)\s*\.\s*[xyz]\b", tail.replace("(int)threadIdx.x", "T"))
+    assert "__shared__ float A_shared" not in body
+    # hfuse: every __syncthreads() of a side becomes that side's barrier
+    _, outh = run_fuser(tmp_path, )
+    th = (outh / "mm_tiled_row_scale_hfuse.hip").read_text()
+    assert th.count("__syncthreads()") == 1          # the one that publishes the zeroed counters
+    assert th.count("bfuse_side_barrier(&bfuse_arrive_[0], 4u") == 2
+    assert th.count("bfuse_side_barrier(&bfuse_arrive_[1], 2u") == 1
+
+
+def test_hfuse_ranges(tmp_path):
+    _, out = run_fuser(tmp_path)
+    text = (out / "mm_tiled_ew_max_hfuse.hip").read_text()
+    # 256 threads, then 152 padded to the next wavefront: [0,256) and [256,408), block 448
+    assert "threadIdx.x >= 0 && (int)threadIdx.x < 256" in text
+    assert "threadIdx.x >= 256 && (int)threadIdx.x < 408" in text
+    r, out32 = run_fuser(tmp_path, "-w", "32")
+    assert "warning" in r.stderr
+    info = config.load_kernels_yaml(str(out32 / "hfuse_kernels.yaml"))["mm_tiled_ew_max_fused_hfuse"]
+    assert info.BlockDim == (416, 1, 1)               # the reference's 32-thread padding: 256 + 160
+
+
+def test_errors(tmp_path):
+    bad = tmp_path / "bad_fusions.yaml"
+    bad.write_text("- File: kernels.cu\n  Kernels:\n  - mm_tiled\n  - nope\n")
+    r, _ = run_fuser(tmp_path, "-b", fusions=str(bad), check=False)
+    assert r.returncode != 0 and "nope" in r.stderr
+    bad.write_text("- File: missing.cu\n  Kernels:\n  - mm_tiled\n  - ew_max\n")
+    r, _ = run_fuser(tmp_path, "-b", fusions=str(bad), check=False)
+    assert r.returncode != 0 and "missing.cu" in r.stderr
+    r, _ = run_fuser(tmp_path, "-b", "-p", "spiral", check=False)
+    assert r.returncode != 0 and "spiral" in r.stderr
+    src = tmp_path / "src"
+    src.mkdir()
+    (src / "kernels.cu").write_text('extern "C" __global__ void mm_tiled(float* A);\n')
+    r, _ = run_fuser(tmp_path, "-b", src=str(src), check=False)
+    assert r.returncode != 0 and "mm_tiled" in r.stderr
+
+
+def test_reference_style_source(tmp_path):
+    """A kernel in the shape TVM prints for the reference (attribute after the return type,
+    `__shared__` arrays, casts around every builtin) goes through unchanged in meaning."""
+    src = tmp_path / "src"
+    src.mkdir()
+    (src / "k.cu").write_text(
+        'extern "C" __global__ void __launch_bounds__(64) a0(float* __restrict__ p, float* __restrict__ q, float* __restrict__ r) {\n'
+        "  __shared__ float buf[64];\n  buf[((int)threadIdx.x)] = p[((int)blockIdx.x) * 64 + ((int)threadIdx.x)];\n  __syncthreads();\n"
+        "  r[((int)blockIdx.x) * 64 + ((int)threadIdx.x)] = buf[63 - ((int)threadIdx.x)] + q[0];\n}\n"
+        'extern "C" __global__ void __launch_bounds__(128) a1(float* __restrict__ p, float* __restrict__ q, float* __restrict__ r) {\n'
+        "  r[((int)blockIdx.x) * 128 + ((int)threadIdx.x)] = p[((int)blockIdx.x) * 128 + ((int)threadIdx.x)] * q[0];\n}\n")
+    k = {n: {"KernelName": n, "HasBarriers": n == "a0", "GridDim": {"X": g, "Y": 1, "Z": 1},
+             "BlockDim": {"X": b, "Y": 1, "Z": 1}, "Reg": 32, "ExecTime": -1} for n, g, b in (("a0", 10, 64), ("a1", 7, 128))}
+    (tmp_path / "k.yaml").write_text(yaml.safe_dump(k))
+    (tmp_path / "f.yaml").write_text(yaml.safe_dump([{"File": "k.cu", "Kernels": ["a0", "a1"]}]))
+    _, out = run_fuser(tmp_path, "-b", fusions=str(tmp_path / "f.yaml"), kernels=str(tmp_path / "k.yaml"), src=str(src))
+    info = config.load_kernels_yaml(str(out / "bfuse_kernels.yaml"))["a0_a1_fused_bfuse"]
+    assert info.GridDim == (17, 1, 1) and info.BlockDim == (128, 1, 1)
+    unf = (out / "kernels.hip").read_text()
+    assert '__launch_bounds__(64) void a0(' in unf and '__launch_bounds__(128) void a1(' in unf

@@ -34,7 +34,8 @@ def test_pair_fused_bit_exact_and_close_to_cpu(number):
     pair = PAIRS[number]
     _say(f"[pair {number}] {pair.title}")
     I1, F1, I2, F2 = pair.inputs()
-    first = None
+    _say(f"[pair {number}] CPU oracle")
+    E1, E2 = oracle_cases.expected(number, I1, F1, I2, F2)
     for (k1, k2), variants in fusions(pair).items():
         with bf.Operation(k1, k2) as op:
             _say(f"[pair {number}] run_kernel1 {k1}")
@@ -52,25 +53,17 @@ def test_pair_fused_bit_exact_and_close_to_cpu(number):
                 Q1, Q2 = op.run_fuse(fused, I1, F1, I2, F2)
                 assert np.array_equal(Q1.view(np.uint8), O1.view(np.uint8)), f"{fused.name}: side 1 differs from unfused"
                 assert np.array_equal(Q2.view(np.uint8), O2.view(np.uint8)), f"{fused.name}: side 2 differs from unfused"
-        if first is None:
-            first = (O1, O2)
+        # every built implementation of a side (other tilings sum in another order, so they are
+        # not bit-equal to each other) is held to the CPU reference on its own
+        R1, X1 = (E1.pick(O1), E1.values) if isinstance(E1, oracle_cases.Sampled) else (O1, E1)
+        if pair.dtype == "bf16":
+            R1, R2, X1, X2 = (bf.operation.bf16_to_f32(x) for x in (R1, O2, X1, E2))
         else:
-            # other launch shapes of the same operator compute the same values
-            assert np.array_equal(O1.view(np.uint8), first[0].view(np.uint8)), f"{k1} differs from {pair.k1}"
-            assert np.array_equal(O2.view(np.uint8), first[1].view(np.uint8)), f"{k2} differs from {pair.k2}"
-    O1, O2 = first
-    _say(f"[pair {number}] CPU oracle")
-    E1, E2 = oracle_cases.expected(number, I1, F1, I2, F2)
-    if isinstance(E1, oracle_cases.Sampled):
-        O1, E1 = E1.pick(O1), E1.values
-    if pair.dtype == "bf16":
-        O1f, O2f, E1, E2 = (bf.operation.bf16_to_f32(x) for x in (O1, O2, E1, E2))
-    else:
-        O1f, O2f = O1, O2
-    e1 = oracle_cases.rel_error(O1f.ravel(), E1.ravel())
-    e2 = oracle_cases.rel_error(O2f.ravel(), E2.ravel())
-    _say(f"[pair {number}] max rel err side1 {e1:.3e} side2 {e2:.3e} (tol {pair.tol:g})")
-    assert e1 <= pair.tol and e2 <= pair.tol
+            R2, X2 = O2, E2
+        e1 = oracle_cases.rel_error(R1.ravel(), X1.ravel())
+        e2 = oracle_cases.rel_error(R2.ravel(), X2.ravel())
+        _say(f"[pair {number}] {k1} | {k2}: max rel err side1 {e1:.3e} side2 {e2:.3e} (tol {pair.tol:g})")
+        assert e1 <= pair.tol and e2 <= pair.tol, (k1, k2)
 
 
 def test_device_block_map_equals_host_and_oracle():
