@@ -593,7 +593,6 @@ string emit_hfuse(const vector<Kernel>& ks, const vector<KernelInfo>& infos, con
         o << "      (void)blockIdx_x_; (void)blockIdx_y_; (void)blockIdx_z_; (void)threadIdx_x_; (void)threadIdx_y_; (void)threadIdx_z_;\n";
         o << "      (void)gridDim_x_; (void)gridDim_y_; (void)gridDim_z_; (void)blockDim_x_; (void)blockDim_y_; (void)blockDim_z_;\n";
         o << "      unsigned int bfuse_epoch_ = 0u; (void)bfuse_epoch_;\n";
-        for (auto& d : ks[i].shared) o << "      __shared__ " << d.type << " " << d.name << d.extent << ";\n";
         o << indent_block(body, "    ") << "  }\n";
     }
     o << "}\n";
@@ -689,7 +688,9 @@ int main(int argc, char** argv)
                 u << ")\n{" << k.body << "}\n";
                 unfused[kn] = u.str();
             }
-            hoist_shared(k);
+            // block fusion overlays the LDS arrays of the sides in one union; thread fusion leaves
+            // every `__shared__` declaration where it is, so the sides' LDS adds up (Matchers.cc:322-412)
+            if (opt.bfuse) hoist_shared(k);
             for (auto& p : k.params) k.body = replace_ident(k.body, p.name, kn + "_" + p.name + "_");
             k.body = rewrite_builtins(k.body);
             ks.push_back(k);

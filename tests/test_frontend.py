@@ -107,16 +107,18 @@ def test_emitted_prologue_is_the_library_plan(tmp_path, opts, pattern, p0, p1):
 def test_body_rewrite(tmp_path):
     _, out = run_fuser(tmp_path, "-b")
     text = (out / "mm_tiled_row_scale_bfuse.hip").read_text()
-    body = text[text.index("switch") if "switch" in text else 0:]
+    bodies = text[text.index("__shared__ ShrdUnionTy_ SU_;"):]
     # parameters are renamed `<kernel>_<param>_`, builtins become the prologue's variables,
-    # LDS arrays live in one union, and no bare builtin is left in a kernel body
-    assert "mm_tiled_A_[" in text and "row_scale_X_[" in text
-    assert "union" in text and ".mm_tiled.A_shared" in text and ".row_scale.S_shared" in text
-    tail = text[text.index("KernelID_ == 0") if "KernelID_ == 0" in text else text.rindex("else"):]
-    assert not re.search(r"\b(threadIdx|blockDim|gridDim)\s*\.\s*[xyz]\b", tail.replace("(int)threadIdx.x", "T"))
-    assert "__shared__ float A_shared" not in body
+    # LDS arrays live in one union (Tools.cc:219-251), and the only builtin left in the two
+    # bodies is the physical thread index of the branch guards
+    assert "mm_tiled_A_[" in bodies and "row_scale_X_[" in bodies
+    assert "SU_.mm_tiled.A_shared[" in bodies and "SU_.row_scale.S_shared[" in bodies
+    assert "__shared__ float" not in bodies
+    assert not re.search(r"\b(blockIdx|blockDim|gridDim)\s*\.", bodies)
+    assert set(re.findall(r"threadIdx\.x < (\d+)", bodies)) == {"256", "128"}
+    assert len(re.findall(r"threadIdx\s*\.", bodies)) == 2
     # hfuse: every __syncthreads() of a side becomes that side's barrier
-    _, outh = run_fuser(tmp_path, )
+    _, outh = run_fuser(tmp_path)
     th = (outh / "mm_tiled_row_scale_hfuse.hip").read_text()
     assert th.count("__syncthreads()") == 1          # the one that publishes the zeroed counters
     assert th.count("bfuse_side_barrier(&bfuse_arrive_[0], 4u") == 2
@@ -172,3 +174,64 @@ def test_reference_style_source(tmp_path):
     assert info.GridDim == (17, 1, 1) and info.BlockDim == (128, 1, 1)
     unf = (out / "kernels.hip").read_text()
     assert '__launch_bounds__(64) void a0(' in unf and '__launch_bounds__(128) void a1(' in unf
+
+
+# ---- against what the reference's own fuser emitted ------------------------------------------
+GOLDEN = os.path.join(ROOT, "tests", "golden")
+
+
+def _suite(tmp_path, grids, blocks):
+    """A two-kernel suite with the golden's launch shapes and empty bodies."""
+    src = tmp_path / "src"
+    src.mkdir(exist_ok=True)
+    (src / "k.cu").write_text("".join(
+        f'extern "C" __global__ void __launch_bounds__({b[0] * b[1] * b[2]}) k{i}(float* __restrict__ a, float* __restrict__ b, float* __restrict__ c) {{\n}}\n'
+        for i, b in enumerate(blocks)))
+    ky = {f"k{i}": {"KernelName": f"k{i}", "HasBarriers": True, "GridDim": dict(zip("XYZ", g)),
+                    "BlockDim": dict(zip("XYZ", b)), "Reg": 32, "ExecTime": -1} for i, (g, b) in enumerate(zip(grids, blocks))}
+    (tmp_path / "k.yaml").write_text(yaml.safe_dump(ky))
+    (tmp_path / "f.yaml").write_text(yaml.safe_dump([{"File": "k.cu", "Kernels": sorted(ky)}]))
+    return dict(fusions=str(tmp_path / "f.yaml"), kernels=str(tmp_path / "k.yaml"), src=str(src))
+
+
+def test_emitted_prologue_matches_reference_outputs(tmp_path):
+    """bfuse_maps.json holds, for 90 kernels the reference's fuser emitted (1:1 zig-zag, M and
+    N ratio sweeps, the 84-SM chunk pattern), what their dispatch chains evaluate to at sampled
+    block ids.  The chain this front end prints for the same launch shapes and options must
+    evaluate to the same (kernel, virtual block) at every sample."""
+    import json
+    entries = json.load(open(os.path.join(GOLDEN, "bfuse_maps.json")))
+    assert len(entries) >= 90
+    for n, e in enumerate(entries):
+        case = tmp_path / f"c{n}"
+        case.mkdir()
+        if e["pattern"] == "zigzag":
+            opts = ["-M", str(e["params"]["M"]), "-N", str(e["params"]["N"])]
+        else:
+            opts = ["-p", "chunked", "-c", str(e["params"]["TotalSM"])]
+        _, out = run_fuser(case, "-b", *opts, **_suite(case, e["grids"], e["blocks"]))
+        info = config.load_kernels_yaml(str(out / "bfuse_kernels.yaml"))["k0_k1_fused_bfuse"]
+        assert info.GridDim == (e["fused_grid"], 1, 1) and info.BlockDim == (e["fused_block"], 1, 1), e["source"]
+        text = (out / "k0_k1_bfuse.hip").read_text()
+        for bid, kid, virt in e["samples"]:
+            assert eval_prologue(text, bid) == (kid, virt), (e["source"], bid)
+
+
+def test_emitted_hfuse_guards_match_reference_outputs(tmp_path):
+    """hfuse_ranges.json: thread ranges, block bounds and fused block sizes of kernels the
+    reference's fuser emitted (32-thread padding, Algorithms.cc:23-35), reproduced with -w 32."""
+    import json
+    entries = json.load(open(os.path.join(GOLDEN, "hfuse_ranges.json")))
+    for n, e in enumerate(entries):
+        case = tmp_path / f"h{n}"
+        case.mkdir()
+        # the fixture stores the remap divisors (x, y, x*y) of each side; z follows from the totals
+        grids = [[s["grid_xy"][0], s["grid_xy"][1], s["blocks"] // s["grid_xy"][2]] for s in e["sides"]]
+        blocks = [[s["block_xy"][0], s["block_xy"][1], (s["thr_hi"] - s["thr_lo"]) // s["block_xy"][2]] for s in e["sides"]]
+        _, out = run_fuser(case, "-w", "32", **_suite(case, grids, blocks))
+        info = config.load_kernels_yaml(str(out / "hfuse_kernels.yaml"))["k0_k1_fused_hfuse"]
+        assert info.BlockDim == (e["fused_block"], 1, 1), e["source"]
+        assert info.GridDim == (max(s["blocks"] for s in e["sides"]), 1, 1)
+        text = (out / "k0_k1_hfuse.hip").read_text()
+        guards = re.findall(r"threadIdx\.x >= (\d+) && \(int\)threadIdx\.x < (\d+)\) && \(\(int\)blockIdx\.x >= 0 && \(int\)blockIdx\.x < (\d+)\)", text)
+        assert [(int(a), int(b), int(c)) for a, b, c in guards] == [(s["thr_lo"], s["thr_hi"], s["blocks"]) for s in e["sides"]], e["source"]
