@@ -6,6 +6,7 @@
 #include "fuse.h"
 #include "ops_conv.h"
 #include "ops_gemm_bf16.h"
+#include "ops_gemm_bf16_ring.h"
 #include "ops_gemm_f32.h"
 #include "ops_gemm_f32_lds.h"
 #include "ops_rowwise.h"
@@ -28,6 +29,9 @@ using PoolS = MaxPool3x3S2<4, 16, 16, 64>;
 using GemmB1 = GemmBf16NT<128, 1792, 64, 128, 224>;                   // one K-step
 using GemmB2 = GemmBf16NT<256, 1792, 192, 128, 224>;                  // two M-tiles, three K-steps
 using GemmB3 = GemmBf16NTDma<256, 1792, 320, 128, 224, 3>;             // direct-to-LDS ring, five K-steps
+using GemmB5 = GemmBf16NTDma<256, 1792, 320, 128, 224, 3, 4, 4, 2>;       // the same with eight waves (uneven load groups per wave)
+using GemmB6 = GemmBf16NTRing<256, 1792, 320, 128, 224, 7, 4, 2>;         // ring of seven 32-k stages, ten K-steps, eight waves
+using GemmB7 = GemmBf16NTRing<256, 1792, 320, 128, 224, 4, 2, 2>;         // ring of four, four waves (four A fragments per wave)
 using GemmB4 = GemmBf16NTDma<128, 1792, 192, 128, 224, 2>;             // two stages, three K-steps
 using NormRopeS = RmsNormRope<6, 8, 128, 2>;
 
@@ -45,6 +49,9 @@ BFUSE_KERNEL(maxpool3x3s2_f32_4x16x16, PoolS, ({{1, 4, 16, 16}, 4}), ({{1, 1, 1,
 BFUSE_KERNEL(gemm_bf16_128x64x1792, GemmB1, ({{128, 64, 1, 1}, 2}), ({{1792, 64, 1, 1}, 2}), ({{128, 1792, 1, 1}, 2}))
 BFUSE_KERNEL(gemm_bf16_256x192x1792, GemmB2, ({{256, 192, 1, 1}, 2}), ({{1792, 192, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
 BFUSE_KERNEL(gemm_bf16_256x320x1792_d, GemmB3, ({{256, 320, 1, 1}, 2}), ({{1792, 320, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
+BFUSE_KERNEL(gemm_bf16_256x320x1792_w8, GemmB5, ({{256, 320, 1, 1}, 2}), ({{1792, 320, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
+BFUSE_KERNEL(gemm_bf16_256x320x1792_r, GemmB6, ({{256, 320, 1, 1}, 2}), ({{1792, 320, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
+BFUSE_KERNEL(gemm_bf16_256x320x1792_r4, GemmB7, ({{256, 320, 1, 1}, 2}), ({{1792, 320, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
 BFUSE_KERNEL(gemm_bf16_128x192x1792_d4, GemmB4, ({{128, 192, 1, 1}, 2}), ({{1792, 192, 1, 1}, 2}), ({{128, 1792, 1, 1}, 2}))
 BFUSE_KERNEL(rmsnorm_rope_bf16_6x1024, NormRopeS, ({{6, 1024, 1, 1}, 2}), ({{(int)NormRopeS::F_BYTES, 1, 1, 1}, 1}), ({{6, 1024, 1, 1}, 2}))
 
@@ -66,3 +73,4 @@ BFUSE_HFUSE_KERNEL(maxpool3x3s2_f32_4x16x16, PoolS, layernorm_8x256, LayerNormS)
 // the direct-to-LDS GEMM under horizontal fusion: its fence-free barrier becomes the LDS-counter one
 BFUSE_HFUSE_KERNEL(gemm_bf16_256x320x1792_d, GemmB3, rmsnorm_rope_bf16_6x1024, NormRopeS)
 BFUSE_HFUSE_KERNEL(gemm_f32_128x160x192_l, GemmS4, bias_relu_4096, BiasReluS)
+BFUSE_HFUSE_KERNEL(gemm_bf16_256x320x1792_r, GemmB6, rmsnorm_rope_bf16_6x1024, NormRopeS)

@@ -168,22 +168,32 @@ struct GemmBf16NT {
 // 16 bytes contiguously (8 rows of 128 bytes), so rows cannot be padded; instead the
 // 16-byte chunk c of row r is stored at chunk position c ^ ((r >> 1) & 7), which makes the
 // 128-bit operand reads of 16 consecutive rows hit 16 different bank groups.
-template <int M_, int N_, int K_, int BM_, int BN_, int NSTG_ = 3, int PD_ = 4>
+//
+// Waves: WGM_ x WGN_ of them tile the workgroup's BM x BN block.  One wave per SIMD (2 x 2)
+// cannot keep the matrix core busy with 16x16x32 MFMAs: measured on MI355X, a lone wave
+// issues one every ~28 clocks where the pipe takes 16, and two waves per SIMD reach ~18.
+// The 4 x 2 layout (eight waves of 32 x BN/2) therefore trades 40 % more LDS operand reads
+// (still under 60 % of the ~250 B/clk the LDS delivers to eight waves) for a 1.5x higher
+// MFMA issue ceiling.
+template <int M_, int N_, int K_, int BM_, int BN_, int NSTG_ = 3, int PD_ = 4, int WGM_ = 2, int WGN_ = 2>
 struct GemmBf16NTDma {
     static constexpr int M = M_, N = N_, K = K_, BM = BM_, BN = BN_, NSTG = NSTG_;
     static constexpr int BK = 64;
-    static constexpr int THREADS = 256;
-    static constexpr int WM = BM / 2, WN = BN / 2;
+    static constexpr int WGM = WGM_, WGN = WGN_, NWAVES = WGM_ * WGN_;
+    static constexpr int THREADS = 64 * NWAVES;
+    static constexpr int WM = BM / WGM, WN = BN / WGN;
     static constexpr int TM = WM / 16, TN = WN / 16;
     static constexpr int NKT = K / BK;
     static constexpr int ROWS = BM + BN;
     static constexpr int GROUPS = ROWS / 8;             // wave-level loads per stage
-    static constexpr int GPW = GROUPS / 4;              // per wave
+    static constexpr int GPW = (GROUPS + NWAVES - 1) / NWAVES;   // per wave: waves < GEXTRA issue GPW, the others GPW - 1
+    static constexpr int GEXTRA = GROUPS % NWAVES == 0 ? NWAVES : GROUPS % NWAVES;
     static constexpr int STAGE_BYTES = ROWS * 128;
     static constexpr int CPITCH = BN + 8;
     static constexpr int OCHUNKS = BM * (BN / 8);
     static_assert(M % BM == 0 && N % BN == 0 && K % BK == 0, "tile must divide the problem");
-    static_assert(WM % 16 == 0 && WN % 16 == 0 && BM % 8 == 0 && GROUPS % 4 == 0, "tile shape");
+    static_assert(BM % WGM == 0 && BN % WGN == 0 && WM % 16 == 0 && WN % 16 == 0 && BM % 8 == 0 && BN % 8 == 0, "tile shape");
+    static_assert(TM == 2 || TM == 4, "the hand-written LDS wait lists two or four A fragments");
     static_assert(OCHUNKS % THREADS == 0 && NSTG >= 2 && NSTG <= 4 && NKT >= NSTG - 1, "pipeline shape");
     static_assert(PD_ >= 1 && PD_ < (BK / 32) * (BN / 32), "read-ahead distance");
     static constexpr int MT = M / BM, NT = N / BN;
@@ -206,14 +216,27 @@ struct GemmBf16NTDma {
 
     typedef __attribute__((address_space(3))) unsigned char lds_u8;
 
-    // this wave's GPW wave-level loads of K-step kt into LDS stage `stage`
-    __device__ static __forceinline__ void issue(const unsigned short* const (&src)[GPW], lds_u8* wave_base, int stage, int kt)
+    // this wave's wave-level loads of K-step kt into LDS stage `stage`: group wave + i * NWAVES
+    // (8 rows each); `full` says whether this wave owns a group in the last, partial round
+    __device__ static __forceinline__ void issue(const unsigned short* const (&src)[GPW], lds_u8* wave_base, int stage, int kt, bool full)
     {
 #if defined(__HIP_DEVICE_COMPILE__)
 #pragma unroll
         for (int i = 0; i < GPW; ++i)
-            __builtin_amdgcn_global_load_lds(src[i] + kt * BK, wave_base + stage * STAGE_BYTES + i * 1024, 16, 0, 0);
+            if (i + 1 < GPW || full)
+                __builtin_amdgcn_global_load_lds(src[i] + kt * BK, wave_base + stage * STAGE_BYTES + i * NWAVES * 1024, 16, 0, 0);
 #endif
+    }
+    // "the loads of the K-step that is due have landed": at most `newer` K-steps' loads outstanding
+    template <int NEWER>
+    __device__ static __forceinline__ void wait_stage(bool full)
+    {
+        if constexpr (GEXTRA == NWAVES) {
+            wait_vm<GPW * NEWER>();
+        } else {
+            if (full) wait_vm<GPW * NEWER>();
+            else wait_vm<(GPW - 1) * NEWER>();
+        }
     }
 
     // ---- operand reads are issued and waited for by hand ------------------------------------
@@ -240,8 +263,11 @@ struct GemmBf16NTDma {
     __device__ static __forceinline__ void wait_lds(bf16x8& b, bf16x8 (&a)[TM])
     {
 #if defined(__HIP_DEVICE_COMPILE__)
-        static_assert(TM == 4, "the dependency list below names four A fragments");
-        asm volatile("s_waitcnt lgkmcnt(%5)" : "+v"(b), "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]) : "n"(N_OUT));
+        if constexpr (TM == 4) {
+            asm volatile("s_waitcnt lgkmcnt(%5)" : "+v"(b), "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]) : "n"(N_OUT));
+        } else {
+            asm volatile("s_waitcnt lgkmcnt(%3)" : "+v"(b), "+v"(a[0]), "+v"(a[1]) : "n"(N_OUT));
+        }
 #endif
     }
 
@@ -286,14 +312,14 @@ struct GemmBf16NTDma {
     template <int U, class Sync>
     __device__ static __forceinline__ void k_step(int kt, f32x4 (&acc)[TM][TN], const int (&a_ad)[BK / 32][TM],
                                                   const int (&b_ad)[BK / 32][TN], const unsigned short* const (&src)[GPW],
-                                                  lds_u8* lds, Sync& sync)
+                                                  lds_u8* lds, bool full, Sync& sync)
     {
         if (kt >= NKT) return;
         // loads of K-step kt have landed once at most the newer steps' loads are outstanding
-        if (kt + NSTG - 2 < NKT) wait_vm<GPW * (NSTG - 2)>();
+        if (kt + NSTG - 2 < NKT) wait_stage<NSTG - 2>(full);
         else wait_vm<0>();
         sync.raw();  // everyone's part of step kt is in LDS; everyone is done reading step kt-1
-        if (kt + NSTG - 1 < NKT) issue(src, lds, (U + NSTG - 1) % NSTG, kt + NSTG - 1);
+        if (kt + NSTG - 1 < NKT) issue(src, lds, (U + NSTG - 1) % NSTG, kt + NSTG - 1, full);
         constexpr int OFF = U * STAGE_BYTES;
         bf16x8 af[BK / 32][TM], bq[RING];
 #pragma unroll
@@ -315,18 +341,20 @@ struct GemmBf16NTDma {
         const int nt = xcd * (NT / 8) + slot / MT, mt = slot % MT;
         const int m0 = mt * BM, n0 = nt * BN;
         const int wave = tid >> 6, lane = tid & 63;
-        const int wm = wave >> 1, wn = wave & 1;
+        const int wm = wave / WGN, wn = wave % WGN;
         const int li = lane & 15, kq = lane >> 4;
+        const bool full = wave < GEXTRA;
 
-        // per-lane source of each of this wave's GPW loads (K-step 0); swizzled chunk
+        // per-lane source of each of this wave's loads (K-step 0); swizzled chunk
         const unsigned short* src[GPW];
 #pragma unroll
         for (int i = 0; i < GPW; ++i) {
-            const int row = 8 * (wave * GPW + i) + (lane >> 3);
+            int row = 8 * (wave + i * NWAVES) + (lane >> 3);
+            if (row >= ROWS) row = ROWS - 1;  // slot not issued (see `full`)
             const int gc = (lane & 7) ^ ((row >> 1) & 7);
             src[i] = (row < BM ? A + (size_t)(m0 + row) * K : Wt + (size_t)(n0 + row - BM) * K) + gc * 8;
         }
-        lds_u8* const lds = (lds_u8*)sm.t + wave * GPW * 1024;
+        lds_u8* const lds = (lds_u8*)sm.t + wave * 1024;
 
         f32x4 acc[TM][TN];
 #pragma unroll
@@ -335,7 +363,7 @@ struct GemmBf16NTDma {
             for (int b = 0; b < TN; ++b) acc[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
 
 #pragma unroll
-        for (int s = 0; s < NSTG - 1; ++s) issue(src, lds, s, s);
+        for (int s = 0; s < NSTG - 1; ++s) issue(src, lds, s, s, full);
 
         // byte offset inside a stage of every operand fragment this lane reads (K-substep ks,
         // block a / b), with the chunk swizzle folded in: loop invariant
@@ -367,10 +395,10 @@ struct GemmBf16NTDma {
 
         // K-steps are taken NSTG at a time so that the LDS stage of each is a compile-time constant
         for (int kt0 = 0; kt0 < NKT; kt0 += NSTG) {
-            k_step<0>(kt0, acc, a_ad, b_ad, src, lds, sync);
-            if constexpr (NSTG > 1) k_step<1>(kt0 + 1, acc, a_ad, b_ad, src, lds, sync);
-            if constexpr (NSTG > 2) k_step<2>(kt0 + 2, acc, a_ad, b_ad, src, lds, sync);
-            if constexpr (NSTG > 3) k_step<3>(kt0 + 3, acc, a_ad, b_ad, src, lds, sync);
+            k_step<0>(kt0, acc, a_ad, b_ad, src, lds, full, sync);
+            if constexpr (NSTG > 1) k_step<1>(kt0 + 1, acc, a_ad, b_ad, src, lds, full, sync);
+            if constexpr (NSTG > 2) k_step<2>(kt0 + 2, acc, a_ad, b_ad, src, lds, full, sync);
+            if constexpr (NSTG > 3) k_step<3>(kt0 + 3, acc, a_ad, b_ad, src, lds, full, sync);
         }
         sync();  // all waves are done reading the last stage before the tile buffer overwrites it
 

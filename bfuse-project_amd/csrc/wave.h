@@ -61,6 +61,15 @@ struct BlockSync {
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
     }
+    // The instruction alone: nothing of this wave is drained.  For kernels that keep LDS reads
+    // in flight across the barrier and count them by hand; the caller guarantees that whatever
+    // another wave may overwrite after the barrier has already been consumed by this one.
+    __device__ __forceinline__ void bare() const
+    {
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    }
 };
 
 // Barrier over the waves of ONE side of a horizontally fused workgroup.  gfx950 has no
@@ -97,6 +106,8 @@ struct GroupSync {
     // Same meeting point without fences (see BlockSync::raw): the caller has already waited
     // for the loads the other waves depend on; LDS operations of one wave execute in order,
     // so reads issued after the poll see what the other waves wrote before they arrived.
+    // the counter barrier uses LDS operations itself, so it cannot leave the caller's in flight
+    __device__ __forceinline__ void bare() { raw(); }
     __device__ __forceinline__ void raw()
     {
         ++epoch;

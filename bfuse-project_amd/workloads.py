@@ -145,7 +145,10 @@ PAIRS: Dict[int, Pair] = {
             "gemm_bf16_512x4096x14336", "rmsnorm_rope_bf16_512x4096", "bfuse",
             [("bfuse", ""), ("bfuse", "_c256")],
             [("gemm_bf16_512x4096x14336", "rmsnorm_rope_bf16_512x4096_w4", "bfuse", "_c256"),
-             ("gemm_bf16_512x4096x14336_v", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256")], _pair5_inputs,
+             ("gemm_bf16_512x4096x14336_v", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
+             ("gemm_bf16_512x4096x14336_w8", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
+             ("gemm_bf16_512x4096x14336_r", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
+             ("gemm_bf16_512x4096x14336_w8", "rmsnorm_rope_bf16_512x4096_w2", "hfuse", "")], _pair5_inputs,
             bytes1=(512 * 4096 + 4096 * 14336 + 512 * 14336) * 2, bytes2=2 * 512 * 4096 * 2 + 4096 * 2,
             flops=2 * 512 * 4096 * 14336, bound="mfma", peak=2500.0, dtype="bf16", tol=1e-2),
 }
@@ -166,7 +169,7 @@ HEADLINE = {
     2: ("gemm_f32_512x768x2304", "layernorm_512x768_w1", "bfuse", "_r"),
     3: ("conv3x3_f32_64x56x56_64", "maxpool3x3s2_f32_64x112x112", "bfuse", "_c256"),
     4: ("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072_l", "bfuse", "_c256"),
-    5: ("gemm_bf16_512x4096x14336", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
+    5: ("gemm_bf16_512x4096x14336_w8", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
 }
 
 
@@ -177,6 +180,6 @@ MEASURED_TRAFFIC = {
     "gemm_f32_512x512x512_bias_relu_1048576_fused_hfuse": 23_190_000,
     "gemm_f32_512x768x2304_layernorm_512x768_w1_fused_bfuse_r": 28_460_000,
     "conv3x3_f32_64x56x56_64_maxpool3x3s2_f32_64x112x112_fused_bfuse_c256": 11_060_000,
-    "softmax_causal_12x512x512_r3_gemm_gelu_f32_512x768x3072_h_fused_hfuse": 48_150_000,
+    "softmax_causal_12x512x512_gemm_gelu_f32_512x768x3072_l_fused_bfuse_c256": 47_740_000,
     "gemm_bf16_512x4096x14336_rmsnorm_rope_bf16_512x4096_fused_bfuse_c256": 174_890_000,
 }

@@ -61,6 +61,12 @@ def _cases():
                                    lambda I, F: orf.gemm_bf16(I.reshape(256, 192), F.reshape(1792, 192), b_is_nk=True), 1e-2, True),
         "gemm_bf16_256x320x1792_d": (lambda s: (f32_to_bf16(fill_normal(s, 256 * 320, 0, 1)), f32_to_bf16(fill_normal(s + 1, 1792 * 320, 0, 0.1))),
                                      lambda I, F: orf.gemm_bf16(I.reshape(256, 320), F.reshape(1792, 320), b_is_nk=True), 1e-2, True),
+        "gemm_bf16_256x320x1792_w8": (lambda s: (f32_to_bf16(fill_normal(s, 256 * 320, 0, 1)), f32_to_bf16(fill_normal(s + 1, 1792 * 320, 0, 0.1))),
+                                      lambda I, F: orf.gemm_bf16(I.reshape(256, 320), F.reshape(1792, 320), b_is_nk=True), 1e-2, True),
+        "gemm_bf16_256x320x1792_r": (lambda s: (f32_to_bf16(fill_normal(s, 256 * 320, 0, 1)), f32_to_bf16(fill_normal(s + 1, 1792 * 320, 0, 0.1))),
+                                     lambda I, F: orf.gemm_bf16(I.reshape(256, 320), F.reshape(1792, 320), b_is_nk=True), 1e-2, True),
+        "gemm_bf16_256x320x1792_r4": (lambda s: (f32_to_bf16(fill_normal(s, 256 * 320, 0, 1)), f32_to_bf16(fill_normal(s + 1, 1792 * 320, 0, 0.1))),
+                                      lambda I, F: orf.gemm_bf16(I.reshape(256, 320), F.reshape(1792, 320), b_is_nk=True), 1e-2, True),
         "gemm_bf16_128x192x1792_d4": (lambda s: (f32_to_bf16(fill_normal(s, 128 * 192, 0, 1)), f32_to_bf16(fill_normal(s + 1, 1792 * 192, 0, 0.1))),
                                       lambda I, F: orf.gemm_bf16(I.reshape(128, 192), F.reshape(1792, 192), b_is_nk=True), 1e-2, True),
         "rmsnorm_rope_bf16_6x1024": (lambda s: (f32_to_bf16(fill_normal(s, 6 * 1024, 0, 1.5)), _norm_rope_operand(6, 1024, 128, s + 1)),
@@ -79,6 +85,7 @@ FUSIONS = [
     ("maxpool3x3s2_f32_4x16x16", "layernorm_8x256", "hfuse", ""),
     ("gemm_f32_128x160x192_l", "bias_relu_4096", "hfuse", ""),
     ("gemm_bf16_256x320x1792_d", "rmsnorm_rope_bf16_6x1024", "hfuse", ""),
+    ("gemm_bf16_256x320x1792_r", "rmsnorm_rope_bf16_6x1024", "hfuse", ""),
 ]
 
 
