@@ -5,6 +5,13 @@
 //            virtual block through a compile-time BlockPlan; LDS is a union of both sides
 //            (the reference's emitted form: horizontal-fuser/src/Matchers.cc:523-602,
 //            union layout Tools.cc:219-251)
+//   bfuse_rt : block fusion whose BlockPlan is DATA (set by the host before the launch) and
+//            whose workgroups are persistent: workgroup w handles fused block ids w, w + gridDim.x,
+//            ...  Launched with gridDim.x = the plan's fused grid it is plain block fusion with
+//            a run-time pattern (what the reference's legacy ratio sweep re-generated and
+//            re-compiled for every M:N, legacy/tests/single_bgemm_conv2d/auto.py:9-14); launched
+//            with a few workgroups per CU it is the persistent-block form of
+//            legacy/tests/thread_pooling_test/temp.cu:576-612
 //   hfuse  : horizontal fusion -- one workgroup hosts both operators on disjoint wave
 //            ranges; LDS is the sum of both sides; an intra-side barrier is the LDS-counter
 //            GroupSync instead of CUDA's bar.sync id,count (Matchers.cc:288-320, 655-727)
@@ -73,6 +80,55 @@ __device__ __forceinline__ void bfuse_body(const void* I1, const void* F1, void*
 }
 
 template <class A, class B>
+struct BfuseRtPair {
+    static constexpr int THREADS = imax(A::THREADS, B::THREADS);
+    static constexpr int GRID = A::GRID.size() + B::GRID.size();
+    static_assert(A::THREADS % kWaveSize == 0 && B::THREADS % kWaveSize == 0, "block sizes must be whole waves");
+};
+
+// A workgroup runs blocks of both operators one after the other, so waves that one operator
+// does not use cannot simply exit as they do under plain block fusion; they skip the body and
+// wait at the next iteration's workgroup barrier.  An operator narrower than the workgroup
+// therefore cannot use s_barrier inside its body (the idle waves would be counted): it gets the
+// LDS-counter barrier over its own waves, as under horizontal fusion.
+template <class A, class B>
+__device__ __forceinline__ void bfuse_rt_body(const BlockPlan& plan, const void* I1, const void* F1, void* O1,
+                                              const void* I2, const void* F2, void* O2)
+{
+    struct Shrd {
+        union {
+            typename A::Smem a;
+            typename B::Smem b;
+        } u;
+        // arrival counters of the LDS-counter barriers, three sets used in rotation: the set
+        // zeroed at the top of iteration i is the one iteration i+1 will use, and it is not the
+        // one a slow wave may still be polling from iteration i-1
+        unsigned int arrive[3][2];
+    };
+    __shared__ Shrd sh;
+    constexpr int T = BfuseRtPair<A, B>::THREADS;
+    const int tid = (int)threadIdx.x;
+    const int total = plan.fused_grid;
+    if (tid < 6) (&sh.arrive[0][0])[tid] = 0u;
+    int set = 0;
+    for (int id = (int)blockIdx.x; id < total; id += (int)gridDim.x) {
+        const int next = set == 2 ? 0 : set + 1;
+        if (tid < 2) sh.arrive[next][tid] = 0u;
+        __syncthreads();  // every wave has left the previous iteration: its LDS contents are dead
+        int virt = 0;
+        const int kernel_id = map_block(plan, id, &virt);
+        if (kernel_id == 0 && tid < A::THREADS) {
+            if constexpr (A::THREADS == T) A::run(virt, tid, sh.u.a, I1, F1, O1, BlockSync{});
+            else A::run(virt, tid, sh.u.a, I1, F1, O1, GroupSync{&sh.arrive[set][0], (unsigned)(A::THREADS / kWaveSize), 0u});
+        } else if (kernel_id == 1 && tid < B::THREADS) {
+            if constexpr (B::THREADS == T) B::run(virt, tid, sh.u.b, I2, F2, O2, BlockSync{});
+            else B::run(virt, tid, sh.u.b, I2, F2, O2, GroupSync{&sh.arrive[set][1], (unsigned)(B::THREADS / kWaveSize), 0u});
+        }
+        set = next;
+    }
+}
+
+template <class A, class B>
 struct HfusePair {
     static constexpr LaunchDims dims[2] = {{A::GRID, A::BLOCK}, {B::GRID, B::BLOCK}};
     static constexpr ThreadPlan plan() { return plan_threads(2, dims, kWaveSize); }
@@ -104,7 +160,7 @@ __device__ __forceinline__ void hfuse_body(const void* I1, const void* F1, void*
 }
 
 // ---- registry ---------------------------------------------------------------------------
-enum KernelKind : int { kSingle = 0, kBfuse = 1, kHfuse = 2 };
+enum KernelKind : int { kSingle = 0, kBfuse = 1, kHfuse = 2, kBfuseRt = 3 };
 
 struct TensorDesc {
     int shape[4];   // padded with 1s, as the reference's macro.h tables (macro_h.py:28-42)
@@ -121,6 +177,7 @@ struct KernelEntry {
     std::string side[2];    // fused: names of the two standalone kernels
     int pattern, p0, p1;    // bfuse: dispatch pattern and its parameters
     unsigned (*read_sync_timeouts)();  // device counter of GroupSync give-ups in this module
+    int (*set_plan)(const BlockPlan*); // bfuse_rt: copies a plan into the kernel's device-side plan (0 = ok)
 };
 
 std::vector<KernelEntry>& registry();
@@ -211,3 +268,26 @@ KernelEntry make_fused_entry(const char* name, const void* func, int kind, const
         bfuse::make_fused_entry<bfuse::HfusePair<OP1, OP2>>(                                         \
             #K1 "_" #K2 "_fused_hfuse", (const void*)&K1##_##K2##_fused_hfuse, bfuse::kHfuse, #K1, #K2, \
             OP1::HAS_BARRIERS || OP2::HAS_BARRIERS, -1, 0, 0, &bfuse_module_read_sync_timeouts));
+
+// The plan sits in device memory next to the kernel; the host writes it with an ordinary
+// (stream-ordered) copy before launching.
+#define BFUSE_BFUSE_RT_KERNEL(K1, OP1, K2, OP2)                                                      \
+    static __device__ bfuse::BlockPlan plan_##K1##_##K2##_rt;                                        \
+    extern "C" __global__ __launch_bounds__((bfuse::BfuseRtPair<OP1, OP2>::THREADS), bfuse::kMinWavesPerEu)                 \
+    void K1##_##K2##_fused_bfuse_rt(const void* __restrict__ I1, const void* __restrict__ F1,        \
+                                    void* __restrict__ O1, const void* __restrict__ I2,              \
+                                    const void* __restrict__ F2, void* __restrict__ O2)              \
+    {                                                                                               \
+        bfuse::bfuse_rt_body<OP1, OP2>(plan_##K1##_##K2##_rt, I1, F1, O1, I2, F2, O2);               \
+    }                                                                                               \
+    static int set_plan_##K1##_##K2##_rt(const bfuse::BlockPlan* p)                                  \
+    {                                                                                               \
+        return hipMemcpyToSymbol(HIP_SYMBOL(plan_##K1##_##K2##_rt), p, sizeof(*p)) == hipSuccess ? 0 : 1; \
+    }                                                                                               \
+    static bfuse::Registrar reg_##K1##_##K2##_bfuse_rt([] {                                          \
+        bfuse::KernelEntry e = bfuse::make_fused_entry<bfuse::BfuseRtPair<OP1, OP2>>(                \
+            #K1 "_" #K2 "_fused_bfuse_rt", (const void*)&K1##_##K2##_fused_bfuse_rt, bfuse::kBfuseRt, #K1, #K2, \
+            true, -1, 0, 0, &bfuse_module_read_sync_timeouts);                                       \
+        e.set_plan = &set_plan_##K1##_##K2##_rt;                                                     \
+        return e;                                                                                   \
+    }());

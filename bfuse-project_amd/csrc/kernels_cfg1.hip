@@ -18,3 +18,5 @@ BFUSE_KERNEL(bias_relu_1048576, BiasRelu1M, ({{1048576, 1, 1, 1}, 4}), ({{104857
 BFUSE_HFUSE_KERNEL(gemm_f32_512x512x512, Gemm512, bias_relu_1048576, BiasRelu1M)
 BFUSE_BFUSE_KERNEL(gemm_f32_512x512x512, Gemm512, bias_relu_1048576, BiasRelu1M, , bfuse::kZigzag, 1, 1)
 BFUSE_BFUSE_KERNEL(gemm_f32_512x512x512, Gemm512, bias_relu_1048576, BiasRelu1M, _c8, bfuse::kChunked, 8, 1)
+// the same pair with its dispatch plan as run-time data and persistent workgroups
+BFUSE_BFUSE_RT_KERNEL(gemm_f32_512x512x512, Gemm512, bias_relu_1048576, BiasRelu1M)

@@ -38,3 +38,5 @@ BFUSE_BFUSE_KERNEL(gemm_f32_512x768x2304, GemmQkv, layernorm_512x768, LnBert, , 
 BFUSE_BFUSE_KERNEL(gemm_f32_512x768x2304, GemmQkv, layernorm_512x768, LnBert, _z2, bfuse::kZigzag, 2, 1)
 BFUSE_BFUSE_KERNEL(gemm_f32_512x768x2304, GemmQkv, layernorm_512x768, LnBert, _c8, bfuse::kChunked, 8, 1)
 BFUSE_BFUSE_KERNEL(gemm_f32_512x768x2304, GemmQkv, layernorm_512x768, LnBert, _r, bfuse::kRanges, 0, 0)
+// the same pair with its dispatch plan as run-time data and persistent workgroups
+BFUSE_BFUSE_RT_KERNEL(gemm_f32_512x768x2304, GemmQkv, layernorm_512x768_w1, LnBert1)

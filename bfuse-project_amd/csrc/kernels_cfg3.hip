@@ -22,3 +22,5 @@ BFUSE_BFUSE_KERNEL(conv3x3_f32_64x56x56_64, Conv64, maxpool3x3s2_f32_64x112x112,
 BFUSE_HFUSE_KERNEL(conv3x3_f32_64x56x56_64, Conv64, maxpool3x3s2_f32_64x112x112, Pool)
 BFUSE_BFUSE_KERNEL(conv3x3_f32_64x56x56_64_h, Conv32, maxpool3x3s2_f32_64x112x112, Pool, , bfuse::kZigzag, 1, 1)
 BFUSE_BFUSE_KERNEL(conv3x3_f32_64x56x56_64_h, Conv32, maxpool3x3s2_f32_64x112x112, Pool, _c8, bfuse::kChunked, 8, 1)
+// the same pair with its dispatch plan as run-time data and persistent workgroups
+BFUSE_BFUSE_RT_KERNEL(conv3x3_f32_64x56x56_64, Conv64, maxpool3x3s2_f32_64x112x112, Pool)

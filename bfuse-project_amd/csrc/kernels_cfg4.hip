@@ -54,3 +54,5 @@ BFUSE_KERNEL(gemm_gelu_f32_512x768x3072_l, GemmFcL, ({{512, 768, 1, 1}, 4}), ({{
 BFUSE_HFUSE_KERNEL(softmax_causal_12x512x512_r6, Softmax4x6, gemm_gelu_f32_512x768x3072_l, GemmFcL)
 BFUSE_BFUSE_KERNEL(softmax_causal_12x512x512_b4, Softmax4b, gemm_gelu_f32_512x768x3072_l, GemmFcL, _c256, bfuse::kChunked, 256, 1)
 BFUSE_BFUSE_KERNEL(softmax_causal_12x512x512, Softmax4, gemm_gelu_f32_512x768x3072_l, GemmFcL, _c256, bfuse::kChunked, 256, 1)
+// the same pair with its dispatch plan as run-time data and persistent workgroups
+BFUSE_BFUSE_RT_KERNEL(softmax_causal_12x512x512, Softmax4, gemm_gelu_f32_512x768x3072_l, GemmFcL)

@@ -34,3 +34,5 @@ BFUSE_BFUSE_KERNEL(gemm_bf16_512x4096x14336_w8, GemmGate8, rmsnorm_rope_bf16_512
 BFUSE_BFUSE_KERNEL(gemm_bf16_512x4096x14336_r, GemmGateR, rmsnorm_rope_bf16_512x4096, NormRope1, _c256, bfuse::kChunked, 256, 1)
 // thread-level fusion: every workgroup = one GEMM tile (eight waves) + two rows of the norm (two waves)
 BFUSE_HFUSE_KERNEL(gemm_bf16_512x4096x14336_w8, GemmGate8, rmsnorm_rope_bf16_512x4096_w2, NormRope2)
+// the same pair with its dispatch plan as run-time data and persistent workgroups
+BFUSE_BFUSE_RT_KERNEL(gemm_bf16_512x4096x14336_w8, GemmGate8, rmsnorm_rope_bf16_512x4096, NormRope1)

@@ -74,3 +74,8 @@ BFUSE_HFUSE_KERNEL(maxpool3x3s2_f32_4x16x16, PoolS, layernorm_8x256, LayerNormS)
 BFUSE_HFUSE_KERNEL(gemm_bf16_256x320x1792_d, GemmB3, rmsnorm_rope_bf16_6x1024, NormRopeS)
 BFUSE_HFUSE_KERNEL(gemm_f32_128x160x192_l, GemmS4, bias_relu_4096, BiasReluS)
 BFUSE_HFUSE_KERNEL(gemm_bf16_256x320x1792_r, GemmB6, rmsnorm_rope_bf16_6x1024, NormRopeS)
+// run-time plans / persistent workgroups: equal and unequal workgroup widths, barrier-bearing sides
+BFUSE_BFUSE_RT_KERNEL(conv3x3_f32_32x12x12_32, ConvS2, gemm_gelu_f32_96x128x192, GemmS2)
+BFUSE_BFUSE_RT_KERNEL(layernorm_8x256, LayerNormS, softmax_causal_2x256x256, SoftmaxS)
+BFUSE_BFUSE_RT_KERNEL(gemm_bf16_256x320x1792_d, GemmB3, rmsnorm_rope_bf16_6x1024, NormRopeS)
+BFUSE_BFUSE_RT_KERNEL(gemm_f32_128x160x192_l, GemmS4, bias_relu_4096, BiasReluS)

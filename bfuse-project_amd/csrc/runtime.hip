@@ -9,6 +9,7 @@
 #include <cstdio>
 #include <cstring>
 #include <string>
+#include <map>
 #include <vector>
 
 #include "../../include/bfuse_rt.h"
@@ -120,6 +121,13 @@ const KernelEntry* entry_of(const void* func)
 // The grid and block a caller passes must be the ones the kernel was built for: the bodies
 // index memory from compile-time shapes, so any other launch shape would read or write out
 // of bounds.
+// plans currently installed in run-time-plan kernels (host copies, for launch validation)
+std::map<const void*, BlockPlan>& installed_plans()
+{
+    static std::map<const void*, BlockPlan> m;
+    return m;
+}
+
 int check_launch(const void* func, const unsigned* grid, const unsigned* block, int want_ptrs)
 {
     if (!func || !grid || !block) return fail(BFUSE_ERR_ARG, "null launch argument");
@@ -127,6 +135,17 @@ int check_launch(const void* func, const unsigned* grid, const unsigned* block, 
     if (!e) return fail(BFUSE_ERR_ARG, "func is not a kernel of this library");
     const int ptrs = e->kind == kSingle ? 3 : 6;
     if (ptrs != want_ptrs) return fail(BFUSE_ERR_ARG, "%s takes %d pointers, not %d", e->name.c_str(), ptrs, want_ptrs);
+    if (e->kind == kBfuseRt) {
+        // persistent workgroups stride over the plan's fused grid: any grid from 1 to that size covers it
+        auto it = installed_plans().find(func);
+        if (it == installed_plans().end()) return fail(BFUSE_ERR_STATE, "%s has no plan: call bfuse_set_plan first", e->name.c_str());
+        for (int i = 0; i < 3; ++i)
+            if (block[i] != e->block[i])
+                return fail(BFUSE_ERR_ARG, "%s must be launched with block (%u,%u,%u)", e->name.c_str(), e->block[0], e->block[1], e->block[2]);
+        if (grid[1] != 1 || grid[2] != 1 || grid[0] < 1 || grid[0] > (unsigned)it->second.fused_grid)
+            return fail(BFUSE_ERR_ARG, "%s takes a 1-D grid of 1..%d workgroups", e->name.c_str(), it->second.fused_grid);
+        return BFUSE_OK;
+    }
     for (int i = 0; i < 3; ++i)
         if (grid[i] != e->grid[i] || block[i] != e->block[i])
             return fail(BFUSE_ERR_ARG, "%s must be launched with grid (%u,%u,%u) block (%u,%u,%u)", e->name.c_str(),
@@ -195,7 +214,7 @@ int sync_and_check(const void* fused_func)
     HIP_TRY(hipGetLastError());
     if (fused_func) {
         const KernelEntry* e = entry_of(fused_func);
-        if (e && e->kind == kHfuse && e->read_sync_timeouts) {
+        if (e && (e->kind == kHfuse || e->kind == kBfuseRt) && e->read_sync_timeouts) {
             unsigned n = e->read_sync_timeouts();
             if (n) return fail(BFUSE_ERR_SYNC, "%s: %u side-barrier waits gave up", e->name.c_str(), n);
         }
@@ -223,7 +242,7 @@ int validate_mode(int mode, const void* fa, const unsigned* ga, const unsigned* 
         case BFUSE_MODE_BFUSE: {
             if ((rc = check_launch(fa, ga, ba, 6)) || (rc = check_fused_fits(fa))) return rc;
             const KernelEntry* e = entry_of(fa);
-            if ((mode == BFUSE_MODE_HFUSE) != (e->kind == kHfuse))
+            if ((mode == BFUSE_MODE_HFUSE) != (e->kind == kHfuse))  // bfuse mode takes compile-time and run-time plans alike
                 return fail(BFUSE_ERR_ARG, "%s is not a %s kernel", e->name.c_str(), mode == BFUSE_MODE_HFUSE ? "hfuse" : "bfuse");
             break;
         }
@@ -379,6 +398,47 @@ int bfuse_map_blocks_device(const bfuse_block_plan* plan, int lo, int hi, int* k
     HIP_TRY(hipMemcpy(virt_out, dv, sizeof(int) * (size_t)n, hipMemcpyDeviceToHost));
     HIP_TRY(hipFree(dk));
     HIP_TRY(hipFree(dv));
+    return BFUSE_OK;
+}
+
+int bfuse_set_plan(const void* func, const bfuse_block_plan* plan)
+{
+    if (!g.inited) return fail(BFUSE_ERR_STATE, "bfuse_init has not been called");
+    if (!func || !plan) return fail(BFUSE_ERR_ARG, "null argument");
+    const KernelEntry* e = entry_of(func);
+    if (!e || e->kind != kBfuseRt || !e->set_plan) return fail(BFUSE_ERR_ARG, "func is not a run-time-plan (bfuse_rt) kernel");
+    BlockPlan p;
+    memcpy(&p, plan, sizeof(p));
+    // The kernel trusts the plan for every index it forms, so it is checked here in full: it must
+    // send the fused block ids one-to-one onto the blocks of the two sides.
+    int side_grid[2] = {0, 0};
+    for (int k = 0; k < 2; ++k)
+        for (const auto& c : registry())
+            if (c.kind == kSingle && c.name == e->side[k]) side_grid[k] = (int)c.grid[0];
+    if (p.n_kernels != 2 || p.n_seg < 1 || p.n_seg > kMaxSegments) return fail(BFUSE_ERR_ARG, "plan: bad kernel or segment count");
+    if (p.fused_grid != side_grid[0] + side_grid[1])
+        return fail(BFUSE_ERR_ARG, "plan covers %d blocks, %s has %d + %d", p.fused_grid, e->name.c_str(), side_grid[0], side_grid[1]);
+    for (int i = 0; i < p.n_seg; ++i) {
+        const Segment& sg = p.seg[i];
+        if (sg.period < 1 || sg.n_slot < 1 || sg.n_slot > kMaxKernels || sg.lo < 0 || sg.hi < sg.lo) return fail(BFUSE_ERR_ARG, "plan: malformed segment %d", i);
+        for (int j = 0; j < sg.n_slot; ++j)
+            if (sg.slot[j].kern < 0 || sg.slot[j].kern > 1 || sg.slot[j].width < 1 || sg.slot[j].off < 0 || sg.slot[j].base < 0)
+                return fail(BFUSE_ERR_ARG, "plan: malformed slot %d of segment %d", j, i);
+    }
+    std::vector<unsigned char> seen[2] = {std::vector<unsigned char>((size_t)side_grid[0], 0), std::vector<unsigned char>((size_t)side_grid[1], 0)};
+    for (int bid = 0; bid < p.fused_grid; ++bid) {
+        int v = -1;
+        const int k = map_block(p, bid, &v);
+        if (k < 0 || k > 1 || v < 0 || v >= side_grid[k] || seen[k][(size_t)v])
+            return fail(BFUSE_ERR_ARG, "plan: fused block %d maps to kernel %d block %d (out of range or visited twice)", bid, k, v);
+        seen[k][(size_t)v] = 1;
+    }
+    HIP_TRY(hipDeviceSynchronize());  // no launch may still be reading the old plan
+    if (e->set_plan(&p)) {
+        (void)hipGetLastError();
+        return fail(BFUSE_ERR_HIP, "could not copy the plan to the device");
+    }
+    installed_plans()[func] = p;
     return BFUSE_OK;
 }
 

@@ -3,7 +3,7 @@ operation_cu.py:123-256): initialize / run_kernel1 / run_kernel2 / run_parallel 
 finalize over numpy buffers, plus the device-resident launch and GPU-side timing entry points.
 """
 import ctypes as C
-from dataclasses import dataclass
+from dataclasses import dataclass, replace
 from typing import List, Optional, Sequence
 
 import numpy as np
@@ -17,7 +17,7 @@ MODES = {"kernel1": 0, "kernel2": 1, "parallel": 2, "hfuse": 3, "bfuse": 4, "ser
 class KernelHandle:
     name: str
     func: int
-    kind: int                 # 0 single, 1 bfuse, 2 hfuse
+    kind: int                 # 0 single, 1 bfuse, 2 hfuse, 3 bfuse with a run-time plan (persistent workgroups)
     grid: tuple
     block: tuple
     has_barriers: bool
@@ -115,6 +115,17 @@ class Operation:
 
     def fused(self, kind: str, suffix: str = "") -> KernelHandle:
         return kernel_info(f"{self.k[0].name}_{self.k[1].name}_fused_{kind}{suffix}")
+
+    def fused_rt(self) -> KernelHandle:
+        """The block-fused kernel of this pair whose dispatch plan is set at run time."""
+        return kernel_info(f"{self.k[0].name}_{self.k[1].name}_fused_bfuse_rt")
+
+    def set_plan(self, fused: KernelHandle, plan, workgroups: Optional[int] = None) -> KernelHandle:
+        """Installs `plan` (patterns.BlockPlan) in a run-time-plan kernel and returns the handle to
+        launch it with: the plan's fused grid, or `workgroups` persistent workgroups striding over it."""
+        _lib.check(self.l.bfuse_set_plan(fused.func, C.byref(plan.c)))
+        n = plan.fused_grid if workgroups is None else min(int(workgroups), plan.fused_grid)
+        return replace(fused, grid=(n, 1, 1))
 
     # -- operation.h mirror (H2D, launch, sync, D2H) ---------------------------------------
     def run_kernel(self, side: int, I, F) -> np.ndarray:

@@ -1,0 +1,83 @@
+"""Pattern / ratio chooser for a pair, measured at run time.
+
+The reference hard-codes the live pattern and its M, N in Contexts.cc:64-79 and sweeps ratios
+by editing that file and rebuilding the tool and the suite for every point
+(legacy/tests/single_bgemm_conv2d/auto.py:9-30: M in 1..512 with N = 1, then N in 1..512 with
+M = 1).  Here the dispatch table of a `..._fused_bfuse_rt` kernel is data, so the same sweep is
+a loop of `set_plan` + timed launches over resident buffers, and it also covers what the
+reference never made selectable (its chunked and proportional patterns, plain ranges) and
+persistent workgroups.
+
+`static_choice` is the part that needs no measurement: it reads what the code objects say
+(KernelInfo.Reg / LDS / HasBarriers, fields the reference parses and never uses) and prunes.
+"""
+from dataclasses import dataclass
+from typing import List, Optional, Sequence
+
+import numpy as np
+
+from . import config, patterns
+from .operation import KernelHandle, Operation
+
+
+@dataclass
+class Candidate:
+    label: str
+    pattern: str
+    p0: int = 1
+    p1: int = 1
+    workgroups: Optional[int] = None   # None: one workgroup per fused block; else persistent
+
+
+def ratio_sweep(max_ratio: int = 512) -> List[Candidate]:
+    """The reference's sweep: M = 1, 2, 4, ... with N = 1, then N = 2, 4, ... with M = 1."""
+    out = [Candidate("zigzag 1:1", "zigzag", 1, 1)]
+    r = 2
+    while r <= max_ratio:
+        out.append(Candidate(f"zigzag M={r}", "zigzag", r, 1))
+        out.append(Candidate(f"zigzag N={r}", "zigzag", 1, r))
+        r *= 2
+    return out
+
+
+def default_candidates(g1: int, g2: int, cus: int = 256) -> List[Candidate]:
+    small, big = min(g1, g2), max(g1, g2)
+    out = [Candidate("ranges", "ranges")]
+    for c in (cus // 4, cus // 2, cus, 2 * cus):
+        if c < big:
+            out.append(Candidate(f"chunk {c}", "chunked", c))
+    out.append(Candidate("zigzag 1:1", "zigzag", 1, 1))
+    r = 2
+    while r <= max(2, big // max(small, 1)) and r <= 64:
+        out.append(Candidate(f"zigzag M={r}", "zigzag", r, 1))
+        r *= 2
+    out.append(Candidate("proportional", "proportional", 1))
+    for k in (1, 2, 4):
+        if k * cus < g1 + g2:
+            out.append(Candidate(f"chunk {cus}, {k * cus} persistent workgroups", "chunked", cus, 1, k * cus))
+    return out
+
+
+def static_choice(a: KernelHandle, b: KernelHandle, cus: int = 256) -> dict:
+    """What the code-object metadata alone says (no launch)."""
+    ka = config.KernelInfo(a.name, a.has_barriers, a.grid, a.block, max(a.regs, 1))
+    kb = config.KernelInfo(b.name, b.has_barriers, b.grid, b.block, max(b.regs, 1))
+    return config.choose_fusion(ka, kb, max(a.lds_bytes, 0), max(b.lds_bytes, 0), cus)
+
+
+def autotune(op: Operation, candidates: Optional[Sequence[Candidate]] = None, warmup: int = 3, reps: int = 30,
+             cus: int = 256) -> List[dict]:
+    """Times every candidate plan of the pair's run-time-plan kernel over the buffers `op` holds
+    (upload operands first).  Returns rows sorted by mean GPU time; row 0 is the choice."""
+    rt = op.fused_rt()
+    dims = [k_.grid[0] for k_ in op.k]
+    ldims = [patterns.LaunchDims(tuple(k_.grid), tuple(k_.block)) for k_ in op.k]
+    rows = []
+    for c in (candidates if candidates is not None else default_candidates(dims[0], dims[1], cus)):
+        plan = patterns.plan_blocks(c.pattern, ldims, c.p0, c.p1)
+        h = op.set_plan(rt, plan, c.workgroups)
+        t = op.time("bfuse", h, warmup=warmup, reps=reps)[0]
+        rows.append({"label": c.label, "pattern": c.pattern, "p0": c.p0, "p1": c.p1, "workgroups": h.grid[0],
+                     "us_mean": float(np.mean(t)), "us_min": float(np.min(t)), "us_std": float(np.std(t))})
+    rows.sort(key=lambda r: r["us_mean"])
+    return rows

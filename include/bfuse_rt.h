@@ -82,6 +82,16 @@ int bfuse_map_block(const bfuse_block_plan* plan, int bid, int* virt_block);
 int bfuse_map_thread(const bfuse_thread_plan* plan, int bid, int tid, int* local_tid);
 /* Evaluates bfuse_map_block for bid in [lo,hi) ON THE GPU with the device build of the map
  * (one thread per fused block) and copies the tables back. */
+/* Installs `plan` in a run-time-plan kernel (`<K1>_<K2>_fused_bfuse_rt`, kind 3): the same block
+ * fusion, with the dispatch table as data instead of compiled in, so patterns and M:N ratios can
+ * be swept without rebuilding (the reference's sweep edits Contexts.cc and rebuilds per ratio,
+ * legacy/tests/single_bgemm_conv2d/auto.py:9-14).  The plan must map the fused block ids
+ * one-to-one onto the blocks of the two sides; anything else is refused.  Afterwards the kernel
+ * may be launched (mode BFUSE_MODE_BFUSE) with any 1-D grid from 1 to plan->fused_grid
+ * workgroups: workgroup w handles fused blocks w, w + grid, ... (persistent workgroups, the
+ * reference's legacy/tests/thread_pooling_test/temp.cu:576-612). */
+int bfuse_set_plan(const void* func, const bfuse_block_plan* plan);
+
 int bfuse_map_blocks_device(const bfuse_block_plan* plan, int lo, int hi, int* kernel_out, int* virt_out);
 
 /* ------------------------------------------------------------------------------------------

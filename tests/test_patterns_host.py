@@ -106,3 +106,16 @@ def test_bad_arguments_are_rejected():
         bf.plan_blocks("zigzag", [bf.LaunchDims((0, 1, 1), (64, 1, 1))] * 2, 1, 1)
     with pytest.raises(bf.BfuseError):
         bf.plan_threads(d * 5)
+
+
+def test_tuner_candidates():
+    from bfuse_project_amd import tuner
+    sweep = tuner.ratio_sweep(512)
+    # the reference's sweep: M = 1..512 with N = 1, then N = 2..512 with M = 1 (auto.py:9-14)
+    assert [(c.p0, c.p1) for c in sweep if c.p1 == 1] == [(1 << i, 1) for i in range(10)]
+    assert [(c.p0, c.p1) for c in sweep if c.p0 == 1 and c.p1 > 1] == [(1, 1 << i) for i in range(1, 10)]
+    cands = tuner.default_candidates(256, 512, cus=256)
+    labels = [c.label for c in cands]
+    assert "ranges" in labels and "zigzag 1:1" in labels and "chunk 256" in labels and "proportional" in labels
+    assert all(c.workgroups is None or c.workgroups < 256 + 512 for c in cands)
+    assert any(c.workgroups == 256 for c in cands)
