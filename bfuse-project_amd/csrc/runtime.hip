@@ -284,6 +284,21 @@ __global__ void map_blocks_kernel(BlockPlan plan, int lo, int hi, int* kernel_ou
     }
 }
 
+// Where the hardware put each workgroup: HW_ID (wave, SIMD, CU, shader array, shader engine) and
+// XCC_ID of the wave that runs thread 0, plus a wall-clock stamp.  The workgroup spins for
+// `hold` clock reads so that later workgroups cannot reuse its slot.
+__global__ void placement_kernel(unsigned* hw_id, unsigned* xcc_id, unsigned long long* t_start, int hold)
+{
+    const unsigned long long t0 = wall_clock64();
+    if (threadIdx.x == 0) {
+        hw_id[blockIdx.x] = __builtin_amdgcn_s_getreg((31 << 11) | 4);    // HW_REG_HW_ID, 32 bits
+        xcc_id[blockIdx.x] = __builtin_amdgcn_s_getreg((3 << 11) | 20);   // HW_REG_XCC_ID, bits 3:0
+        t_start[blockIdx.x] = t0;
+    }
+    for (int i = 0; i < hold; ++i)
+        if (wall_clock64() == 0ull) hw_id[0] = 0u;  // never true: keeps the loop
+}
+
 inline unsigned long long splitmix64(unsigned long long x)
 {
     x += 0x9E3779B97F4A7C15ull;
@@ -398,6 +413,38 @@ int bfuse_map_blocks_device(const bfuse_block_plan* plan, int lo, int hi, int* k
     HIP_TRY(hipMemcpy(virt_out, dv, sizeof(int) * (size_t)n, hipMemcpyDeviceToHost));
     HIP_TRY(hipFree(dk));
     HIP_TRY(hipFree(dv));
+    return BFUSE_OK;
+}
+
+int bfuse_probe_placement(int workgroups, int threads, int hold, unsigned* xcc, unsigned* se, unsigned* cu, unsigned* simd,
+                          unsigned long long* start_ticks)
+{
+    if (!g.inited) return fail(BFUSE_ERR_STATE, "bfuse_init has not been called");
+    if (workgroups < 1 || workgroups > (1 << 20) || threads < 64 || threads > 1024 || threads % 64 || hold < 0 || hold > 100000)
+        return fail(BFUSE_ERR_ARG, "bad argument");
+    unsigned *d_hw = nullptr, *d_xcc = nullptr;
+    unsigned long long* d_t = nullptr;
+    HIP_TRY(hipMalloc(&d_hw, sizeof(unsigned) * (size_t)workgroups));
+    HIP_TRY(hipMalloc(&d_xcc, sizeof(unsigned) * (size_t)workgroups));
+    HIP_TRY(hipMalloc(&d_t, sizeof(unsigned long long) * (size_t)workgroups));
+    hipLaunchKernelGGL(placement_kernel, dim3(workgroups), dim3(threads), 0, nullptr, d_hw, d_xcc, d_t, hold);
+    HIP_TRY(hipGetLastError());
+    std::vector<unsigned> hw((size_t)workgroups), xc((size_t)workgroups);
+    std::vector<unsigned long long> ts((size_t)workgroups);
+    HIP_TRY(hipMemcpy(hw.data(), d_hw, sizeof(unsigned) * hw.size(), hipMemcpyDeviceToHost));
+    HIP_TRY(hipMemcpy(xc.data(), d_xcc, sizeof(unsigned) * xc.size(), hipMemcpyDeviceToHost));
+    HIP_TRY(hipMemcpy(ts.data(), d_t, sizeof(unsigned long long) * ts.size(), hipMemcpyDeviceToHost));
+    HIP_TRY(hipFree(d_hw));
+    HIP_TRY(hipFree(d_xcc));
+    HIP_TRY(hipFree(d_t));
+    for (int i = 0; i < workgroups; ++i) {
+        const unsigned h = hw[(size_t)i];  // gfx9 layout: wave 3:0, simd 5:4, pipe 7:6, cu 11:8, sh 12, se 15:13
+        if (xcc) xcc[i] = xc[(size_t)i] & 0xFu;
+        if (se) se[i] = (h >> 13) & 0x7u;
+        if (cu) cu[i] = ((h >> 12) & 0x1u) * 16u + ((h >> 8) & 0xFu);
+        if (simd) simd[i] = (h >> 4) & 0x3u;
+        if (start_ticks) start_ticks[i] = ts[(size_t)i];
+    }
     return BFUSE_OK;
 }
 

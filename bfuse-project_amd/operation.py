@@ -288,6 +288,18 @@ def check_matrix(o: np.ndarray, o_ans: np.ndarray, eps: float = 1e-3) -> int:
     return _lib.lib().bfuse_check_matrix(o.ctypes.data, a.ctypes.data, o.size, eps)
 
 
+def probe_placement(workgroups: int, threads: int = 256, hold: int = 2000) -> dict:
+    """Where the hardware puts consecutive workgroup ids: arrays of XCD, shader engine, CU and SIMD
+    per workgroup, plus start ticks."""
+    l = _lib.lib()
+    _lib.check(l.bfuse_init(0))
+    out = {k: np.zeros(workgroups, np.uint32) for k in ("xcc", "se", "cu", "simd")}
+    out["start"] = np.zeros(workgroups, np.uint64)
+    _lib.check(l.bfuse_probe_placement(workgroups, threads, hold, out["xcc"].ctypes.data, out["se"].ctypes.data,
+                                       out["cu"].ctypes.data, out["simd"].ctypes.data, out["start"].ctypes.data))
+    return out
+
+
 def device_name() -> str:
     buf = C.create_string_buffer(256)
     cus, lds, wave = C.c_int(), C.c_int(), C.c_int()

@@ -1,0 +1,344 @@
+"""Pair-matrix driver: run every (kernel1, kernel2) of two fusion sets in every mode, keep the
+GPU-side traces, and tabulate speed-ups.
+
+Counterpart of the reference's suite scripts:
+
+  * scripts/profile_test_suite.py:13-140 -- the command matrix over `benchmark T K1 K2` for the
+    methods kernel1, kernel2, parallel, hfuse, bfuse, 3 warm-up + 30 timed launches, one GPU
+    trace per command (there: nsys; here: rocprofv3 --kernel-trace, or the library's own
+    dispatch timestamps when run in-process);
+  * scripts/analyze_test_suite.py:103-161 -- per-trace statistics (warm-ups dropped; for two
+    kernels on two streams the span from the first start to the later end);
+  * scripts/analyze_test_suite.py:425-428 -- serial = kernel1 + kernel2, speed-up = serial / variant.
+
+The suite description is the reference's `info.yaml`: `FusionSet: [{Set: [...]}, {Set: [...]}]`.
+Set members are kernel names of the library's registry (the reference's `KernelInfo` block,
+operator shapes for TVM, is accepted and ignored: shapes are compiled into the kernels).
+
+    python -m bfuse_project_amd.suite info.yaml -o OUT            # run in-process, write traces + tables
+    python -m bfuse_project_amd.suite info.yaml -o OUT --commands # only print the rocprofv3 command matrix
+    python -m bfuse_project_amd.suite info.yaml -o OUT --analyze  # tables from traces already under OUT/exec
+"""
+import argparse
+import csv
+import json
+import os
+import sys
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+import yaml
+
+METHODS = ["kernel1", "kernel2", "parallel", "hfuse", "bfuse"]   # profile_test_suite.py:25
+WARMUP_TRIALS = 3                                                  # profile_test_suite.py:10-11
+TIMED_TRIALS = 30
+
+
+# ---- suite description ------------------------------------------------------------------
+def load_info(path: str) -> dict:
+    with open(path) as f:
+        info = yaml.safe_load(f)
+    sets = info.get("FusionSet") if isinstance(info, dict) else None
+    if not isinstance(sets, list) or len(sets) != 2:
+        raise ValueError("Number of fusion sets are only 2.")          # profile_test_suite.py:19-21
+    for s in sets:
+        if not isinstance(s, dict) or not isinstance(s.get("Set"), list) or not s["Set"]:
+            raise ValueError("every FusionSet entry needs a non-empty 'Set' list")
+    return info
+
+
+def set_names(info: dict) -> Tuple[List[str], List[str]]:
+    return list(info["FusionSet"][0]["Set"]), list(info["FusionSet"][1]["Set"])
+
+
+def combos(info: dict, triangular: bool = False) -> List[Tuple[int, int]]:
+    """Index pairs to run.  The reference's two sets list the same operators twice and it walks
+    the upper triangle (`for kidx2 in range(kidx1, kernel2_size)`); with distinct sets the full
+    matrix is wanted, which is the default here."""
+    a, b = set_names(info)
+    return [(i, j) for i in range(len(a)) for j in range(i if triangular else 0, len(b))]
+
+
+# ---- command matrix (profile_test_suite.py:13-140) ----------------------------------------------
+def valid_commands(info: dict, benchmark_path: str, triangular: bool = False) -> List[List[str]]:
+    a, b = set_names(info)
+    common = [os.path.abspath(benchmark_path), "-v"]
+    out = []
+    for idx, _ in enumerate(METHODS):
+        if idx == 0:
+            out += [common + [str(idx), k, b[0]] for k in a]
+        elif idx == 1:
+            out += [common + [str(idx), a[0], k] for k in b]
+        else:
+            out += [common + [str(idx), a[i], b[j]] for i, j in combos(info, triangular)]
+    return out
+
+
+def exec_commands(info: dict, benchmark_path: str, exec_path: str, triangular: bool = False) -> List[List[str]]:
+    """One rocprofv3 kernel-trace run per (method, k1, k2); the trace lands in
+    `<exec_path>/<method index>_<i>_<j>_kernel_trace.csv` (the reference's file naming with the
+    profiler's suffix)."""
+    a, b = set_names(info)
+    bench = os.path.abspath(benchmark_path)
+    n = str(WARMUP_TRIALS + TIMED_TRIALS)
+
+    def one(idx, i, j):
+        return ["rocprofv3", "--kernel-trace", "--output-format", "csv", "-d", exec_path, "-o", f"{idx}_{i}_{j}", "--",
+                bench, "-n", n, str(idx), a[i], b[j]]
+    out = []
+    for idx, _ in enumerate(METHODS):
+        if idx == 0:
+            out += [one(idx, i, 0) for i in range(len(a))]
+        elif idx == 1:
+            out += [one(idx, 0, j) for j in range(len(b))]
+        else:
+            out += [one(idx, i, j) for i, j in combos(info, triangular)]
+    return out
+
+
+# ---- traces ---------------------------------------------------------------------------------
+def write_trace(path: str, rows: Sequence[dict]) -> None:
+    with open(path, "w", newline="") as f:
+        w = csv.DictWriter(f, fieldnames=["Start", "Duration", "Name"])
+        w.writeheader()
+        for r in rows:
+            w.writerow({"Start": r["Start"], "Duration": r["Duration"], "Name": r["Name"]})
+
+
+def read_trace(path: str) -> List[dict]:
+    """Rows {Name, Start, Duration} (ns) in start order, from this module's own trace files,
+    from rocprofv3's `*_kernel_trace.csv` (Kernel_Name, Start_Timestamp, End_Timestamp), or from the
+    reference's nsys export (`Start (ns)`, `Duration (ns)`, `Name`)."""
+    out = []
+    with open(path, newline="") as f:
+        for r in csv.DictReader(f):
+            if "Kernel_Name" in r:
+                s, e = float(r["Start_Timestamp"]), float(r["End_Timestamp"])
+                out.append({"Name": r["Kernel_Name"], "Start": s, "Duration": e - s})
+            elif "Start (ns)" in r:
+                if not r.get("Duration (ns)"):
+                    continue
+                out.append({"Name": r["Name"], "Start": float(r["Start (ns)"]), "Duration": float(r["Duration (ns)"])})
+            else:
+                out.append({"Name": r["Name"], "Start": float(r["Start"]), "Duration": float(r["Duration"])})
+    out.sort(key=lambda r: r["Start"])
+    return out
+
+
+def _stats(v: Sequence[float]) -> Tuple[float, float, float, float]:
+    if not len(v):
+        raise ValueError("no timed launches in the trace")
+    a = np.asarray(v, np.float64)
+    return float(a.min()), float(a.max()), float(a.mean()), float(a.std())
+
+
+def single_statistics(rows: Sequence[dict], kernel_name: str, warmup: int = WARMUP_TRIALS):
+    """(min, max, mean, std) of the durations of `kernel_name`, first `warmup` launches dropped
+    (analyze_test_suite.py:103-124)."""
+    d = [r["Duration"] for r in rows if r["Name"] == kernel_name]
+    return _stats(d[warmup:])
+
+
+def parallel_statistics(rows: Sequence[dict], kernel_names: Sequence[str], warmup: int = WARMUP_TRIALS):
+    """Two kernels per repetition: the repetition's time is the first one's duration if it ends
+    last, else the span from its start to the second one's end (analyze_test_suite.py:126-161)."""
+    if len(kernel_names) != 2:
+        raise ValueError("Number of kernel_names must be 2.")
+    sel = [r for r in rows if r["Name"] in kernel_names][warmup * 2:]
+    res = []
+    for first, second in zip(sel[0::2], sel[1::2]):
+        if first["Start"] + first["Duration"] > second["Start"] + second["Duration"]:
+            res.append(first["Duration"])
+        else:
+            res.append(second["Start"] - first["Start"] + second["Duration"])
+    return _stats(res)
+
+
+# ---- in-process run -------------------------------------------------------------------------
+def fused_variants(k1: str, k2: str) -> Dict[str, list]:
+    """Fused kernels the library holds for (k1, k2), by kind ('hfuse' / 'bfuse')."""
+    from .operation import list_kernels
+    out = {"hfuse": [], "bfuse": []}
+    for h in list_kernels():
+        if h.sides == (k1, k2):
+            if h.kind == 2:
+                out["hfuse"].append(h)
+            elif h.kind == 1:
+                out["bfuse"].append(h)
+    return out
+
+
+def _synthetic(handle, seed):
+    """Seeded U(-0.5, 0.5) operands, as the reference's harness fills them (utils_cc.py:28-31)."""
+    from .operation import fill_uniform, f32_to_bf16
+    if handle.name.startswith("rmsnorm_rope_bf16"):
+        # second operand is a byte blob (bf16 weight, fp32 cos and sin tables of 128-wide heads)
+        from .workloads import pack_norm_rope_operand, rope_tables
+        rows, d = handle.shapes[0][0], handle.shapes[0][1]
+        cosv, sinv = rope_tables(rows, 128, 500000.0)
+        return [f32_to_bf16(fill_uniform(seed, rows * d, -0.5, 0.5)),
+                pack_norm_rope_operand(f32_to_bf16(fill_uniform(seed + 1, d, 0.5, 1.5)), cosv, sinv)]
+    out = []
+    for idx in (0, 1):
+        n = int(np.prod(handle.shapes[idx]))
+        eb = handle.elem_bytes[idx]
+        v = fill_uniform(seed + idx, n if eb != 1 else (n + 3) // 4, -0.5, 0.5)
+        out.append(v if eb == 4 else f32_to_bf16(v) if eb == 2 else v.view(np.uint8)[:n].copy())
+    return out
+
+
+def run_suite(info: dict, out_dir: str, validate: bool = True, triangular: bool = False, log=print) -> List[dict]:
+    """Runs the matrix over resident buffers with the library's dispatch timestamps, writes one
+    trace per (method, i, j) under `<out_dir>/exec/` and returns the analysed rows."""
+    from .operation import Operation
+    a, b = set_names(info)
+    exec_dir = os.path.join(out_dir, "exec")
+    os.makedirs(exec_dir, exist_ok=True)
+    n_rep = TIMED_TRIALS
+
+    def trace_of(t_tot, t_a, t_b, names):
+        rows, clock = [], 0.0
+        for r in range(len(t_tot)):
+            if len(names) == 1:
+                rows.append({"Name": names[0], "Start": clock, "Duration": float(t_tot[r]) * 1e3})
+            else:
+                # two dispatches: the first starts the repetition, the second ends it
+                rows.append({"Name": names[0], "Start": clock, "Duration": float(t_a[r]) * 1e3})
+                rows.append({"Name": names[1], "Start": clock + (float(t_tot[r]) - float(t_b[r])) * 1e3, "Duration": float(t_b[r]) * 1e3})
+            clock += float(t_tot[r]) * 1e3 + 1e3
+        return rows
+
+    for i, j in combos(info, triangular):
+        k1, k2 = a[i], b[j]
+        with Operation(k1, k2) as op:
+            I1, F1 = _synthetic(op.k[0], 0xB5F05E + 2 * i)
+            I2, F2 = _synthetic(op.k[1], 0xB5F05E + 1000 + 2 * j)
+            op.upload(0, I1, F1)
+            op.upload(1, I2, F2)
+            base = None
+            if validate:
+                base = (op.run_kernel(0, I1, F1), op.run_kernel(1, I2, F2))
+                op.upload(0, I1, F1)
+                op.upload(1, I2, F2)
+            # warm-ups are part of the trace, as in the reference's -n 33 runs
+            t = op.time("kernel1", warmup=0, reps=WARMUP_TRIALS + n_rep)
+            write_trace(os.path.join(exec_dir, f"0_{i}_0.csv"), trace_of(t[0], t[1], t[2], [k1]))
+            t = op.time("kernel2", warmup=0, reps=WARMUP_TRIALS + n_rep)
+            write_trace(os.path.join(exec_dir, f"1_0_{j}.csv"), trace_of(t[0], t[1], t[2], [k2]))
+            t = op.time("parallel", warmup=0, reps=WARMUP_TRIALS + n_rep)
+            write_trace(os.path.join(exec_dir, f"2_{i}_{j}.csv"), trace_of(t[0], t[1], t[2], [k1, k2]))
+            for kind, idx in (("hfuse", 3), ("bfuse", 4)):
+                best = None
+                for h in fused_variants(k1, k2)[kind]:
+                    if validate:
+                        op.zero_outputs()
+                        Q1, Q2 = op.run_fuse(h, I1, F1, I2, F2)
+                        if not (np.array_equal(Q1.view(np.uint8), base[0].view(np.uint8)) and np.array_equal(Q2.view(np.uint8), base[1].view(np.uint8))):
+                            raise RuntimeError(f"{h.name}: output differs from the unfused kernels")
+                    t = op.time(kind, h, warmup=0, reps=WARMUP_TRIALS + n_rep)
+                    m = float(np.mean(t[0][WARMUP_TRIALS:]))
+                    if best is None or m < best[0]:
+                        best = (m, h, t)
+                if best:
+                    _, h, t = best
+                    write_trace(os.path.join(exec_dir, f"{idx}_{i}_{j}.csv"), trace_of(t[0], t[1], t[2], [h.name]))
+                    with open(os.path.join(exec_dir, f"{idx}_{i}_{j}.name"), "w") as f:
+                        f.write(h.name + "\n")
+        log(f"[suite] {k1} x {k2} done")
+    return analyze(info, exec_dir, triangular)
+
+
+# ---- tables (analyze_test_suite.py:425-428) -----------------------------------------------------
+def _find(exec_dir: str, stem: str) -> Optional[str]:
+    for suffix in (".csv", "_kernel_trace.csv"):
+        p = os.path.join(exec_dir, stem + suffix)
+        if os.path.exists(p):
+            return p
+    return None
+
+
+def analyze(info: dict, exec_dir: str, triangular: bool = False) -> List[dict]:
+    a, b = set_names(info)
+    rows = []
+    for i, j in combos(info, triangular):
+        k1, k2 = a[i], b[j]
+        p1, p2 = _find(exec_dir, f"0_{i}_0"), _find(exec_dir, f"1_0_{j}")
+        if not p1 or not p2:
+            continue
+        t1 = single_statistics(read_trace(p1), k1)[2]
+        t2 = single_statistics(read_trace(p2), k2)[2]
+        row = {"kernel1": k1, "kernel2": k2, "kernel1_ns": t1, "kernel2_ns": t2, "serial_ns": t1 + t2}
+        pp = _find(exec_dir, f"2_{i}_{j}")
+        if pp:
+            row["parallel_ns"] = parallel_statistics(read_trace(pp), [k1, k2])[2]
+            row["parallel_speedup"] = row["serial_ns"] / row["parallel_ns"]
+        for kind, idx in (("hfuse", 3), ("bfuse", 4)):
+            pf = _find(exec_dir, f"{idx}_{i}_{j}")
+            if not pf:
+                continue
+            tr = read_trace(pf)
+            name_file = os.path.join(exec_dir, f"{idx}_{i}_{j}.name")
+            if os.path.exists(name_file):
+                name = open(name_file).read().strip()
+            else:
+                name = next((r["Name"] for r in tr if r["Name"].startswith(f"{k1}_{k2}_fused_{kind}")), None)
+            if name is None:
+                continue
+            row[f"{kind}_kernel"] = name
+            row[f"{kind}_ns"] = single_statistics(tr, name)[2]
+            row[f"{kind}_speedup"] = row["serial_ns"] / row[f"{kind}_ns"]
+        rows.append(row)
+    return rows
+
+
+def geomean(values: Sequence[float]) -> float:
+    v = np.asarray([x for x in values if x and x > 0], np.float64)
+    return float(np.exp(np.log(v).mean())) if len(v) else float("nan")
+
+
+def to_markdown(rows: Sequence[dict]) -> str:
+    head = "| kernel1 | kernel2 | k1 us | k2 us | serial us | parallel | hfuse | bfuse | bfuse kernel |\n|---|---|---|---|---|---|---|---|---|\n"
+    body = ""
+    for r in rows:
+        def f(k):
+            return f"{r[k + '_ns'] / 1e3:.2f} ({r[k + '_speedup']:.2f}x)" if k + "_ns" in r else "-"
+        body += (f"| {r['kernel1']} | {r['kernel2']} | {r['kernel1_ns'] / 1e3:.2f} | {r['kernel2_ns'] / 1e3:.2f} | {r['serial_ns'] / 1e3:.2f} | "
+                 f"{f('parallel')} | {f('hfuse')} | {f('bfuse')} | {r.get('bfuse_kernel', '-')} |\n")
+    tail = "\ngeomean speed-up over serial: " + ", ".join(
+        f"{k} {geomean([r.get(k + '_speedup') for r in rows]):.3f}x" for k in ("parallel", "hfuse", "bfuse"))
+    return head + body + tail + "\n"
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
+    ap.add_argument("file", help="info.yaml with the two fusion sets")
+    ap.add_argument("-o", dest="out", default="suite_out", help="output directory")
+    ap.add_argument("--commands", action="store_true", help="print the rocprofv3 command matrix and exit")
+    ap.add_argument("--analyze", action="store_true", help="only analyse traces already under OUT/exec")
+    ap.add_argument("--triangular", action="store_true", help="walk the upper triangle as the reference does")
+    ap.add_argument("--no-validate", action="store_true")
+    ap.add_argument("--benchmark", default=os.path.join(os.path.dirname(os.path.abspath(__file__)), "benchmark"))
+    args = ap.parse_args(argv)
+    try:
+        info = load_info(args.file)
+    except (OSError, ValueError) as e:
+        print(f"error: {e}", file=sys.stderr)
+        return 1
+    exec_dir = os.path.join(args.out, "exec")
+    if args.commands:
+        for c in exec_commands(info, args.benchmark, exec_dir, args.triangular):
+            print(" ".join(c))
+        return 0
+    rows = analyze(info, exec_dir, args.triangular) if args.analyze else run_suite(info, args.out, not args.no_validate, args.triangular)
+    os.makedirs(args.out, exist_ok=True)
+    with open(os.path.join(args.out, "summary.json"), "w") as f:
+        json.dump(rows, f, indent=1)
+    md = to_markdown(rows)
+    with open(os.path.join(args.out, "summary.md"), "w") as f:
+        f.write(md)
+    print(md)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -82,6 +82,15 @@ int bfuse_map_block(const bfuse_block_plan* plan, int bid, int* virt_block);
 int bfuse_map_thread(const bfuse_thread_plan* plan, int bid, int tid, int* local_tid);
 /* Evaluates bfuse_map_block for bid in [lo,hi) ON THE GPU with the device build of the map
  * (one thread per fused block) and copies the tables back. */
+/* Placement probe: launches `workgroups` workgroups of `threads` threads that each record where
+ * the hardware put them (XCD, shader engine, CU within the engine, SIMD) and when they started
+ * (100 MHz wall-clock ticks), holding their slot for `hold` clock reads.  The counterpart of the
+ * reference's `%smid` experiment (legacy/tests/block_scheduler_test/cuda/kernels.cu, the
+ * "Block: %d | SM: %d" printf) -- on MI355X the answer decides which dispatch pattern works.
+ * Output arrays have `workgroups` entries; any may be NULL. */
+int bfuse_probe_placement(int workgroups, int threads, int hold, unsigned* xcc, unsigned* se, unsigned* cu, unsigned* simd,
+                          unsigned long long* start_ticks);
+
 /* Installs `plan` in a run-time-plan kernel (`<K1>_<K2>_fused_bfuse_rt`, kind 3): the same block
  * fusion, with the dispatch table as data instead of compiled in, so patterns and M:N ratios can
  * be swept without rebuilding (the reference's sweep edits Contexts.cc and rebuilds per ratio,

@@ -1,0 +1,31 @@
+"""Suite driver on the GPU: a 2 x 2 matrix of small kernels through every method, traces on
+disk, speed-up table.  Validation inside the run is the reference's `-v` check tightened to
+bit equality (main_cc.py:246-268)."""
+import os
+
+import pytest
+import yaml
+
+from bfuse_project_amd import suite
+
+pytestmark = pytest.mark.gpu
+
+
+def test_small_matrix(tmp_path):
+    info_path = tmp_path / "info.yaml"
+    info_path.write_text(yaml.safe_dump({"FusionSet": [{"Set": ["conv3x3_f32_32x12x12_32", "layernorm_8x256"]},
+                                                       {"Set": ["gemm_gelu_f32_96x128x192", "softmax_causal_2x256x256"]}]}))
+    info = suite.load_info(str(info_path))
+    rows = suite.run_suite(info, str(tmp_path), validate=True, log=lambda m: print(m, flush=True))
+    assert len(rows) == 4
+    by = {(r["kernel1"], r["kernel2"]): r for r in rows}
+    r = by[("conv3x3_f32_32x12x12_32", "gemm_gelu_f32_96x128x192")]
+    assert r["bfuse_kernel"].startswith("conv3x3_f32_32x12x12_32_gemm_gelu_f32_96x128x192_fused_bfuse")
+    assert r["serial_ns"] == pytest.approx(r["kernel1_ns"] + r["kernel2_ns"]) and r["bfuse_ns"] > 0 and r["parallel_ns"] > 0
+    assert "bfuse_ns" in by[("layernorm_8x256", "softmax_causal_2x256x256")]
+    assert "bfuse_ns" not in by[("layernorm_8x256", "gemm_gelu_f32_96x128x192")]      # no fused kernel built for it
+    for stem in ("0_0_0", "1_0_1", "2_1_1", "4_0_0"):
+        assert os.path.exists(tmp_path / "exec" / f"{stem}.csv")
+    # the traces hold the warm-ups too; the analysis drops them
+    assert len(suite.read_trace(str(tmp_path / "exec" / "0_0_0.csv"))) == suite.WARMUP_TRIALS + suite.TIMED_TRIALS
+    print(suite.to_markdown(rows))

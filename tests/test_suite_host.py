@@ -1,0 +1,113 @@
+"""Suite driver, host side: the command matrix and the trace statistics.
+
+The statistics restate scripts/analyze_test_suite.py:103-161 and are checked on traces whose
+answers are known by construction, and on rows in the reference's own nsys export format.
+"""
+import os
+
+import numpy as np
+import pytest
+import yaml
+
+from bfuse_project_amd import suite
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture
+def info(tmp_path):
+    p = tmp_path / "info.yaml"
+    p.write_text(yaml.safe_dump({"FusionSet": [{"Set": ["a0", "a1", "a2"]}, {"Set": ["b0", "b1", "b2", "b3"]}],
+                                 "KernelInfo": {"a0": [1, 2, 3]}}))
+    return suite.load_info(str(p))
+
+
+def test_info_must_have_two_sets(tmp_path):
+    p = tmp_path / "bad.yaml"
+    p.write_text(yaml.safe_dump({"FusionSet": [{"Set": ["a"]}]}))
+    with pytest.raises(ValueError, match="only 2"):
+        suite.load_info(str(p))
+    assert suite.main([str(p)]) == 1
+    p.write_text(yaml.safe_dump({"FusionSet": [{"Set": ["a"]}, {"Set": []}]}))
+    with pytest.raises(ValueError):
+        suite.load_info(str(p))
+
+
+def test_command_matrix_follows_the_reference(info):
+    # kernel1: one per first-set member; kernel2: one per second-set member; the three two-kernel
+    # methods: one per pair (profile_test_suite.py:33-45), upper triangle on request
+    full = suite.exec_commands(info, "/x/benchmark", "/out/exec")
+    assert len(full) == 3 + 4 + 3 * 12
+    tri = suite.exec_commands(info, "/x/benchmark", "/out/exec", triangular=True)
+    assert len(tri) == 3 + 4 + 3 * (4 + 3 + 2)
+    c = full[0]
+    assert c[:2] == ["rocprofv3", "--kernel-trace"] and c[c.index("--") + 1:] == ["/x/benchmark", "-n", "33", "0", "a0", "b0"]
+    assert full[3 + 4][-3:] == ["2", "a0", "b0"] and "-o" in c and c[c.index("-o") + 1] == "0_0_0"
+    last = full[-1]
+    assert last[-3:] == ["4", "a2", "b3"] and last[last.index("-o") + 1] == "4_2_3"
+    v = suite.valid_commands(info, "/x/benchmark")
+    assert all(x[1] == "-v" for x in v) and len(v) == len(full)
+
+
+def test_single_and_parallel_statistics():
+    rows = []
+    t = 0.0
+    for r in range(33):
+        rows.append({"Name": "k", "Start": t, "Duration": 100.0 + r})       # 100..132
+        rows.append({"Name": "other", "Start": t + 1, "Duration": 5.0})
+        t += 1000
+    mn, mx, mean, std = suite.single_statistics(rows, "k")
+    assert (mn, mx) == (103.0, 132.0) and mean == pytest.approx(np.mean(np.arange(103, 133))) and std == pytest.approx(np.std(np.arange(103, 133)))
+    with pytest.raises(ValueError):
+        suite.single_statistics(rows, "missing")
+    # two kernels per repetition: second ends later -> span; first ends later -> its duration
+    rows, t = [], 0.0
+    for r in range(5):
+        rows.append({"Name": "a", "Start": t, "Duration": 50.0})
+        rows.append({"Name": "b", "Start": t + 10, "Duration": 60.0 if r != 4 else 20.0})
+        t += 500
+    mn, mx, mean, std = suite.parallel_statistics(rows, ["a", "b"], warmup=3)
+    assert (mn, mx) == (50.0, 70.0) and mean == 60.0
+    with pytest.raises(ValueError, match="must be 2"):
+        suite.parallel_statistics(rows, ["a"])
+
+
+def test_trace_formats(tmp_path):
+    own = tmp_path / "0_0_0.csv"
+    suite.write_trace(str(own), [{"Name": "k", "Start": 5.0, "Duration": 7.0}, {"Name": "k", "Start": 1.0, "Duration": 3.0}])
+    assert [r["Start"] for r in suite.read_trace(str(own))] == [1.0, 5.0]
+    roc = tmp_path / "roc_kernel_trace.csv"
+    roc.write_text('"Kind","Agent_Id","Queue_Id","Kernel_Name","Start_Timestamp","End_Timestamp"\n'
+                   '"KERNEL_DISPATCH",1,1,"k",1000,1800\n"KERNEL_DISPATCH",1,1,"k",3000,3900\n')
+    assert [(r["Name"], r["Duration"]) for r in suite.read_trace(str(roc))] == [("k", 800.0), ("k", 900.0)]
+    # the reference's nsys export: memcpy rows have a duration too, kernels are picked by name later
+    nsys = tmp_path / "nsys.csv"
+    nsys.write_text("Start (ns),Duration (ns),CorrId,GrdX,Name\n288325122,257825,241,,[CUDA memcpy Host-to-Device]\n"
+                    "289000000,41000,250,768,dense1_0_dense2_0_fused_bfuse\n")
+    rows = suite.read_trace(str(nsys))
+    assert rows[-1] == {"Name": "dense1_0_dense2_0_fused_bfuse", "Start": 289000000.0, "Duration": 41000.0}
+
+
+def test_analyze_and_tables(tmp_path, info):
+    exec_dir = tmp_path / "exec"
+    exec_dir.mkdir()
+
+    def trace(name, dur, n=33):
+        return [{"Name": name, "Start": 1000.0 * r, "Duration": dur} for r in range(n)]
+    suite.write_trace(str(exec_dir / "0_0_0.csv"), trace("a0", 100.0))
+    suite.write_trace(str(exec_dir / "1_0_1.csv"), trace("b1", 50.0))
+    suite.write_trace(str(exec_dir / "4_0_1.csv"), trace("a0_b1_fused_bfuse_c256", 120.0))
+    suite.write_trace(str(exec_dir / "3_0_1.csv"), trace("a0_b1_fused_hfuse", 125.0))
+    par = []
+    for r in range(33):
+        par += [{"Name": "a0", "Start": 1000.0 * r, "Duration": 100.0}, {"Name": "b1", "Start": 1000.0 * r + 5, "Duration": 50.0}]
+    suite.write_trace(str(exec_dir / "2_0_1.csv"), par)
+    rows = suite.analyze(info, str(exec_dir))
+    assert len(rows) == 1
+    r = rows[0]
+    assert r["serial_ns"] == 150.0 and r["bfuse_speedup"] == pytest.approx(1.25) and r["hfuse_speedup"] == pytest.approx(1.2)
+    assert r["parallel_ns"] == 100.0 and r["bfuse_kernel"] == "a0_b1_fused_bfuse_c256"
+    md = suite.to_markdown(rows)
+    assert "geomean speed-up over serial" in md and "1.25x" in md
+    assert suite.geomean([2.0, 8.0]) == pytest.approx(4.0)
+    assert suite.main([os.path.join(ROOT, "bfuse-project_amd", "examples", "headline_pairs.yaml"), "--commands", "-o", str(tmp_path)]) == 0
