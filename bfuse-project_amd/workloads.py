@@ -102,7 +102,9 @@ def _pair5_inputs():
 PAIRS: Dict[int, Pair] = {
     1: Pair(1, "GEMM fp32 512x512x512 || ReLU(x+b) over 1Mi fp32, hfuse 128/128",
             "gemm_f32_512x512x512", "bias_relu_1048576", "hfuse",
-            [("hfuse", ""), ("bfuse", ""), ("bfuse", "_c8")], [], _pair1_inputs,
+            [("hfuse", ""), ("bfuse", ""), ("bfuse", "_c8")],
+            [("gemm_f32_512x512x512_k4", "bias_relu_1048576", "hfuse", ""),
+             ("gemm_f32_512x512x512_k8", "bias_relu_1048576", "hfuse", "")], _pair1_inputs,
             bytes1=3 * 512 * 512 * 4, bytes2=3 * 1048576 * 4, flops=2 * 512 ** 3,
             bound="hbm", peak=8000.0, dtype="f32", tol=1e-5),
     2: Pair(2, "GEMM fp32 [512x768].[768x2304] || LayerNorm [512x768], bfuse",

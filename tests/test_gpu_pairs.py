@@ -93,3 +93,29 @@ def test_wrong_launch_shape_is_rejected():
         # a standalone kernel is not a fused kernel
         with pytest.raises(bf.BfuseError):
             op.run_fuse(op.k[0], I1, F1, I2, F2)
+
+
+def test_pair5_gemm_every_output_element_exact_on_selector_inputs():
+    """The CPU reference covers a strided sample of pair 5's 512 x 14336 GEMM (the whole matrix
+    takes minutes on the host).  Selector inputs cover every element exactly: with two ones per
+    row of A, C[r, n] = bf16(W[n, k1(r)] + W[n, k2(r)]) -- one fp32 add of two bf16 values and one
+    rounding, which numpy reproduces bit for bit -- so every tile, K-step and fragment index of
+    the full-size kernel is checked, for each built implementation of the side."""
+    pair = PAIRS[5]
+    _, W, I2, F2 = pair.inputs()
+    M, K, N = 512, 4096, 14336
+    rng = np.random.default_rng(5)
+    k1 = rng.integers(0, K, M)
+    k2 = (k1 + 1 + rng.integers(0, K - 1, M)) % K
+    A = np.zeros((M, K), np.float32)
+    A[np.arange(M), k1] = 1.0
+    A[np.arange(M), k2] = 1.0
+    Wf = bf.operation.bf16_to_f32(W).reshape(N, K)
+    want = bf.operation.f32_to_bf16((Wf[:, k1] + Wf[:, k2]).T.copy())          # [M, N], RNE like the kernel
+    A16 = bf.operation.f32_to_bf16(A.ravel())
+    for name in sorted({k for (k, _) in fusions(pair)}):
+        _say(f"[pair 5] selector inputs through {name}")
+        with bf.Operation(name, pair.k2) as op:
+            got = op.run_kernel(0, A16, W).reshape(M, N)
+        bad = np.nonzero(got != want)
+        assert bad[0].size == 0, f"{name}: {bad[0].size} wrong elements, first at row {bad[0][0]} col {bad[1][0]}"
