@@ -2,6 +2,7 @@
 // LayerNorm over [512x768] (eps 1e-12).
 #include "fuse.h"
 #include "ops_gemm_f32.h"
+#include "ops_gemm_f32_dma.h"
 #include "ops_rowwise.h"
 
 using namespace bfuse;
@@ -40,3 +41,7 @@ BFUSE_BFUSE_KERNEL(gemm_f32_512x768x2304, GemmQkv, layernorm_512x768, LnBert, _c
 BFUSE_BFUSE_KERNEL(gemm_f32_512x768x2304, GemmQkv, layernorm_512x768, LnBert, _r, bfuse::kRanges, 0, 0)
 // the same pair with its dispatch plan as run-time data and persistent workgroups
 BFUSE_BFUSE_RT_KERNEL(gemm_f32_512x768x2304, GemmQkv, layernorm_512x768_w1, LnBert1)
+// operands staged through per-wave LDS rings by direct-to-LDS loads
+using GemmQkvD = GemmF32Dma<512, 2304, 768, 32, 144, 4>;
+BFUSE_KERNEL(gemm_f32_512x768x2304_d, GemmQkvD, ({{512, 768, 1, 1}, 4}), ({{768, 2304, 1, 1}, 4}), ({{512, 2304, 1, 1}, 4}))
+BFUSE_BFUSE_KERNEL(gemm_f32_512x768x2304_d, GemmQkvD, layernorm_512x768_w1, LnBert1, _r, bfuse::kRanges, 0, 0)

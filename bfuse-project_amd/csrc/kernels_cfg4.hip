@@ -2,6 +2,7 @@
 // block-fused with the MLP up-projection GEMM [512x768].[768x3072] fp32 + tanh-GELU.
 #include "fuse.h"
 #include "ops_gemm_f32.h"
+#include "ops_gemm_f32_dma.h"
 #include "ops_gemm_f32_lds.h"
 #include "ops_rowwise.h"
 
@@ -56,3 +57,7 @@ BFUSE_BFUSE_KERNEL(softmax_causal_12x512x512_b4, Softmax4b, gemm_gelu_f32_512x76
 BFUSE_BFUSE_KERNEL(softmax_causal_12x512x512, Softmax4, gemm_gelu_f32_512x768x3072_l, GemmFcL, _c256, bfuse::kChunked, 256, 1)
 // the same pair with its dispatch plan as run-time data and persistent workgroups
 BFUSE_BFUSE_RT_KERNEL(softmax_causal_12x512x512, Softmax4, gemm_gelu_f32_512x768x3072_l, GemmFcL)
+// split-K with per-wave LDS rings
+using GemmFcD = GemmF32Dma<512, 3072, 768, 64, 96, 4, kEpiGeluTanh>;
+BFUSE_KERNEL(gemm_gelu_f32_512x768x3072_d, GemmFcD, ({{512, 768, 1, 1}, 4}), ({{768, 3072, 1, 1}, 4}), ({{512, 3072, 1, 1}, 4}))
+BFUSE_BFUSE_KERNEL(softmax_causal_12x512x512, Softmax4, gemm_gelu_f32_512x768x3072_d, GemmFcD, _c256, bfuse::kChunked, 256, 1)

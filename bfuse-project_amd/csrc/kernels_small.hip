@@ -9,6 +9,7 @@
 #include "ops_gemm_bf16_ring.h"
 #include "ops_gemm_f32.h"
 #include "ops_gemm_f32_lds.h"
+#include "ops_gemm_f32_dma.h"
 #include "ops_rowwise.h"
 
 using namespace bfuse;
@@ -38,6 +39,10 @@ using NormRopeS = RmsNormRope<6, 8, 128, 2>;
 BFUSE_KERNEL(gemm_f32_64x32x48, GemmS1, ({{64, 32, 1, 1}, 4}), ({{32, 48, 1, 1}, 4}), ({{64, 48, 1, 1}, 4}))
 BFUSE_KERNEL(gemm_gelu_f32_96x128x192, GemmS2, ({{96, 128, 1, 1}, 4}), ({{128, 192, 1, 1}, 4}), ({{96, 192, 1, 1}, 4}))
 BFUSE_KERNEL(gemm_f32_32x256x144, GemmS3, ({{32, 256, 1, 1}, 4}), ({{256, 144, 1, 1}, 4}), ({{32, 144, 1, 1}, 4}))
+using GemmS5 = GemmF32Dma<128, 192, 160, 32, 96, 2>;                       // private LDS rings, two waves split K, ten 8-k stages each
+using GemmS6 = GemmF32Dma<64, 288, 192, 32, 144, 4, kEpiGeluTanh>;         // the 32x144 tile (partial last B load), four waves, GELU
+BFUSE_KERNEL(gemm_f32_128x160x192_d, GemmS5, ({{128, 160, 1, 1}, 4}), ({{160, 192, 1, 1}, 4}), ({{128, 192, 1, 1}, 4}))
+BFUSE_KERNEL(gemm_gelu_f32_64x192x288_d, GemmS6, ({{64, 192, 1, 1}, 4}), ({{192, 288, 1, 1}, 4}), ({{64, 288, 1, 1}, 4}))
 BFUSE_KERNEL(gemm_f32_128x160x192_l, GemmS4, ({{128, 160, 1, 1}, 4}), ({{160, 192, 1, 1}, 4}), ({{128, 192, 1, 1}, 4}))
 BFUSE_KERNEL(bias_relu_4096, BiasReluS, ({{4096, 1, 1, 1}, 4}), ({{4096, 1, 1, 1}, 4}), ({{4096, 1, 1, 1}, 4}))
 BFUSE_KERNEL(layernorm_8x256, LayerNormS, ({{8, 256, 1, 1}, 4}), ({{2, 256, 1, 1}, 4}), ({{8, 256, 1, 1}, 4}))
@@ -79,3 +84,5 @@ BFUSE_BFUSE_RT_KERNEL(conv3x3_f32_32x12x12_32, ConvS2, gemm_gelu_f32_96x128x192,
 BFUSE_BFUSE_RT_KERNEL(layernorm_8x256, LayerNormS, softmax_causal_2x256x256, SoftmaxS)
 BFUSE_BFUSE_RT_KERNEL(gemm_bf16_256x320x1792_d, GemmB3, rmsnorm_rope_bf16_6x1024, NormRopeS)
 BFUSE_BFUSE_RT_KERNEL(gemm_f32_128x160x192_l, GemmS4, bias_relu_4096, BiasReluS)
+BFUSE_HFUSE_KERNEL(gemm_f32_128x160x192_d, GemmS5, bias_relu_4096, BiasReluS)
+BFUSE_BFUSE_KERNEL(gemm_gelu_f32_64x192x288_d, GemmS6, layernorm_8x256, LayerNormS, _c4, bfuse::kChunked, 4, 1)

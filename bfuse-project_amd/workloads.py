@@ -114,7 +114,8 @@ PAIRS: Dict[int, Pair] = {
              ("gemm_f32_512x768x2304", "layernorm_512x768_w1", "bfuse", "_r"),
              ("gemm_f32_512x768x2304", "layernorm_512x768_w2", "hfuse", ""),
              ("gemm_f32_512x768x2304_p3", "layernorm_512x768_w2", "hfuse", ""),
-             ("gemm_f32_512x768x2304_p3", "layernorm_512x768_w2", "bfuse", "_r")], _pair2_inputs,
+             ("gemm_f32_512x768x2304_p3", "layernorm_512x768_w2", "bfuse", "_r"),
+             ("gemm_f32_512x768x2304_d", "layernorm_512x768_w1", "bfuse", "_r")], _pair2_inputs,
             bytes1=(512 * 768 + 768 * 2304 + 512 * 2304) * 4, bytes2=(2 * 512 * 768 + 2 * 768) * 4,
             flops=2 * 512 * 768 * 2304, bound="mfma", peak=157.3, dtype="f32", tol=1e-5),
     3: Pair(3, "conv 3x3 s1 p1 [1,64,56,56]->64 fp32 || max-pool 3x3 s2 p1 [1,64,112,112], zig-zag bfuse",
@@ -140,7 +141,8 @@ PAIRS: Dict[int, Pair] = {
              ("softmax_causal_12x512x512_b4", "gemm_gelu_f32_512x768x3072_l", "bfuse", "_c256"),
              ("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072_l", "bfuse", "_c256"),
              ("softmax_causal_12x512x512_r6", "gemm_gelu_f32_512x768x3072", "hfuse", ""),
-             ("softmax_causal_12x512x512_r6", "gemm_gelu_f32_512x768x3072_t32", "hfuse", "")], _pair4_inputs,
+             ("softmax_causal_12x512x512_r6", "gemm_gelu_f32_512x768x3072_t32", "hfuse", ""),
+             ("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072_d", "bfuse", "_c256")], _pair4_inputs,
             bytes1=2 * 12 * 512 * 512 * 4, bytes2=(512 * 768 + 768 * 3072 + 512 * 3072) * 4,
             flops=2 * 512 * 768 * 3072, bound="mfma", peak=157.3, dtype="f32", tol=1e-5),
     5: Pair(5, "GEMM bf16 [512x4096].[14336x4096]^T (fp32 acc) || RMSNorm+RoPE [512x4096] bf16, bfuse",

@@ -41,6 +41,10 @@ def _cases():
                                 lambda I, F: orf.gemm_f32(I.reshape(32, 256), F.reshape(256, 144)), 1e-5, False),
         "gemm_f32_128x160x192_l": (lambda s: (fill_normal(s, 128 * 160, 0, 1), fill_normal(s + 1, 160 * 192, 0, 0.1)),
                                    lambda I, F: orf.gemm_f32(I.reshape(128, 160), F.reshape(160, 192)), 1e-5, False),
+        "gemm_f32_128x160x192_d": (lambda s: (fill_normal(s, 128 * 160, 0, 1), fill_normal(s + 1, 160 * 192, 0, 0.1)),
+                                   lambda I, F: orf.gemm_f32(I.reshape(128, 160), F.reshape(160, 192)), 1e-5, False),
+        "gemm_gelu_f32_64x192x288_d": (lambda s: (fill_normal(s, 64 * 192, 0, 1), fill_normal(s + 1, 192 * 288, 0, 0.1)),
+                                       lambda I, F: orf.gemm_f32(I.reshape(64, 192), F.reshape(192, 288), epilogue=1), 1e-5, False),
         "bias_relu_4096": (lambda s: (fill_normal(s, 4096, 0, 1), fill_normal(s + 1, 4096, 0, 0.1)),
                            lambda I, F: orf.bias_relu(I, F), 0.0, False),
         "layernorm_8x256": (lambda s: (fill_normal(s, 8 * 256, 0.5, 2), np.concatenate([fill_normal(s + 1, 256, 1, 0.1), fill_normal(s + 2, 256, 0, 0.1)])),
@@ -84,6 +88,8 @@ FUSIONS = [
     ("gemm_bf16_256x192x1792", "rmsnorm_rope_bf16_6x1024", "bfuse", "_c8"),
     ("maxpool3x3s2_f32_4x16x16", "layernorm_8x256", "hfuse", ""),
     ("gemm_f32_128x160x192_l", "bias_relu_4096", "hfuse", ""),
+    ("gemm_f32_128x160x192_d", "bias_relu_4096", "hfuse", ""),
+    ("gemm_gelu_f32_64x192x288_d", "layernorm_8x256", "bfuse", "_c4"),
     ("gemm_bf16_256x320x1792_d", "rmsnorm_rope_bf16_6x1024", "hfuse", ""),
     ("gemm_bf16_256x320x1792_r", "rmsnorm_rope_bf16_6x1024", "hfuse", ""),
 ]
