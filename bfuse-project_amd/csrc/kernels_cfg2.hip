@@ -21,9 +21,6 @@ using LnBert2 = LayerNorm<512, 768, 2, 1>;
 using LnBert1 = LayerNorm<512, 768, 1, 1>;
 BFUSE_KERNEL(layernorm_512x768_w2, LnBert2, ({{512, 768, 1, 1}, 4}), ({{2, 768, 1, 1}, 4}), ({{512, 768, 1, 1}, 4}))
 BFUSE_KERNEL(layernorm_512x768_w1, LnBert1, ({{512, 768, 1, 1}, 4}), ({{2, 768, 1, 1}, 4}), ({{512, 768, 1, 1}, 4}))
-// deeper operand prefetch
-using GemmQkv3 = GemmF32<512, 2304, 768, 32, 144, 4, kEpiNone, 3>;
-BFUSE_KERNEL(gemm_f32_512x768x2304_p3, GemmQkv3, ({{512, 768, 1, 1}, 4}), ({{768, 2304, 1, 1}, 4}), ({{512, 2304, 1, 1}, 4}))
 
 using GemmQkvS0 = GemmF32<512, 2304, 768, 32, 144, 4, kEpiNone, 2, 0>;
 using GemmQkvS0p3 = GemmF32<512, 2304, 768, 32, 144, 4, kEpiNone, 3, 0>;
@@ -32,8 +29,6 @@ BFUSE_KERNEL(gemm_f32_512x768x2304_s0p3, GemmQkvS0p3, ({{512, 768, 1, 1}, 4}), (
 BFUSE_BFUSE_KERNEL(gemm_f32_512x768x2304, GemmQkv, layernorm_512x768_w2, LnBert2, _r, bfuse::kRanges, 0, 0)
 BFUSE_BFUSE_KERNEL(gemm_f32_512x768x2304, GemmQkv, layernorm_512x768_w1, LnBert1, _r, bfuse::kRanges, 0, 0)
 BFUSE_HFUSE_KERNEL(gemm_f32_512x768x2304, GemmQkv, layernorm_512x768_w2, LnBert2)
-BFUSE_HFUSE_KERNEL(gemm_f32_512x768x2304_p3, GemmQkv3, layernorm_512x768_w2, LnBert2)
-BFUSE_BFUSE_KERNEL(gemm_f32_512x768x2304_p3, GemmQkv3, layernorm_512x768_w2, LnBert2, _r, bfuse::kRanges, 0, 0)
 
 BFUSE_BFUSE_KERNEL(gemm_f32_512x768x2304, GemmQkv, layernorm_512x768, LnBert, , bfuse::kZigzag, 1, 1)
 BFUSE_BFUSE_KERNEL(gemm_f32_512x768x2304, GemmQkv, layernorm_512x768, LnBert, _z2, bfuse::kZigzag, 2, 1)
@@ -45,3 +40,6 @@ BFUSE_BFUSE_RT_KERNEL(gemm_f32_512x768x2304, GemmQkv, layernorm_512x768_w1, LnBe
 using GemmQkvD = GemmF32Dma<512, 2304, 768, 32, 144, 4>;
 BFUSE_KERNEL(gemm_f32_512x768x2304_d, GemmQkvD, ({{512, 768, 1, 1}, 4}), ({{768, 2304, 1, 1}, 4}), ({{512, 2304, 1, 1}, 4}))
 BFUSE_BFUSE_KERNEL(gemm_f32_512x768x2304_d, GemmQkvD, layernorm_512x768_w1, LnBert1, _r, bfuse::kRanges, 0, 0)
+using GemmQkvPc = GemmF32Dma<512, 2304, 768, 32, 144, 4, kEpiNone, 3, 1>;   // + one producer wave per k-range
+BFUSE_KERNEL(gemm_f32_512x768x2304_pc, GemmQkvPc, ({{512, 768, 1, 1}, 4}), ({{768, 2304, 1, 1}, 4}), ({{512, 2304, 1, 1}, 4}))
+BFUSE_BFUSE_KERNEL(gemm_f32_512x768x2304_pc, GemmQkvPc, layernorm_512x768_w1, LnBert1, _r, bfuse::kRanges, 0, 0)

@@ -33,6 +33,7 @@ using GemmB3 = GemmBf16NTDma<256, 1792, 320, 128, 224, 3>;             // direct
 using GemmB5 = GemmBf16NTDma<256, 1792, 320, 128, 224, 3, 4, 4, 2>;       // the same with eight waves (uneven load groups per wave)
 using GemmB6 = GemmBf16NTRing<256, 1792, 320, 128, 224, 7, 4, 2>;         // ring of seven 32-k stages, ten K-steps, eight waves
 using GemmB7 = GemmBf16NTRing<256, 1792, 320, 128, 224, 4, 2, 2>;         // ring of four, four waves (four A fragments per wave)
+using GemmB8 = GemmBf16NTDma<256, 1792, 384, 128, 224, 3, 4, 4, 2, 4>;    // eight compute + four producer waves
 using GemmB4 = GemmBf16NTDma<128, 1792, 192, 128, 224, 2>;             // two stages, three K-steps
 using NormRopeS = RmsNormRope<6, 8, 128, 2>;
 
@@ -57,6 +58,7 @@ BFUSE_KERNEL(gemm_bf16_256x320x1792_d, GemmB3, ({{256, 320, 1, 1}, 2}), ({{1792,
 BFUSE_KERNEL(gemm_bf16_256x320x1792_w8, GemmB5, ({{256, 320, 1, 1}, 2}), ({{1792, 320, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
 BFUSE_KERNEL(gemm_bf16_256x320x1792_r, GemmB6, ({{256, 320, 1, 1}, 2}), ({{1792, 320, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
 BFUSE_KERNEL(gemm_bf16_256x320x1792_r4, GemmB7, ({{256, 320, 1, 1}, 2}), ({{1792, 320, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
+BFUSE_KERNEL(gemm_bf16_256x384x1792_p, GemmB8, ({{256, 384, 1, 1}, 2}), ({{1792, 384, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
 BFUSE_KERNEL(gemm_bf16_128x192x1792_d4, GemmB4, ({{128, 192, 1, 1}, 2}), ({{1792, 192, 1, 1}, 2}), ({{128, 1792, 1, 1}, 2}))
 BFUSE_KERNEL(rmsnorm_rope_bf16_6x1024, NormRopeS, ({{6, 1024, 1, 1}, 2}), ({{(int)NormRopeS::F_BYTES, 1, 1, 1}, 1}), ({{6, 1024, 1, 1}, 2}))
 
@@ -76,7 +78,6 @@ BFUSE_BFUSE_KERNEL(layernorm_8x256, LayerNormS, softmax_causal_2x256x256, Softma
 BFUSE_BFUSE_KERNEL(gemm_bf16_256x192x1792, GemmB2, rmsnorm_rope_bf16_6x1024, NormRopeS, _c8, bfuse::kChunked, 8, 1)
 BFUSE_HFUSE_KERNEL(maxpool3x3s2_f32_4x16x16, PoolS, layernorm_8x256, LayerNormS)
 // the direct-to-LDS GEMM under horizontal fusion: its fence-free barrier becomes the LDS-counter one
-BFUSE_HFUSE_KERNEL(gemm_bf16_256x320x1792_d, GemmB3, rmsnorm_rope_bf16_6x1024, NormRopeS)
 BFUSE_HFUSE_KERNEL(gemm_f32_128x160x192_l, GemmS4, bias_relu_4096, BiasReluS)
 BFUSE_HFUSE_KERNEL(gemm_bf16_256x320x1792_r, GemmB6, rmsnorm_rope_bf16_6x1024, NormRopeS)
 // run-time plans / persistent workgroups: equal and unequal workgroup widths, barrier-bearing sides
@@ -86,3 +87,6 @@ BFUSE_BFUSE_RT_KERNEL(gemm_bf16_256x320x1792_d, GemmB3, rmsnorm_rope_bf16_6x1024
 BFUSE_BFUSE_RT_KERNEL(gemm_f32_128x160x192_l, GemmS4, bias_relu_4096, BiasReluS)
 BFUSE_HFUSE_KERNEL(gemm_f32_128x160x192_d, GemmS5, bias_relu_4096, BiasReluS)
 BFUSE_BFUSE_KERNEL(gemm_gelu_f32_64x192x288_d, GemmS6, layernorm_8x256, LayerNormS, _c4, bfuse::kChunked, 4, 1)
+using GemmS7 = GemmF32Dma<64, 288, 192, 32, 144, 4, kEpiGeluTanh, 3, 1>;   // four compute + four producer waves
+BFUSE_KERNEL(gemm_gelu_f32_64x192x288_pc, GemmS7, ({{64, 192, 1, 1}, 4}), ({{192, 288, 1, 1}, 4}), ({{64, 288, 1, 1}, 4}))
+BFUSE_BFUSE_KERNEL(gemm_gelu_f32_64x192x288_pc, GemmS7, layernorm_8x256, LayerNormS, _c4, bfuse::kChunked, 4, 1)

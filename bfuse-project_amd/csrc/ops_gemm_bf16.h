@@ -175,12 +175,20 @@ struct GemmBf16NT {
 // The 4 x 2 layout (eight waves of 32 x BN/2) therefore trades 40 % more LDS operand reads
 // (still under 60 % of the ~250 B/clk the LDS delivers to eight waves) for a 1.5x higher
 // MFMA issue ceiling.
-template <int M_, int N_, int K_, int BM_, int BN_, int NSTG_ = 3, int PD_ = 4, int WGM_ = 2, int WGN_ = 2>
+//
+// Producer waves (PW_ > 0): measured on MI355X, every global load a wave issues -- to VGPRs or
+// direct to LDS -- keeps that wave from issuing anything else for ~110-125 clocks, an LDS read
+// for ~26; a wave that only issues loads leaves an MFMA wave on the same SIMD undisturbed.  With
+// PW_ extra waves the direct-to-LDS loads are issued by them and the WGM_ x WGN_ compute waves
+// issue only LDS reads and MFMAs.  All waves take part in every barrier.
+template <int M_, int N_, int K_, int BM_, int BN_, int NSTG_ = 3, int PD_ = 4, int WGM_ = 2, int WGN_ = 2, int PW_ = 0>
 struct GemmBf16NTDma {
     static constexpr int M = M_, N = N_, K = K_, BM = BM_, BN = BN_, NSTG = NSTG_;
     static constexpr int BK = 64;
-    static constexpr int WGM = WGM_, WGN = WGN_, NWAVES = WGM_ * WGN_;
-    static constexpr int THREADS = 64 * NWAVES;
+    static constexpr int WGM = WGM_, WGN = WGN_, NCOMP = WGM_ * WGN_, PW = PW_;
+    static constexpr int NWAVES = PW_ > 0 ? PW_ : NCOMP;   // waves that issue the global loads
+    static constexpr int THREADS = 64 * (NCOMP + PW_);
+    static constexpr int CTHREADS = 64 * NCOMP;           // compute threads (they also store the tile)
     static constexpr int WM = BM / WGM, WN = BN / WGN;
     static constexpr int TM = WM / 16, TN = WN / 16;
     static constexpr int NKT = K / BK;
@@ -194,8 +202,8 @@ struct GemmBf16NTDma {
     static_assert(M % BM == 0 && N % BN == 0 && K % BK == 0, "tile must divide the problem");
     static_assert(BM % WGM == 0 && BN % WGN == 0 && WM % 16 == 0 && WN % 16 == 0 && BM % 8 == 0 && BN % 8 == 0, "tile shape");
     static_assert(TM == 2 || TM == 4, "the hand-written LDS wait lists two or four A fragments");
-    static_assert(OCHUNKS % THREADS == 0 && NSTG >= 2 && NSTG <= 4 && NKT >= NSTG - 1, "pipeline shape");
-    static_assert(PD_ >= 1 && PD_ < (BK / 32) * (BN / 32), "read-ahead distance");
+    static_assert(OCHUNKS % CTHREADS == 0 && NSTG >= 2 && NSTG <= 4 && NKT >= NSTG - 1, "pipeline shape");
+    static_assert(PD_ >= 1 && PD_ < (BK / 32) * (BN / WGN_ / 16), "read-ahead distance");
     static constexpr int MT = M / BM, NT = N / BN;
     static_assert((MT * NT) % 8 == 0 && NT % 8 == 0, "tiles are dealt to 8 XCDs");
 
@@ -204,7 +212,7 @@ struct GemmBf16NTDma {
     static constexpr bool HAS_BARRIERS = true;
     static constexpr int EPI_BYTES = BM * CPITCH * 2;
     struct Smem {
-        __attribute__((aligned(1024))) unsigned char t[(NSTG * STAGE_BYTES > EPI_BYTES) ? NSTG * STAGE_BYTES : EPI_BYTES];
+        __attribute__((aligned(1024))) unsigned char t[((NSTG * STAGE_BYTES > EPI_BYTES) ? NSTG * STAGE_BYTES : EPI_BYTES)];
     };
 
     // s_waitcnt vmcnt(n), other counters untouched (gfx9 encoding: vmcnt in bits 3:0 and 15:14)
@@ -271,7 +279,7 @@ struct GemmBf16NTDma {
 #endif
     }
 
-    static constexpr int STEPS = (BK / 32) * TN;
+    static constexpr int STEPS = BK / 32 * TN;
     static constexpr int PD = PD_;      // B fragments are read PD MFMA groups ahead
     static constexpr int RING = PD + 1;
     // reads still allowed in flight when MFMA group `st` starts: the B fragments ahead of it,
@@ -309,10 +317,9 @@ struct GemmBf16NTDma {
     }
 
     // one K-step out of LDS stage U
+    // the loading half of a K-step: wait for own loads of step kt, meet, refill the stage step kt-1 used
     template <int U, class Sync>
-    __device__ static __forceinline__ void k_step(int kt, f32x4 (&acc)[TM][TN], const int (&a_ad)[BK / 32][TM],
-                                                  const int (&b_ad)[BK / 32][TN], const unsigned short* const (&src)[GPW],
-                                                  lds_u8* lds, bool full, Sync& sync)
+    __device__ static __forceinline__ void load_step(int kt, const unsigned short* const (&src)[GPW], lds_u8* lds, bool full, Sync& sync)
     {
         if (kt >= NKT) return;
         // loads of K-step kt have landed once at most the newer steps' loads are outstanding
@@ -320,6 +327,17 @@ struct GemmBf16NTDma {
         else wait_vm<0>();
         sync.raw();  // everyone's part of step kt is in LDS; everyone is done reading step kt-1
         if (kt + NSTG - 1 < NKT) issue(src, lds, (U + NSTG - 1) % NSTG, kt + NSTG - 1, full);
+    }
+
+    // LOADS: this wave also issues loads (no producer waves); otherwise it only meets the producers
+    template <int U, bool LOADS, class Sync>
+    __device__ static __forceinline__ void k_step(int kt, f32x4 (&acc)[TM][TN], const int (&a_ad)[BK / 32][TM],
+                                                  const int (&b_ad)[BK / 32][TN], const unsigned short* const (&src)[GPW],
+                                                  lds_u8* lds, bool full, Sync& sync)
+    {
+        if (kt >= NKT) return;
+        if constexpr (LOADS) load_step<U>(kt, src, lds, full, sync);
+        else sync.raw();
         constexpr int OFF = U * STAGE_BYTES;
         bf16x8 af[BK / 32][TM], bq[RING];
 #pragma unroll
@@ -340,21 +358,24 @@ struct GemmBf16NTDma {
         const int xcd = vblock & 7, slot = vblock >> 3;
         const int nt = xcd * (NT / 8) + slot / MT, mt = slot % MT;
         const int m0 = mt * BM, n0 = nt * BN;
-        const int wave = tid >> 6, lane = tid & 63;
-        const int wm = wave / WGN, wn = wave % WGN;
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;   // wave-uniform: scalar branches
+        const bool compute = wave < NCOMP;                   // wave-uniform roles
+        const bool loader = PW == 0 || !compute;
+        const int lw = PW == 0 ? wave : (compute ? 0 : wave - NCOMP);   // index among the loading waves
+        const int wm = (compute ? wave : 0) / WGN, wn = (compute ? wave : 0) % WGN;
         const int li = lane & 15, kq = lane >> 4;
-        const bool full = wave < GEXTRA;
+        const bool full = lw < GEXTRA;
 
         // per-lane source of each of this wave's loads (K-step 0); swizzled chunk
         const unsigned short* src[GPW];
 #pragma unroll
         for (int i = 0; i < GPW; ++i) {
-            int row = 8 * (wave + i * NWAVES) + (lane >> 3);
+            int row = 8 * (lw + i * NWAVES) + (lane >> 3);
             if (row >= ROWS) row = ROWS - 1;  // slot not issued (see `full`)
             const int gc = (lane & 7) ^ ((row >> 1) & 7);
             src[i] = (row < BM ? A + (size_t)(m0 + row) * K : Wt + (size_t)(n0 + row - BM) * K) + gc * 8;
         }
-        lds_u8* const lds = (lds_u8*)sm.t + wave * 1024;
+        lds_u8* const lds = (lds_u8*)sm.t + lw * 1024;
 
         f32x4 acc[TM][TN];
 #pragma unroll
@@ -362,8 +383,23 @@ struct GemmBf16NTDma {
 #pragma unroll
             for (int b = 0; b < TN; ++b) acc[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+        if (loader) {
 #pragma unroll
-        for (int s = 0; s < NSTG - 1; ++s) issue(src, lds, s, s, full);
+            for (int s = 0; s < NSTG - 1; ++s) issue(src, lds, s, s, full);
+        }
+        if (PW > 0 && !compute) {
+            // a producer wave's whole K loop: the barriers of the compute waves, in the same order
+#pragma unroll 1
+            for (int kt0 = 0; kt0 < NKT; kt0 += NSTG) {
+                load_step<0>(kt0, src, lds, full, sync);
+                if constexpr (NSTG > 1) load_step<1>(kt0 + 1, src, lds, full, sync);
+                if constexpr (NSTG > 2) load_step<2>(kt0 + 2, src, lds, full, sync);
+                if constexpr (NSTG > 3) load_step<3>(kt0 + 3, src, lds, full, sync);
+            }
+            sync();  // the two barriers of the epilogue
+            sync();
+            return;
+        }
 
         // byte offset inside a stage of every operand fragment this lane reads (K-substep ks,
         // block a / b), with the chunk swizzle folded in: loop invariant
@@ -393,31 +429,39 @@ struct GemmBf16NTDma {
             for (int b = 0; b < TN; ++b) b_ad[ks][b] = b_rd[ks][b] + (int)lds_base;
         }
 
-        // K-steps are taken NSTG at a time so that the LDS stage of each is a compile-time constant
+        // K-steps are taken NSTG at a time so that the LDS stage of each is a compile-time constant;
+        // the loop stays rolled whatever K is: operand registers with reads in flight must never be
+        // spilled (the compiler takes an asm output for written when the asm is issued), and a
+        // fully unrolled short loop is where the register allocator runs out
+#pragma unroll 1
         for (int kt0 = 0; kt0 < NKT; kt0 += NSTG) {
-            k_step<0>(kt0, acc, a_ad, b_ad, src, lds, full, sync);
-            if constexpr (NSTG > 1) k_step<1>(kt0 + 1, acc, a_ad, b_ad, src, lds, full, sync);
-            if constexpr (NSTG > 2) k_step<2>(kt0 + 2, acc, a_ad, b_ad, src, lds, full, sync);
-            if constexpr (NSTG > 3) k_step<3>(kt0 + 3, acc, a_ad, b_ad, src, lds, full, sync);
+            k_step<0, PW == 0>(kt0, acc, a_ad, b_ad, src, lds, full, sync);
+            if constexpr (NSTG > 1) k_step<1, PW == 0>(kt0 + 1, acc, a_ad, b_ad, src, lds, full, sync);
+            if constexpr (NSTG > 2) k_step<2, PW == 0>(kt0 + 2, acc, a_ad, b_ad, src, lds, full, sync);
+            if constexpr (NSTG > 3) k_step<3, PW == 0>(kt0 + 3, acc, a_ad, b_ad, src, lds, full, sync);
         }
         sync();  // all waves are done reading the last stage before the tile buffer overwrites it
 
         unsigned short* ct = reinterpret_cast<unsigned short*>(sm.t);
+        if (compute) {
 #pragma unroll
-        for (int a = 0; a < TM; ++a)
+            for (int a = 0; a < TM; ++a)
 #pragma unroll
-            for (int b = 0; b < TN; ++b)
+                for (int b = 0; b < TN; ++b)
 #pragma unroll
-                for (int v = 0; v < 4; ++v)
-                    ct[(wm * WM + a * 16 + 4 * kq + v) * CPITCH + wn * WN + b * 16 + li] =
-                        (unsigned short)f32_to_bf16_bits(acc[a][b][v]);
+                    for (int v = 0; v < 4; ++v)
+                        ct[(wm * WM + a * 16 + 4 * kq + v) * CPITCH + wn * WN + b * 16 + li] =
+                            (unsigned short)f32_to_bf16_bits(acc[a][b][v]);
+        }
         sync();
+        if (compute) {
 #pragma unroll
-        for (int i = 0; i < OCHUNKS / THREADS; ++i) {
-            const int c = tid + i * THREADS;
-            const int row = c / (BN / 8), col = (c % (BN / 8)) * 8;
-            *reinterpret_cast<u32x4*>(C + (size_t)(m0 + row) * N + n0 + col) =
-                *reinterpret_cast<const u32x4*>(ct + row * CPITCH + col);
+            for (int i = 0; i < OCHUNKS / CTHREADS; ++i) {
+                const int c = tid + i * CTHREADS;
+                const int row = c / (BN / 8), col = (c % (BN / 8)) * 8;
+                *reinterpret_cast<u32x4*>(C + (size_t)(m0 + row) * N + n0 + col) =
+                    *reinterpret_cast<const u32x4*>(ct + row * CPITCH + col);
+            }
         }
     }
 };

@@ -250,6 +250,7 @@ struct GemmBf16NTRing {
         __builtin_amdgcn_sched_barrier(0);
 
         int cur = 0;
+#pragma unroll 1   // stays rolled: registers with reads in flight must never be spilled
         for (int kt = 0; kt < NKT; kt += 2) {
             int nxt = cur + STAGE_BYTES;
             if (nxt == NSTG * STAGE_BYTES) nxt = 0;

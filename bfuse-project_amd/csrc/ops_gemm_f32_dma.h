@@ -32,7 +32,12 @@ namespace bfuse {
 
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 
-template <int M_, int N_, int K_, int BM_, int BN_, int KS_, int EPI_ = kEpiNone, int NSTG_ = 3>
+//
+// PW_ = 1 adds one producer wave per k-range: it issues that range's direct-to-LDS loads and the
+// compute wave issues only LDS reads and MFMAs (a global load costs the issuing wave ~110 clocks
+// in which it cannot issue an MFMA; a wave that only loads does not disturb an MFMA wave on the
+// same SIMD).  Producer and compute waves meet at one workgroup barrier per K-stage.
+template <int M_, int N_, int K_, int BM_, int BN_, int KS_, int EPI_ = kEpiNone, int NSTG_ = 3, int PW_ = 0>
 struct GemmF32Dma {
     static constexpr int M = M_, N = N_, K = K_, BM = BM_, BN = BN_, KS = KS_, EPI = EPI_, NSTG = NSTG_;
     static constexpr int TM = BM / 16;
@@ -54,11 +59,14 @@ struct GemmF32Dma {
     static_assert(BM % 32 == 0 && BN % 16 == 0 && N % 4 == 0 && K % 4 == 0, "shape/tile mismatch");   // A stage = whole loads
     static_assert(NSTG >= 2 && NSTAGE >= NSTG && NSTAGE % 2 == 0, "pipeline shape");
     static_assert((NSTG - 1) * LPS <= 63, "vmcnt range");
+    static_assert(!(PW_ && KS_ == 1), "producer waves go with a K split");
 
     static constexpr Dims3 GRID{N / BN, M / BM, 1};
-    static constexpr Dims3 BLOCK{64 * KS, 1, 1};
-    static constexpr int THREADS = 64 * KS;
-    static constexpr bool HAS_BARRIERS = KS > 1;
+    static constexpr int PW = PW_;
+    static constexpr int NW = KS * (1 + PW_);   // waves in the workgroup
+    static constexpr Dims3 BLOCK{64 * NW, 1, 1};
+    static constexpr int THREADS = 64 * NW;
+    static constexpr bool HAS_BARRIERS = NW > 1;
     static constexpr int NUNIT = TM * (G4 + G1);
     static constexpr int RING_BYTES = KS * WAVE_BYTES;
     static constexpr int PART_BYTES = KS > 1 ? KS * TM * NB * 64 * 16 : 16;
@@ -169,9 +177,9 @@ struct GemmF32Dma {
     __device__ static __forceinline__ void mem_op(int s, int slot, int next_off, Frag& nxt, const Ctx& c)
     {
         if constexpr (OP < LPS) {
-            if constexpr (REFILL) issue_one<OP>(c, slot, s + NSTG);
+            if constexpr (REFILL && !PW) issue_one<OP>(c, slot, s + NSTG);
         } else if constexpr (OP == LPS) {
-            if constexpr (NEXT) {
+            if constexpr (NEXT && !PW) {
                 if constexpr (REFILL) wait_vm<(NSTG - 1) * LPS>();
                 else wait_vm<0>();
             }
@@ -209,11 +217,15 @@ struct GemmF32Dma {
 
     // one K-stage: fragments of stage s are in `cur`; refill its slot with stage s+NSTG, read
     // stage s+1 into `nxt`, multiply -- the memory operations dealt between the MFMA groups
-    __device__ static __forceinline__ void step(int s, int& slot, f32x4 (&acc)[TM][NB], Frag& cur, Frag& nxt, const Ctx& c)
+    template <class Sync>
+    __device__ static __forceinline__ void step(int s, int& slot, f32x4 (&acc)[TM][NB], Frag& cur, Frag& nxt, const Ctx& c, Sync& sync)
     {
         int next_slot = slot + 1;
         if (next_slot == NSTG) next_slot = 0;
         const int next_off = next_slot * STAGE_BYTES;
+        // barrier of stage s (producer mode): stage s+1 is in LDS (the producers waited for it)
+        // and every compute wave holds stage s in registers, so its slot can be refilled
+        if constexpr (PW) sync.raw();
         if (s + NSTG < NSTAGE) groups<0, true, true>(s, slot, next_off, acc, cur, nxt, c);
         else if (s + 1 < NSTAGE) groups<0, false, true>(s, slot, next_off, acc, cur, nxt, c);
         else groups<0, false, false>(s, slot, next_off, acc, cur, nxt, c);
@@ -238,10 +250,12 @@ struct GemmF32Dma {
         const int m0 = vb.y * BM, n0 = vb.x * BN;
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
         const int li = lane & 15, kq = lane >> 4;
-        const int kbeg = wave * KW;
+        const bool producer = PW && wave >= KS;
+        const int part = wave < KS ? wave : wave - KS;        // k-range this wave computes or loads
+        const int kbeg = part * KW;
 
         Ctx c;
-        c.ring = (lds_u8*)sm.t + wave * WAVE_BYTES;
+        c.ring = (lds_u8*)sm.t + part * WAVE_BYTES;
         // A slot: [BM][8] floats; a wave-level load covers 32 rows (two lanes per 32-byte row)
 #pragma unroll
         for (int i = 0; i < A_LOADS; ++i)
@@ -274,17 +288,40 @@ struct GemmF32Dma {
             for (int b = 0; b < NB; ++b) acc[tm][b] = f32x4{0.f, 0.f, 0.f, 0.f};
 
         // stages 0 .. NSTG-1 go out; stage 0's fragments are read before the loop
+        if (producer) {
+            // the producer's whole K loop: same barriers as the compute waves, in the same order
 #pragma unroll
-        for (int s = 0; s < NSTG; ++s) issue_all<0>(c, s, s);
-        wait_vm<(NSTG - 1) * LPS>();
-        Frag f0, f1;
-        read_stage(f0, c, 0);
-        wait_reads(f0);
-
-        int slot = 0;
-        for (int s = 0; s < NSTAGE; s += 2) {
-            step(s, slot, acc, f0, f1, c);
-            step(s + 1, slot, acc, f1, f0, c);
+            for (int s = 0; s < NSTG; ++s) issue_all<0>(c, s, s);
+            wait_vm<(NSTG - 1) * LPS>();
+            sync.raw();   // stage 0 is in LDS
+            int slot = 0;
+#pragma unroll 1
+            for (int s = 0; s < NSTAGE; ++s) {
+                if (s + 1 < NSTAGE) {
+                    if (s + NSTG - 1 < NSTAGE) wait_vm<(NSTG - 2) * LPS>();
+                    else wait_vm<0>();
+                }
+                sync.raw();
+                if (s + NSTG < NSTAGE) issue_all<0>(c, slot, s + NSTG);
+                slot = slot + 1 == NSTG ? 0 : slot + 1;
+            }
+        } else {
+            Frag f0, f1;
+            if constexpr (!PW) {
+#pragma unroll
+                for (int s = 0; s < NSTG; ++s) issue_all<0>(c, s, s);
+                wait_vm<(NSTG - 1) * LPS>();
+            } else {
+                sync.raw();   // stage 0 is in LDS
+            }
+            read_stage(f0, c, 0);
+            wait_reads(f0);
+            int slot = 0;
+#pragma unroll 1
+            for (int s = 0; s < NSTAGE; s += 2) {
+                step(s, slot, acc, f0, f1, c, sync);
+                step(s + 1, slot, acc, f1, f0, c, sync);
+            }
         }
 
         if constexpr (KS == 1) {
@@ -303,13 +340,16 @@ struct GemmF32Dma {
             // the barrier below orders the other waves' ring reads before this wave's writes)
             sync();
             f32x4(*part)[TM * NB][64] = reinterpret_cast<f32x4(*)[TM * NB][64]>(sm.t);
+            if (!producer) {
 #pragma unroll
-            for (int tm = 0; tm < TM; ++tm)
+                for (int tm = 0; tm < TM; ++tm)
 #pragma unroll
-                for (int b = 0; b < NB; ++b) part[wave][tm * NB + b][lane] = acc[tm][b];
+                    for (int b = 0; b < NB; ++b) part[wave][tm * NB + b][lane] = acc[tm][b];
+            }
             sync();
+            // every wave of the workgroup, producers included, finishes units
 #pragma unroll
-            for (int u0 = 0; u0 < NUNIT; u0 += KS) {
+            for (int u0 = 0; u0 < NUNIT; u0 += NW) {
                 const int u = u0 + wave;
                 if (u < NUNIT) {
                     const int tm = u / (G4 + G1), g = u % (G4 + G1);

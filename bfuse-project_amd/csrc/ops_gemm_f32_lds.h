@@ -197,6 +197,7 @@ struct GemmF32Lds {
         Frag f[2];
         read_set(f[0], a_rd[0], b_rd[0], 0);
         int stage_off = 0;
+#pragma unroll 1   // stays rolled: registers with reads in flight must never be spilled
         for (int kt = 0; kt < NKT; ++kt) {
 #pragma unroll
             for (int ks = 0; ks < BK / 16; ++ks) {

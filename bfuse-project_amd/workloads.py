@@ -113,9 +113,8 @@ PAIRS: Dict[int, Pair] = {
             [("gemm_f32_512x768x2304", "layernorm_512x768_w2", "bfuse", "_r"),
              ("gemm_f32_512x768x2304", "layernorm_512x768_w1", "bfuse", "_r"),
              ("gemm_f32_512x768x2304", "layernorm_512x768_w2", "hfuse", ""),
-             ("gemm_f32_512x768x2304_p3", "layernorm_512x768_w2", "hfuse", ""),
-             ("gemm_f32_512x768x2304_p3", "layernorm_512x768_w2", "bfuse", "_r"),
-             ("gemm_f32_512x768x2304_d", "layernorm_512x768_w1", "bfuse", "_r")], _pair2_inputs,
+             ("gemm_f32_512x768x2304_d", "layernorm_512x768_w1", "bfuse", "_r"),
+             ("gemm_f32_512x768x2304_pc", "layernorm_512x768_w1", "bfuse", "_r")], _pair2_inputs,
             bytes1=(512 * 768 + 768 * 2304 + 512 * 2304) * 4, bytes2=(2 * 512 * 768 + 2 * 768) * 4,
             flops=2 * 512 * 768 * 2304, bound="mfma", peak=157.3, dtype="f32", tol=1e-5),
     3: Pair(3, "conv 3x3 s1 p1 [1,64,56,56]->64 fp32 || max-pool 3x3 s2 p1 [1,64,112,112], zig-zag bfuse",
@@ -152,7 +151,7 @@ PAIRS: Dict[int, Pair] = {
              ("gemm_bf16_512x4096x14336_v", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
              ("gemm_bf16_512x4096x14336_w8", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
              ("gemm_bf16_512x4096x14336_r", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
-             ("gemm_bf16_512x4096x14336_w8", "rmsnorm_rope_bf16_512x4096_w2", "hfuse", "")], _pair5_inputs,
+             ("gemm_bf16_512x4096x14336_p", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256")], _pair5_inputs,
             bytes1=(512 * 4096 + 4096 * 14336 + 512 * 14336) * 2, bytes2=2 * 512 * 4096 * 2 + 4096 * 2,
             flops=2 * 512 * 4096 * 14336, bound="mfma", peak=2500.0, dtype="bf16", tol=1e-2),
 }
@@ -173,7 +172,7 @@ HEADLINE = {
     2: ("gemm_f32_512x768x2304", "layernorm_512x768_w1", "bfuse", "_r"),
     3: ("conv3x3_f32_64x56x56_64", "maxpool3x3s2_f32_64x112x112", "bfuse", "_c256"),
     4: ("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072_l", "bfuse", "_c256"),
-    5: ("gemm_bf16_512x4096x14336_w8", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
+    5: ("gemm_bf16_512x4096x14336_p", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
 }
 
 
@@ -185,5 +184,5 @@ MEASURED_TRAFFIC = {
     "gemm_f32_512x768x2304_layernorm_512x768_w1_fused_bfuse_r": 28_460_000,
     "conv3x3_f32_64x56x56_64_maxpool3x3s2_f32_64x112x112_fused_bfuse_c256": 11_060_000,
     "softmax_causal_12x512x512_gemm_gelu_f32_512x768x3072_l_fused_bfuse_c256": 47_740_000,
-    "gemm_bf16_512x4096x14336_w8_rmsnorm_rope_bf16_512x4096_fused_bfuse_c256": 174_780_000,
+    "gemm_bf16_512x4096x14336_p_rmsnorm_rope_bf16_512x4096_fused_bfuse_c256": 174_820_000,
 }

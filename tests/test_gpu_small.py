@@ -45,6 +45,8 @@ def _cases():
                                    lambda I, F: orf.gemm_f32(I.reshape(128, 160), F.reshape(160, 192)), 1e-5, False),
         "gemm_gelu_f32_64x192x288_d": (lambda s: (fill_normal(s, 64 * 192, 0, 1), fill_normal(s + 1, 192 * 288, 0, 0.1)),
                                        lambda I, F: orf.gemm_f32(I.reshape(64, 192), F.reshape(192, 288), epilogue=1), 1e-5, False),
+        "gemm_gelu_f32_64x192x288_pc": (lambda s: (fill_normal(s, 64 * 192, 0, 1), fill_normal(s + 1, 192 * 288, 0, 0.1)),
+                                        lambda I, F: orf.gemm_f32(I.reshape(64, 192), F.reshape(192, 288), epilogue=1), 1e-5, False),
         "bias_relu_4096": (lambda s: (fill_normal(s, 4096, 0, 1), fill_normal(s + 1, 4096, 0, 0.1)),
                            lambda I, F: orf.bias_relu(I, F), 0.0, False),
         "layernorm_8x256": (lambda s: (fill_normal(s, 8 * 256, 0.5, 2), np.concatenate([fill_normal(s + 1, 256, 1, 0.1), fill_normal(s + 2, 256, 0, 0.1)])),
@@ -71,6 +73,8 @@ def _cases():
                                      lambda I, F: orf.gemm_bf16(I.reshape(256, 320), F.reshape(1792, 320), b_is_nk=True), 1e-2, True),
         "gemm_bf16_256x320x1792_r4": (lambda s: (f32_to_bf16(fill_normal(s, 256 * 320, 0, 1)), f32_to_bf16(fill_normal(s + 1, 1792 * 320, 0, 0.1))),
                                       lambda I, F: orf.gemm_bf16(I.reshape(256, 320), F.reshape(1792, 320), b_is_nk=True), 1e-2, True),
+        "gemm_bf16_256x384x1792_p": (lambda s: (f32_to_bf16(fill_normal(s, 256 * 384, 0, 1)), f32_to_bf16(fill_normal(s + 1, 1792 * 384, 0, 0.1))),
+                                     lambda I, F: orf.gemm_bf16(I.reshape(256, 384), F.reshape(1792, 384), b_is_nk=True), 1e-2, True),
         "gemm_bf16_128x192x1792_d4": (lambda s: (f32_to_bf16(fill_normal(s, 128 * 192, 0, 1)), f32_to_bf16(fill_normal(s + 1, 1792 * 192, 0, 0.1))),
                                       lambda I, F: orf.gemm_bf16(I.reshape(128, 192), F.reshape(1792, 192), b_is_nk=True), 1e-2, True),
         "rmsnorm_rope_bf16_6x1024": (lambda s: (f32_to_bf16(fill_normal(s, 6 * 1024, 0, 1.5)), _norm_rope_operand(6, 1024, 128, s + 1)),
@@ -90,7 +94,7 @@ FUSIONS = [
     ("gemm_f32_128x160x192_l", "bias_relu_4096", "hfuse", ""),
     ("gemm_f32_128x160x192_d", "bias_relu_4096", "hfuse", ""),
     ("gemm_gelu_f32_64x192x288_d", "layernorm_8x256", "bfuse", "_c4"),
-    ("gemm_bf16_256x320x1792_d", "rmsnorm_rope_bf16_6x1024", "hfuse", ""),
+    ("gemm_gelu_f32_64x192x288_pc", "layernorm_8x256", "bfuse", "_c4"),
     ("gemm_bf16_256x320x1792_r", "rmsnorm_rope_bf16_6x1024", "hfuse", ""),
 ]
 
