@@ -43,3 +43,4 @@ BFUSE_BFUSE_KERNEL(gemm_f32_512x768x2304_d, GemmQkvD, layernorm_512x768_w1, LnBe
 using GemmQkvPc = GemmF32Dma<512, 2304, 768, 32, 144, 4, kEpiNone, 3, 1>;   // + one producer wave per k-range
 BFUSE_KERNEL(gemm_f32_512x768x2304_pc, GemmQkvPc, ({{512, 768, 1, 1}, 4}), ({{768, 2304, 1, 1}, 4}), ({{512, 2304, 1, 1}, 4}))
 BFUSE_BFUSE_KERNEL(gemm_f32_512x768x2304_pc, GemmQkvPc, layernorm_512x768_w1, LnBert1, _r, bfuse::kRanges, 0, 0)
+BFUSE_BFUSE_RT_KERNEL(gemm_f32_512x768x2304_d, GemmQkvD, layernorm_512x768_w1, LnBert1)

@@ -226,13 +226,25 @@ struct GemmBf16NTDma {
 
     // this wave's wave-level loads of K-step kt into LDS stage `stage`: group wave + i * NWAVES
     // (8 rows each); `full` says whether this wave owns a group in the last, partial round
-    __device__ static __forceinline__ void issue(const unsigned short* const (&src)[GPW], lds_u8* wave_base, int stage, int kt, bool full)
+    // Addresses are a wave-uniform base (scalar registers, advanced per K-step by scalar adds) plus a
+    // per-lane 32-bit offset that never changes: a 64-bit vector add per load would cost the SIMD's
+    // MFMA stream ~20 clocks each, whichever wave issues it.
+    struct Src {
+        const char* a_ub;      // A + m0 * K           (bytes)
+        const char* w_ub;      // W + n0 * K
+        unsigned voff[GPW];    // (row within its operand) * K * 2 + swizzled chunk * 16
+        int lw;                // index among the loading waves
+    };
+    __device__ static __forceinline__ void issue(const Src& src, unsigned wave_base, int stage, int kt, bool full)
     {
 #if defined(__HIP_DEVICE_COMPILE__)
 #pragma unroll
         for (int i = 0; i < GPW; ++i)
-            if (i + 1 < GPW || full)
-                __builtin_amdgcn_global_load_lds(src[i] + kt * BK, wave_base + stage * STAGE_BYTES + i * NWAVES * 1024, 16, 0, 0);
+            if (i + 1 < GPW || full) {
+                const bool is_a = 8 * (src.lw + i * NWAVES) < BM;   // wave-uniform: a group of 8 rows is all A or all W
+                const char* ub = (is_a ? src.a_ub : src.w_ub) + (size_t)kt * (BK * 2);
+                dma_load_lds_b128(src.voff[i], ub, wave_base + stage * STAGE_BYTES + i * NWAVES * 1024);
+            }
 #endif
     }
     // "the loads of the K-step that is due have landed": at most `newer` K-steps' loads outstanding
@@ -319,7 +331,7 @@ struct GemmBf16NTDma {
     // one K-step out of LDS stage U
     // the loading half of a K-step: wait for own loads of step kt, meet, refill the stage step kt-1 used
     template <int U, class Sync>
-    __device__ static __forceinline__ void load_step(int kt, const unsigned short* const (&src)[GPW], lds_u8* lds, bool full, Sync& sync)
+    __device__ static __forceinline__ void load_step(int kt, const Src& src, unsigned lds, bool full, Sync& sync)
     {
         if (kt >= NKT) return;
         // loads of K-step kt have landed once at most the newer steps' loads are outstanding
@@ -332,8 +344,8 @@ struct GemmBf16NTDma {
     // LOADS: this wave also issues loads (no producer waves); otherwise it only meets the producers
     template <int U, bool LOADS, class Sync>
     __device__ static __forceinline__ void k_step(int kt, f32x4 (&acc)[TM][TN], const int (&a_ad)[BK / 32][TM],
-                                                  const int (&b_ad)[BK / 32][TN], const unsigned short* const (&src)[GPW],
-                                                  lds_u8* lds, bool full, Sync& sync)
+                                                  const int (&b_ad)[BK / 32][TN], const Src& src,
+                                                  unsigned lds, bool full, Sync& sync)
     {
         if (kt >= NKT) return;
         if constexpr (LOADS) load_step<U>(kt, src, lds, full, sync);
@@ -367,15 +379,19 @@ struct GemmBf16NTDma {
         const bool full = lw < GEXTRA;
 
         // per-lane source of each of this wave's loads (K-step 0); swizzled chunk
-        const unsigned short* src[GPW];
+        Src src;
+        src.a_ub = reinterpret_cast<const char*>(A + (size_t)m0 * K);
+        src.w_ub = reinterpret_cast<const char*>(Wt + (size_t)n0 * K);
+        src.lw = lw;
 #pragma unroll
         for (int i = 0; i < GPW; ++i) {
             int row = 8 * (lw + i * NWAVES) + (lane >> 3);
             if (row >= ROWS) row = ROWS - 1;  // slot not issued (see `full`)
             const int gc = (lane & 7) ^ ((row >> 1) & 7);
-            src[i] = (row < BM ? A + (size_t)(m0 + row) * K : Wt + (size_t)(n0 + row - BM) * K) + gc * 8;
+            src.voff[i] = (unsigned)((row < BM ? row : row - BM) * K + gc * 8) * 2u;
         }
-        lds_u8* const lds = (lds_u8*)sm.t + lw * 1024;
+        // LDS byte address of this wave's first load of stage 0 (wave-uniform)
+        const unsigned lds = (unsigned)(unsigned long long)(lds_u8*)sm.t + (unsigned)lw * 1024u;
 
         f32x4 acc[TM][TN];
 #pragma unroll

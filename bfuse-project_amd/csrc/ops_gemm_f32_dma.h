@@ -57,8 +57,9 @@ struct GemmF32Dma {
     static constexpr int WAVE_BYTES = NSTG * STAGE_BYTES;
     static_assert(M % BM == 0 && N % BN == 0 && K % (KS * STAGE) == 0, "tile must divide the problem");
     static_assert(BM % 32 == 0 && BN % 16 == 0 && N % 4 == 0 && K % 4 == 0, "shape/tile mismatch");   // A stage = whole loads
-    static_assert(NSTG >= 2 && NSTAGE >= NSTG && NSTAGE % 2 == 0, "pipeline shape");
+    static_assert(NSTG >= 2 && NSTAGE >= NSTG, "pipeline shape");
     static_assert((NSTG - 1) * LPS <= 63, "vmcnt range");
+    static_assert(NSTG * STAGE_BYTES + BN * 8 + 1024 < 65536, "fragment offsets are 16-bit immediates");
     static_assert(!(PW_ && KS_ == 1), "producer waves go with a K split");
 
     static constexpr Dims3 GRID{N / BN, M / BM, 1};
@@ -69,7 +70,13 @@ struct GemmF32Dma {
     static constexpr bool HAS_BARRIERS = NW > 1;
     static constexpr int NUNIT = TM * (G4 + G1);
     static constexpr int RING_BYTES = KS * WAVE_BYTES;
-    static constexpr int PART_BYTES = KS > 1 ? KS * TM * NB * 64 * 16 : 16;
+    // The partial tiles meet in LDS in ROUNDS rounds of TMR row blocks each, so that the reduction
+    // buffer is no larger than the rings it reuses: the static LDS size decides whether a second
+    // workgroup (of either side of a fused kernel) fits on the CU.
+    static constexpr int FULL_PART_BYTES = KS * TM * NB * 64 * 16;
+    static constexpr int ROUNDS = (KS > 1 && FULL_PART_BYTES > RING_BYTES && TM % 2 == 0) ? 2 : 1;
+    static constexpr int TMR = TM / ROUNDS;
+    static constexpr int PART_BYTES = KS > 1 ? KS * TMR * NB * 64 * 16 : 16;
 
     struct Smem {
         __attribute__((aligned(1024))) unsigned char t[RING_BYTES > PART_BYTES ? RING_BYTES : PART_BYTES];
@@ -88,10 +95,15 @@ struct GemmF32Dma {
         float b1[G1 > 0 ? G1 : 1][2];
     };
     struct Ctx {
-        const float* a_src[A_LOADS];   // this lane's source of every A load of stage 0
-        const float* b_src[B_LOADS];
-        lds_u8* ring;                  // this wave's ring
-        int a_rd[TM], b4_rd[G4 > 0 ? G4 : 1][2], b1_rd[G1 > 0 ? G1 : 1][2];   // LDS byte addresses in slot 0
+        // sources: a wave-uniform base (scalar registers) plus this lane's constant byte offset
+        const char* a_ub;              // A + m0 * K + kbeg
+        const char* b_ub;              // B + kbeg * N + n0
+        unsigned a_voff[A_LOADS], b_voff[B_LOADS];
+        unsigned ring;                 // LDS byte address of this wave's ring (wave-uniform)
+        // LDS byte address of this lane's part of each operand in slot 0; every fragment is a
+        // compile-time offset from one of them (an address computed between MFMAs costs the
+        // wave ~20 clocks of MFMA issue, an immediate offset nothing)
+        int a_base, b4_base, b1_base;
     };
 
     // ---- one memory operation at a time, so that they can be dealt between the MFMAs ----------
@@ -103,15 +115,13 @@ struct GemmF32Dma {
     template <int I>
     __device__ static __forceinline__ void issue_one(const Ctx& c, int slot, int s)
     {
-#if defined(__HIP_DEVICE_COMPILE__)
-        lds_u8* dst = c.ring + slot * STAGE_BYTES;
+        const unsigned dst = c.ring + slot * STAGE_BYTES;   // `slot` is a constant wherever a compute wave calls this
         if constexpr (I < A_LOADS) {
-            __builtin_amdgcn_global_load_lds(c.a_src[I] + s * STAGE, dst + I * 1024, 16, 0, 0);
+            dma_load_lds_b128(c.a_voff[I], c.a_ub + (size_t)s * (STAGE * 4), dst + I * 1024);
         } else {
             constexpr int J = I - A_LOADS;
-            __builtin_amdgcn_global_load_lds(c.b_src[J] + (size_t)s * STAGE * N, dst + A_BYTES + J * 1024, 16, 0, 0);
+            dma_load_lds_b128(c.b_voff[J], c.b_ub + (size_t)s * (STAGE * N * 4), dst + A_BYTES + J * 1024);
         }
-#endif
     }
     template <int I>
     __device__ static __forceinline__ void issue_all(const Ctx& c, int slot, int s)
@@ -121,31 +131,28 @@ struct GemmF32Dma {
             issue_all<I + 1>(c, slot, s);
         }
     }
-    template <int J>
-    __device__ static __forceinline__ void read_one(Frag& f, const Ctx& c, int off)
+    template <int J, int SLOT>
+    __device__ static __forceinline__ void read_one(Frag& f, const Ctx& c)
     {
 #if defined(__HIP_DEVICE_COMPILE__)
+        constexpr int S0 = SLOT * STAGE_BYTES;
         if constexpr (J < TM) {
-            asm volatile("ds_read_b64 %0, %1" : "=v"(f.a[J]) : "v"(c.a_rd[J] + off));
+            asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(f.a[J]) : "v"(c.a_base), "n"(S0 + J * 16 * 32));
         } else if constexpr (J < TM + 2 * G4) {
             constexpr int g = (J - TM) / 2, t = (J - TM) % 2;
-            asm volatile("ds_read_b128 %0, %1" : "=v"(f.b4[g][t]) : "v"(c.b4_rd[g][t] + off));
+            asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(f.b4[g][t]) : "v"(c.b4_base), "n"(S0 + (t * BN + g * 64) * 4));
         } else {
             constexpr int g = (J - TM - 2 * G4) / 2, t = (J - TM - 2 * G4) % 2;
-            asm volatile("ds_read_b32 %0, %1" : "=v"(f.b1[g][t]) : "v"(c.b1_rd[g][t] + off));
+            asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(f.b1[g][t]) : "v"(c.b1_base), "n"(S0 + (t * BN + G4 * 64 + g * 16) * 4));
         }
 #endif
     }
-    __device__ static __forceinline__ void read_stage(Frag& f, const Ctx& c, int off)
-    {
-        read_all<0>(f, c, off);
-    }
-    template <int J>
-    __device__ static __forceinline__ void read_all(Frag& f, const Ctx& c, int off)
+    template <int SLOT, int J = 0>
+    __device__ static __forceinline__ void read_stage(Frag& f, const Ctx& c)
     {
         if constexpr (J < NREADS) {
-            read_one<J>(f, c, off);
-            read_all<J + 1>(f, c, off);
+            read_one<J, SLOT>(f, c);
+            read_stage<SLOT, J + 1>(f, c);
         }
     }
     // all LDS reads of this wave have landed; every fragment register is named so that the
@@ -173,32 +180,32 @@ struct GemmF32Dma {
     // then the reads of stage s+1
     // REFILL: stage s+NSTG exists; NEXT: stage s+1 exists.  Compile-time, so that a step's body
     // has no branch in it.
-    template <int OP, bool REFILL, bool NEXT>
-    __device__ static __forceinline__ void mem_op(int s, int slot, int next_off, Frag& nxt, const Ctx& c)
+    template <int OP, int SLOT, bool REFILL, bool NEXT>
+    __device__ static __forceinline__ void mem_op(int s, Frag& nxt, const Ctx& c)
     {
         if constexpr (OP < LPS) {
-            if constexpr (REFILL && !PW) issue_one<OP>(c, slot, s + NSTG);
+            if constexpr (REFILL && !PW) issue_one<OP>(c, SLOT, s + NSTG);
         } else if constexpr (OP == LPS) {
             if constexpr (NEXT && !PW) {
                 if constexpr (REFILL) wait_vm<(NSTG - 1) * LPS>();
                 else wait_vm<0>();
             }
         } else if constexpr (OP < NOPS) {
-            if constexpr (NEXT) read_one<OP - LPS - 1>(nxt, c, next_off);
+            if constexpr (NEXT) read_one<OP - LPS - 1, (SLOT + 1) % NSTG>(nxt, c);
         }
     }
-    template <int G, int K0, bool REFILL, bool NEXT>
-    __device__ static __forceinline__ void mem_ops(int s, int slot, int next_off, Frag& nxt, const Ctx& c)
+    template <int G, int K0, int SLOT, bool REFILL, bool NEXT>
+    __device__ static __forceinline__ void mem_ops(int s, Frag& nxt, const Ctx& c)
     {
         if constexpr (K0 < OPS_PER_GROUP) {
-            mem_op<G * OPS_PER_GROUP + K0, REFILL, NEXT>(s, slot, next_off, nxt, c);
-            mem_ops<G, K0 + 1, REFILL, NEXT>(s, slot, next_off, nxt, c);
+            mem_op<G * OPS_PER_GROUP + K0, SLOT, REFILL, NEXT>(s, nxt, c);
+            mem_ops<G, K0 + 1, SLOT, REFILL, NEXT>(s, nxt, c);
         }
     }
 
     // MFMA group G of a stage, then its share of the memory operations
-    template <int G, bool REFILL, bool NEXT>
-    __device__ static __forceinline__ void groups(int s, int slot, int next_off, f32x4 (&acc)[TM][NB], const Frag& cur, Frag& nxt, const Ctx& c)
+    template <int G, int SLOT, bool REFILL, bool NEXT>
+    __device__ static __forceinline__ void groups(int s, f32x4 (&acc)[TM][NB], const Frag& cur, Frag& nxt, const Ctx& c)
     {
         if constexpr (G < NGROUPS) {
             constexpr int t = G / (TM * (G4 + G1)), tm = (G / (G4 + G1)) % TM, g = G % (G4 + G1);
@@ -209,28 +216,47 @@ struct GemmF32Dma {
             } else {
                 acc[tm][4 * G4 + g - G4] = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.a[tm][t], cur.b1[g - G4][t], acc[tm][4 * G4 + g - G4], 0, 0, 0);
             }
-            mem_ops<G, 0, REFILL, NEXT>(s, slot, next_off, nxt, c);
+            mem_ops<G, 0, SLOT, REFILL, NEXT>(s, nxt, c);
             __builtin_amdgcn_sched_barrier(0);
-            groups<G + 1, REFILL, NEXT>(s, slot, next_off, acc, cur, nxt, c);
+            groups<G + 1, SLOT, REFILL, NEXT>(s, acc, cur, nxt, c);
         }
     }
 
-    // one K-stage: fragments of stage s are in `cur`; refill its slot with stage s+NSTG, read
-    // stage s+1 into `nxt`, multiply -- the memory operations dealt between the MFMA groups
-    template <class Sync>
-    __device__ static __forceinline__ void step(int s, int& slot, f32x4 (&acc)[TM][NB], Frag& cur, Frag& nxt, const Ctx& c, Sync& sync)
+    // one K-stage out of ring slot SLOT: its fragments are in `cur`; refill the slot with stage
+    // s+NSTG (REFILL: that stage exists), read stage s+1 into `nxt` (NEXT), multiply -- the
+    // memory operations dealt between the MFMA groups.  Slot and both flags are compile-time: the
+    // body has no branch and no address arithmetic in it.
+    template <int SLOT, bool REFILL, bool NEXT, class Sync>
+    __device__ static __forceinline__ void step(int s, f32x4 (&acc)[TM][NB], Frag& cur, Frag& nxt, const Ctx& c, Sync& sync)
     {
-        int next_slot = slot + 1;
-        if (next_slot == NSTG) next_slot = 0;
-        const int next_off = next_slot * STAGE_BYTES;
         // barrier of stage s (producer mode): stage s+1 is in LDS (the producers waited for it)
         // and every compute wave holds stage s in registers, so its slot can be refilled
         if constexpr (PW) sync.raw();
-        if (s + NSTG < NSTAGE) groups<0, true, true>(s, slot, next_off, acc, cur, nxt, c);
-        else if (s + 1 < NSTAGE) groups<0, false, true>(s, slot, next_off, acc, cur, nxt, c);
-        else groups<0, false, false>(s, slot, next_off, acc, cur, nxt, c);
+        groups<0, SLOT, REFILL, NEXT>(s, acc, cur, nxt, c);
         wait_reads(nxt);
-        slot = next_slot;
+    }
+
+    // The fragment buffers alternate (period 2) and the ring slots rotate (period NSTG): UNR stages
+    // bring both back to where they started.
+    static constexpr int UNR = NSTG % 2 == 0 ? NSTG : 2 * NSTG;
+    static constexpr int MAIN = NSTAGE > NSTG ? ((NSTAGE - NSTG) / UNR) * UNR : 0;   // stages in the rolled loop: all refill
+    template <int J, class Sync>
+    __device__ static __forceinline__ void main_chain(int s0, f32x4 (&acc)[TM][NB], Frag& f0, Frag& f1, const Ctx& c, Sync& sync)
+    {
+        if constexpr (J < UNR) {
+            if constexpr (J % 2 == 0) step<J % NSTG, true, true>(s0 + J, acc, f0, f1, c, sync);
+            else step<J % NSTG, true, true>(s0 + J, acc, f1, f0, c, sync);
+            main_chain<J + 1>(s0, acc, f0, f1, c, sync);
+        }
+    }
+    template <int S, class Sync>
+    __device__ static __forceinline__ void tail_chain(f32x4 (&acc)[TM][NB], Frag& f0, Frag& f1, const Ctx& c, Sync& sync)
+    {
+        if constexpr (S < NSTAGE) {
+            if constexpr (S % 2 == 0) step<S % NSTG, (S + NSTG < NSTAGE), (S + 1 < NSTAGE)>(S, acc, f0, f1, c, sync);
+            else step<S % NSTG, (S + NSTG < NSTAGE), (S + 1 < NSTAGE)>(S, acc, f1, f0, c, sync);
+            tail_chain<S + 1>(acc, f0, f1, c, sync);
+        }
     }
 
     __device__ static __forceinline__ float epilogue(float v)
@@ -255,11 +281,13 @@ struct GemmF32Dma {
         const int kbeg = part * KW;
 
         Ctx c;
-        c.ring = (lds_u8*)sm.t + part * WAVE_BYTES;
+        c.ring = (unsigned)(unsigned long long)(lds_u8*)sm.t + (unsigned)part * WAVE_BYTES;
+        c.a_ub = reinterpret_cast<const char*>(A + (size_t)m0 * K + kbeg);
+        c.b_ub = reinterpret_cast<const char*>(B + (size_t)kbeg * N + n0);
         // A slot: [BM][8] floats; a wave-level load covers 32 rows (two lanes per 32-byte row)
 #pragma unroll
         for (int i = 0; i < A_LOADS; ++i)
-            c.a_src[i] = A + (size_t)(m0 + i * 32 + (lane >> 1)) * K + kbeg + (lane & 1) * 4;
+            c.a_voff[i] = (unsigned)((i * 32 + (lane >> 1)) * K + (lane & 1) * 4) * 4u;
         // B slot: [8][BN] floats, 16-byte chunk ch = (row, ch % (BN/4))
 #pragma unroll
         for (int i = 0; i < B_LOADS; ++i) {
@@ -267,19 +295,12 @@ struct GemmF32Dma {
             // the slot's padding (the slot reserves whole loads)
             int ch = i * 64 + lane;
             if (ch >= B_CHUNKS) ch = B_CHUNKS - 1;
-            c.b_src[i] = B + (size_t)(kbeg + ch / (BN / 4)) * N + n0 + (ch % (BN / 4)) * 4;
+            c.b_voff[i] = (unsigned)((ch / (BN / 4)) * N + (ch % (BN / 4)) * 4) * 4u;
         }
-        const int base = (int)(unsigned)(unsigned long long)c.ring;
-#pragma unroll
-        for (int tm = 0; tm < TM; ++tm) c.a_rd[tm] = base + (tm * 16 + li) * 32 + kq * 8;
-#pragma unroll
-        for (int g = 0; g < G4; ++g)
-#pragma unroll
-            for (int t = 0; t < 2; ++t) c.b4_rd[g][t] = base + A_BYTES + ((2 * kq + t) * BN + g * 64 + 4 * li) * 4;
-#pragma unroll
-        for (int g = 0; g < G1; ++g)
-#pragma unroll
-            for (int t = 0; t < 2; ++t) c.b1_rd[g][t] = base + A_BYTES + ((2 * kq + t) * BN + G4 * 64 + g * 16 + li) * 4;
+        const int base = (int)c.ring;
+        c.a_base = base + li * 32 + kq * 8;
+        c.b4_base = base + A_BYTES + (2 * kq * BN + 4 * li) * 4;
+        c.b1_base = base + A_BYTES + (2 * kq * BN + li) * 4;
 
         f32x4 acc[TM][NB];
 #pragma unroll
@@ -314,14 +335,11 @@ struct GemmF32Dma {
             } else {
                 sync.raw();   // stage 0 is in LDS
             }
-            read_stage(f0, c, 0);
+            read_stage<0>(f0, c);
             wait_reads(f0);
-            int slot = 0;
 #pragma unroll 1
-            for (int s = 0; s < NSTAGE; s += 2) {
-                step(s, slot, acc, f0, f1, c, sync);
-                step(s + 1, slot, acc, f1, f0, c, sync);
-            }
+            for (int s0 = 0; s0 < MAIN; s0 += UNR) main_chain<0>(s0, acc, f0, f1, c, sync);
+            tail_chain<MAIN>(acc, f0, f1, c, sync);
         }
 
         if constexpr (KS == 1) {
@@ -338,36 +356,39 @@ struct GemmF32Dma {
         } else {
             // the rings are dead (every wave has consumed its last stage before it gets here, and
             // the barrier below orders the other waves' ring reads before this wave's writes)
-            sync();
-            f32x4(*part)[TM * NB][64] = reinterpret_cast<f32x4(*)[TM * NB][64]>(sm.t);
-            if (!producer) {
+            f32x4(*part)[TMR * NB][64] = reinterpret_cast<f32x4(*)[TMR * NB][64]>(sm.t);
 #pragma unroll
-                for (int tm = 0; tm < TM; ++tm)
+            for (int r = 0; r < ROUNDS; ++r) {
+                sync();   // round 0: rings dead; later rounds: the previous round's sums have been read
+                if (!producer) {
 #pragma unroll
-                    for (int b = 0; b < NB; ++b) part[wave][tm * NB + b][lane] = acc[tm][b];
-            }
-            sync();
-            // every wave of the workgroup, producers included, finishes units
+                    for (int tm = 0; tm < TMR; ++tm)
 #pragma unroll
-            for (int u0 = 0; u0 < NUNIT; u0 += NW) {
-                const int u = u0 + wave;
-                if (u < NUNIT) {
-                    const int tm = u / (G4 + G1), g = u % (G4 + G1);
-                    if (g < G4) {
-                        f32x4 blk[4];
+                        for (int b = 0; b < NB; ++b) part[wave][tm * NB + b][lane] = acc[r * TMR + tm][b];
+                }
+                sync();
+                // every wave of the workgroup, producers included, finishes units
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            f32x4 s = part[0][tm * NB + 4 * g + e][lane];
+                for (int u0 = 0; u0 < NUNIT / ROUNDS; u0 += NW) {
+                    const int u = u0 + wave;
+                    if (u < NUNIT / ROUNDS) {
+                        const int tm = u / (G4 + G1), g = u % (G4 + G1);
+                        if (g < G4) {
+                            f32x4 blk[4];
 #pragma unroll
-                            for (int w = 1; w < KS; ++w) s += part[w][tm * NB + 4 * g + e][lane];
-                            blk[e] = s;
+                            for (int e = 0; e < 4; ++e) {
+                                f32x4 s = part[0][tm * NB + 4 * g + e][lane];
+#pragma unroll
+                                for (int w = 1; w < KS; ++w) s += part[w][tm * NB + 4 * g + e][lane];
+                                blk[e] = s;
+                            }
+                            store_group4(C, m0, n0, r * TMR + tm, g, blk, lane);
+                        } else {
+                            f32x4 s = part[0][tm * NB + 4 * G4 + (g - G4)][lane];
+#pragma unroll
+                            for (int w = 1; w < KS; ++w) s += part[w][tm * NB + 4 * G4 + (g - G4)][lane];
+                            store_group1(C, m0, n0, r * TMR + tm, g - G4, s, lane);
                         }
-                        store_group4(C, m0, n0, tm, g, blk, lane);
-                    } else {
-                        f32x4 s = part[0][tm * NB + 4 * G4 + (g - G4)][lane];
-#pragma unroll
-                        for (int w = 1; w < KS; ++w) s += part[w][tm * NB + 4 * G4 + (g - G4)][lane];
-                        store_group1(C, m0, n0, tm, g - G4, s, lane);
                     }
                 }
             }

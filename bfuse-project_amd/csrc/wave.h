@@ -43,6 +43,24 @@ __device__ __forceinline__ float wave_reduce(float v, Op op)
 __device__ __forceinline__ float wave_sum(float v) { return wave_reduce(v, SumOp{}); }
 __device__ __forceinline__ float wave_max(float v) { return wave_reduce(v, MaxOp{}); }
 
+// ---- direct global -> LDS load with a scalar base ------------------------------------
+// 64 lanes x 16 bytes: lane L fetches base + voff (its own 32-bit byte offset) and the data lands at
+// LDS byte address lds_addr + 16 L.  `base` and `lds_addr` must be wave-uniform (they travel in
+// scalar registers).  Written as asm because the address then costs no vector instruction: the
+// compiler's own selection of this load turns "uniform base + lane offset" into a 64-bit vector add
+// per load whenever the offset was computed outside the loop, and on a SIMD that is streaming MFMAs
+// every vector ALU instruction, from whichever wave, takes ~20 clocks out of that stream.
+// The compiler does not count this load in vmcnt: callers wait with explicit s_waitcnt vmcnt(n).
+__device__ __forceinline__ void dma_load_lds_b128(unsigned voff, const void* base, unsigned lds_addr)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(voff), "s"(base), "s"(lds_addr)
+                 : "memory", "m0");
+#endif
+}
+
 // ---- synchronisation policies ---------------------------------------------------------
 // Counts waits that gave up (see GroupSync); read back by the host after a fused launch.
 static __device__ unsigned int g_sync_timeouts;

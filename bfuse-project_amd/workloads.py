@@ -141,7 +141,11 @@ PAIRS: Dict[int, Pair] = {
              ("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072_l", "bfuse", "_c256"),
              ("softmax_causal_12x512x512_r6", "gemm_gelu_f32_512x768x3072", "hfuse", ""),
              ("softmax_causal_12x512x512_r6", "gemm_gelu_f32_512x768x3072_t32", "hfuse", ""),
-             ("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072_d", "bfuse", "_c256")], _pair4_inputs,
+             ("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072_d", "bfuse", "_c256"),
+             ("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072_dh", "bfuse", "_c256"),
+             ("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072_dh", "bfuse", "_c512"),
+             ("softmax_causal_12x512x512_b4", "gemm_gelu_f32_512x768x3072_dh", "bfuse", "_c256"),
+             ("softmax_causal_12x512x512_r3", "gemm_gelu_f32_512x768x3072_dh", "hfuse", "")], _pair4_inputs,
             bytes1=2 * 12 * 512 * 512 * 4, bytes2=(512 * 768 + 768 * 3072 + 512 * 3072) * 4,
             flops=2 * 512 * 768 * 3072, bound="mfma", peak=157.3, dtype="f32", tol=1e-5),
     5: Pair(5, "GEMM bf16 [512x4096].[14336x4096]^T (fp32 acc) || RMSNorm+RoPE [512x4096] bf16, bfuse",
@@ -169,9 +173,9 @@ def fusions(pair: Pair):
 # headline fused variant of each pair: (k1, k2, kind, suffix)
 HEADLINE = {
     1: ("gemm_f32_512x512x512", "bias_relu_1048576", "hfuse", ""),
-    2: ("gemm_f32_512x768x2304", "layernorm_512x768_w1", "bfuse", "_r"),
+    2: ("gemm_f32_512x768x2304_d", "layernorm_512x768_w1", "bfuse", "_r"),
     3: ("conv3x3_f32_64x56x56_64", "maxpool3x3s2_f32_64x112x112", "bfuse", "_c256"),
-    4: ("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072_l", "bfuse", "_c256"),
+    4: ("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072_dh", "bfuse", "_c256"),
     5: ("gemm_bf16_512x4096x14336_p", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
 }
 
