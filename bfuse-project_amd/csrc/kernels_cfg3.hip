@@ -2,6 +2,7 @@
 // zig-zag block-fused with a 3x3 stride-2 max-pool on [1,64,112,112].
 #include "fuse.h"
 #include "ops_conv.h"
+#include "ops_conv_lds.h"
 
 using namespace bfuse;
 
@@ -24,3 +25,8 @@ BFUSE_BFUSE_KERNEL(conv3x3_f32_64x56x56_64_h, Conv32, maxpool3x3s2_f32_64x112x11
 BFUSE_BFUSE_KERNEL(conv3x3_f32_64x56x56_64_h, Conv32, maxpool3x3s2_f32_64x112x112, Pool, _c8, bfuse::kChunked, 8, 1)
 // the same pair with its dispatch plan as run-time data and persistent workgroups
 BFUSE_BFUSE_RT_KERNEL(conv3x3_f32_64x56x56_64, Conv64, maxpool3x3s2_f32_64x112x112, Pool)
+// the image patch staged in per-wave LDS tiles: one 128-bit LDS read per tap and pixel block in the loop
+using Conv64L = Conv3x3F32Lds<64, 64, 56, 56, 16, 4, 4>;    // 196 workgroups, 74 KB
+BFUSE_KERNEL(conv3x3_f32_64x56x56_64_l, Conv64L, ({{1, 64, 56, 56}, 4}), ({{64, 64, 3, 3}, 4}), ({{1, 64, 56, 56}, 4}))
+BFUSE_BFUSE_KERNEL(conv3x3_f32_64x56x56_64_l, Conv64L, maxpool3x3s2_f32_64x112x112, Pool, _c256, bfuse::kChunked, 256, 1)
+BFUSE_HFUSE_KERNEL(conv3x3_f32_64x56x56_64_l, Conv64L, maxpool3x3s2_f32_64x112x112, Pool)

@@ -5,6 +5,7 @@
 // different grid sizes under horizontal fusion, and the ratio / proportional block patterns.
 #include "fuse.h"
 #include "ops_conv.h"
+#include "ops_conv_lds.h"
 #include "ops_gemm_bf16.h"
 #include "ops_gemm_bf16_ring.h"
 #include "ops_gemm_f32.h"
@@ -26,6 +27,9 @@ using SoftmaxS = SoftmaxCausal<2, 256, 2, 2, 2>;
 using ConvS1 = Conv3x3F32<16, 16, 8, 8, 16, 1, 1>;                     // one channel group, one wave
 using ConvS2 = Conv3x3F32<32, 32, 12, 12, 16, 1, 2>;                   // two channel groups on two waves
 using ConvS3 = Conv3x3F32<64, 16, 8, 16, 16, 2, 2>;                    // two groups per wave, two pixel blocks
+using ConvL1 = Conv3x3F32Lds<16, 16, 8, 8, 16, 1, 1>;                  // the same three shapes with the patch staged in LDS
+using ConvL2 = Conv3x3F32Lds<32, 32, 12, 12, 16, 1, 2>;
+using ConvL3 = Conv3x3F32Lds<64, 16, 8, 16, 16, 2, 2>;
 using PoolS = MaxPool3x3S2<4, 16, 16, 64>;
 using GemmB1 = GemmBf16NT<128, 1792, 64, 128, 224>;                   // one K-step
 using GemmB2 = GemmBf16NT<256, 1792, 192, 128, 224>;                  // two M-tiles, three K-steps
@@ -51,6 +55,9 @@ BFUSE_KERNEL(softmax_causal_2x256x256, SoftmaxS, ({{2, 256, 256, 1}, 4}), ({{1, 
 BFUSE_KERNEL(conv3x3_f32_16x8x8_16, ConvS1, ({{1, 16, 8, 8}, 4}), ({{16, 16, 3, 3}, 4}), ({{1, 16, 8, 8}, 4}))
 BFUSE_KERNEL(conv3x3_f32_32x12x12_32, ConvS2, ({{1, 32, 12, 12}, 4}), ({{32, 32, 3, 3}, 4}), ({{1, 32, 12, 12}, 4}))
 BFUSE_KERNEL(conv3x3_f32_64x8x16_16, ConvS3, ({{1, 64, 8, 16}, 4}), ({{16, 64, 3, 3}, 4}), ({{1, 16, 8, 16}, 4}))
+BFUSE_KERNEL(conv3x3_f32_16x8x8_16_l, ConvL1, ({{1, 16, 8, 8}, 4}), ({{16, 16, 3, 3}, 4}), ({{1, 16, 8, 8}, 4}))
+BFUSE_KERNEL(conv3x3_f32_32x12x12_32_l, ConvL2, ({{1, 32, 12, 12}, 4}), ({{32, 32, 3, 3}, 4}), ({{1, 32, 12, 12}, 4}))
+BFUSE_KERNEL(conv3x3_f32_64x8x16_16_l, ConvL3, ({{1, 64, 8, 16}, 4}), ({{16, 64, 3, 3}, 4}), ({{1, 16, 8, 16}, 4}))
 BFUSE_KERNEL(maxpool3x3s2_f32_4x16x16, PoolS, ({{1, 4, 16, 16}, 4}), ({{1, 1, 1, 1}, 4}), ({{1, 4, 8, 8}, 4}))
 BFUSE_KERNEL(gemm_bf16_128x64x1792, GemmB1, ({{128, 64, 1, 1}, 2}), ({{1792, 64, 1, 1}, 2}), ({{128, 1792, 1, 1}, 2}))
 BFUSE_KERNEL(gemm_bf16_256x192x1792, GemmB2, ({{256, 192, 1, 1}, 2}), ({{1792, 192, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
@@ -90,3 +97,5 @@ BFUSE_BFUSE_KERNEL(gemm_gelu_f32_64x192x288_d, GemmS6, layernorm_8x256, LayerNor
 using GemmS7 = GemmF32Dma<64, 288, 192, 32, 144, 4, kEpiGeluTanh, 3, 1>;   // four compute + four producer waves
 BFUSE_KERNEL(gemm_gelu_f32_64x192x288_pc, GemmS7, ({{64, 192, 1, 1}, 4}), ({{192, 288, 1, 1}, 4}), ({{64, 288, 1, 1}, 4}))
 BFUSE_BFUSE_KERNEL(gemm_gelu_f32_64x192x288_pc, GemmS7, layernorm_8x256, LayerNormS, _c4, bfuse::kChunked, 4, 1)
+BFUSE_HFUSE_KERNEL(conv3x3_f32_32x12x12_32_l, ConvL2, bias_relu_4096, BiasReluS)
+BFUSE_BFUSE_KERNEL(conv3x3_f32_64x8x16_16_l, ConvL3, layernorm_8x256, LayerNormS, _c4, bfuse::kChunked, 4, 1)

@@ -1,0 +1,189 @@
+// 3x3 / stride 1 / pad 1 convolution, implicit GEMM on the matrix cores with the image patch
+// staged in LDS.  Same operator, same decomposition and the same arithmetic order as
+// Conv3x3F32 (ops_conv.h): one workgroup owns BM output channels x PB*16 pixels, its KS waves
+// split the reduction by 16-channel group, every wave walks the nine taps of its group, the
+// partial tiles are summed through LDS in wave order.  What differs is where the B operand
+// (image values under a filter tap) comes from.
+//
+// Conv3x3F32 fetches it from global memory tap by tap: 16 scalar loads with a border test and
+// 4 weight loads per 16 MFMAs.  Measured on MI355X, every vector-ALU instruction a wave issues
+// between its MFMAs costs ~20 clocks of MFMA issue and a global load with its address
+// arithmetic 70-110, so that loop spends three quarters of its time not multiplying.  Here a wave
+// first copies the 16 channels x (rows the tile touches + 2) x (W + 2) patch it needs into a
+// zero-padded LDS tile of its own -- once, before the loop, where issue slots are free -- in the
+// layout [channel quad kq][position][4 channels].  In the loop the B operand of a tap is then ONE
+// 128-bit LDS read per 16-pixel block, at a compile-time offset from a per-block base register
+// (the padding removes the border test, the tap is an immediate), and the A operand -- the
+// lane's 4 channels x 9 taps of one filter row, 36 consecutive floats -- sits in registers for
+// the whole group.  Loop body per tap: PB reads, 4*TM*PB MFMAs, no vector ALU.
+//
+// The tile is private to the wave, so the K loop has no barrier; consecutive pixels of a block
+// are consecutive 16-byte slots of a plane, so the reads are free of bank conflicts.
+//
+// Measured on the ResNet shape (64 -> 64 channels, 56 x 56, 196 workgroups): the loop drops to
+// 2.4 us, but the kernel only from 8.0 to 7.7 us -- filter rows 1.4 us and the patch 2.9 us now
+// come first (110 KB per workgroup through the ~30 B/clk global->VGPR path, 22 x the unique data
+// over the grid), the reduction and stores take 0.75 us, and ~1.7 us is launch.  At this problem
+// size the convolution is bounded by getting started, not by its inner loop.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "dispatch.h"
+#include "ops_conv.h"
+#include "wave.h"
+
+namespace bfuse {
+
+template <int CI_, int CO_, int H_, int W_, int BM_, int PB_, int KS_>
+struct Conv3x3F32Lds {
+    static constexpr int CI = CI_, CO = CO_, H = H_, W = W_, BM = BM_, PB = PB_, KS = KS_;
+    static constexpr int HW = H * W;
+    static constexpr int TM = BM / 16;
+    static constexpr int NGROUP = CI / 16;           // 16-channel groups
+    static constexpr int GPW = NGROUP / KS;          // groups per wave
+    static constexpr int TP = 16 * PB;               // pixels per tile (consecutive in row-major order)
+    static constexpr int NPT = HW / TP;
+    static constexpr int SPAN = (TP + W - 2) / W + 1;   // image rows TP consecutive pixels can touch
+    static constexpr int R = SPAN + 2, WP = W + 2;      // staged rows / columns, one of padding on each side
+    static constexpr int NPOS = R * WP;
+    static constexpr int PLANE = NPOS * 16;             // bytes of one channel quad: [position][4 channels]
+    static constexpr int TILE_BYTES = 4 * PLANE;
+    static constexpr int CPR = W / 4;                   // 16-byte chunks per image row
+    static constexpr int NQ = R * CPR * 16;             // chunk loads per group: rows x chunks x channels
+    static constexpr int NLD = (NQ + 63) / 64;
+    static constexpr int NZ = (TILE_BYTES + 1023) / 1024;
+    static_assert(CI % 16 == 0 && CO % BM == 0 && BM % 16 == 0, "channel tiling");
+    static_assert(HW % TP == 0 && NGROUP % KS == 0 && W % 4 == 0, "pixel / reduction tiling");
+    static_assert((2 * WP + 2) * 16 + 3 * PLANE < 65536, "tap offsets are 16-bit immediates");
+
+    static constexpr Dims3 GRID{NPT, CO / BM, 1};
+    static constexpr Dims3 BLOCK{64 * KS, 1, 1};
+    static constexpr int THREADS = 64 * KS;
+    static constexpr bool HAS_BARRIERS = KS > 1;
+    static constexpr int PART_BYTES = KS > 1 ? KS * TM * PB * 1024 : 0;
+
+    struct Smem {
+        __attribute__((aligned(16))) unsigned char t[KS * TILE_BYTES > PART_BYTES ? KS * TILE_BYTES : PART_BYTES];
+    };
+
+    template <class Sync>
+    __device__ static __forceinline__ void run(int vblock, int tid, Smem& sm, const void* I, const void* F,
+                                               void* O, Sync sync)
+    {
+        const float* __restrict__ X = static_cast<const float*>(I);
+        const float* __restrict__ Wt = static_cast<const float*>(F);
+        float* __restrict__ Y = static_cast<float*>(O);
+        const Dims3 vb = delinearize(vblock, GRID);
+        const int p0 = vb.x * TP, co0 = vb.y * BM;
+        const int y_lo = p0 / W;                       // first image row of the tile; staged row 0 is y_lo - 1
+        const int wave = tid >> 6, lane = tid & 63;
+        const int li = lane & 15, kq = lane >> 4;
+        unsigned char* const tile = sm.t + wave * TILE_BYTES;
+
+        // padding (and rows outside the image) read as zero: 0 * w adds exactly 0, as the border
+        // test of the global-memory kernel does
+#pragma unroll
+        for (int z = 0; z < NZ; ++z) {
+            const int off = z * 1024 + lane * 16;
+            if (off < TILE_BYTES) *reinterpret_cast<f32x4*>(tile + off) = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+
+        // this lane's pixel of each block: the top-left tap of its window, plane kq
+        const unsigned char* bbase[PB];
+#pragma unroll
+        for (int pb = 0; pb < PB; ++pb) {
+            const int p = p0 + pb * 16 + li;
+            bbase[pb] = tile + kq * PLANE + ((p / W - y_lo) * WP + p % W) * 16;
+        }
+
+        f32x4 acc[TM][PB];
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+            for (int pb = 0; pb < PB; ++pb) acc[tm][pb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll 1
+        for (int gi = 0; gi < GPW; ++gi) {
+            const int ci0 = (wave + gi * KS) * 16;
+            // A operand: Wt[co][ci0 + 4 kq + t][tap], t = 0..3, tap = 0..8 -- 36 consecutive floats
+            f32x4 aw[TM][9];
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm) {
+                const f32x4* src = reinterpret_cast<const f32x4*>(Wt + ((size_t)(co0 + tm * 16 + li) * CI + ci0 + 4 * kq) * 9);
+#pragma unroll
+                for (int j = 0; j < 9; ++j) aw[tm][j] = src[j];
+            }
+            // stage the patch: chunk q = (channel cl, row r, 16-byte chunk c), chunk fastest, so that a wave-level
+            // load covers whole image rows (224-byte segments) instead of 64 separate cache lines
+            f32x4 v[NLD];
+#pragma unroll
+            for (int j = 0; j < NLD; ++j) {
+                const int q = j * 64 + lane;
+                const int c = q % CPR, r = (q / CPR) % R, cl = q / (CPR * R);
+                const int yy = y_lo - 1 + r;
+                const bool ok = q < NQ && yy >= 0 && yy < H;
+                v[j] = ok ? *reinterpret_cast<const f32x4*>(X + (size_t)(ci0 + cl) * HW + yy * W + 4 * c) : f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+#pragma unroll
+            for (int j = 0; j < NLD; ++j) {
+                const int q = j * 64 + lane;
+                const int c = q % CPR, r = (q / CPR) % R, cl = q / (CPR * R);
+                const int yy = y_lo - 1 + r;
+                if (q < NQ && yy >= 0 && yy < H) {
+                    float* dst = reinterpret_cast<float*>(tile + (cl / 4) * PLANE + (r * WP + 1 + 4 * c) * 16) + cl % 4;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) dst[4 * e] = v[j][e];
+                }
+            }
+
+            // nine taps: read the next tap's operands while this one multiplies
+            f32x4 b[2][PB];
+#pragma unroll
+            for (int pb = 0; pb < PB; ++pb) b[0][pb] = *reinterpret_cast<const f32x4*>(bbase[pb]);
+#pragma unroll
+            for (int tap = 0; tap < 9; ++tap) {
+                if (tap + 1 < 9) {
+                    const int noff = (((tap + 1) / 3) * WP + (tap + 1) % 3) * 16;
+#pragma unroll
+                    for (int pb = 0; pb < PB; ++pb) b[(tap + 1) & 1][pb] = *reinterpret_cast<const f32x4*>(bbase[pb] + noff);
+                }
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+                        for (int pb = 0; pb < PB; ++pb)
+                            acc[tm][pb] = __builtin_amdgcn_mfma_f32_16x16x4f32(aw[tm][(t * 9 + tap) / 4][(t * 9 + tap) % 4],
+                                                                               b[tap & 1][pb][t], acc[tm][pb], 0, 0, 0);
+            }
+        }
+
+        if constexpr (KS == 1) {
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+                for (int pb = 0; pb < PB; ++pb) Conv3x3F32<CI, CO, H, W, BM, PB, KS>::store_block(Y, co0, p0, tm, pb, acc[tm][pb], lane);
+        } else {
+            f32x4(*part)[TM * PB][64] = reinterpret_cast<f32x4(*)[TM * PB][64]>(sm.t);
+            sync();  // the partial tiles overwrite the patches: every wave is done reading its own
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+                for (int pb = 0; pb < PB; ++pb) part[wave][tm * PB + pb][lane] = acc[tm][pb];
+            sync();
+            // block u is finished by wave u mod KS, summing the partials of waves 0..KS-1 in order
+#pragma unroll
+            for (int u0 = 0; u0 < TM * PB; u0 += KS) {
+                const int u = u0 + wave;
+                if (u < TM * PB) {
+                    f32x4 s = part[0][u][lane];
+#pragma unroll
+                    for (int w = 1; w < KS; ++w) s += part[w][u][lane];
+                    Conv3x3F32<CI, CO, H, W, BM, PB, KS>::store_block(Y, co0, p0, u / PB, u % PB, s, lane);
+                }
+            }
+        }
+    }
+};
+
+}  // namespace bfuse

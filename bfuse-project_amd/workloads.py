@@ -121,7 +121,9 @@ PAIRS: Dict[int, Pair] = {
             "conv3x3_f32_64x56x56_64", "maxpool3x3s2_f32_64x112x112", "bfuse",
             [("bfuse", ""), ("bfuse", "_c8"), ("bfuse", "_c256"), ("hfuse", "")],
             [("conv3x3_f32_64x56x56_64_h", "maxpool3x3s2_f32_64x112x112", "bfuse", ""),
-             ("conv3x3_f32_64x56x56_64_h", "maxpool3x3s2_f32_64x112x112", "bfuse", "_c8")], _pair3_inputs,
+             ("conv3x3_f32_64x56x56_64_h", "maxpool3x3s2_f32_64x112x112", "bfuse", "_c8"),
+             ("conv3x3_f32_64x56x56_64_l", "maxpool3x3s2_f32_64x112x112", "bfuse", "_c256"),
+             ("conv3x3_f32_64x56x56_64_l", "maxpool3x3s2_f32_64x112x112", "hfuse", "")], _pair3_inputs,
             bytes1=(64 * 56 * 56 * 2 + 64 * 64 * 9) * 4, bytes2=(64 * 112 * 112 + 64 * 56 * 56) * 4,
             flops=2 * 64 * 64 * 9 * 56 * 56, bound="mfma", peak=157.3, dtype="f32", tol=1e-5),
     4: Pair(4, "causal softmax 12x[512x512] fp32 || GEMM fp32 [512x768].[768x3072] + tanh-GELU, bfuse",

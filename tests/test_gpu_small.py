@@ -59,6 +59,12 @@ def _cases():
                                     lambda I, F: orf.conv2d(I.reshape(1, 32, 12, 12), F.reshape(32, 32, 3, 3)), 1e-5, False),
         "conv3x3_f32_64x8x16_16": (lambda s: (fill_normal(s, 64 * 128, 0, 1), fill_normal(s + 1, 16 * 64 * 9, 0, 0.05)),
                                    lambda I, F: orf.conv2d(I.reshape(1, 64, 8, 16), F.reshape(16, 64, 3, 3)), 1e-5, False),
+        "conv3x3_f32_16x8x8_16_l": (lambda s: (np.maximum(fill_normal(s, 16 * 64, 0, 1), 0), fill_normal(s + 1, 16 * 16 * 9, 0, 0.05)),
+                                    lambda I, F: orf.conv2d(I.reshape(1, 16, 8, 8), F.reshape(16, 16, 3, 3)), 1e-5, False),
+        "conv3x3_f32_32x12x12_32_l": (lambda s: (np.maximum(fill_normal(s, 32 * 144, 0, 1), 0), fill_normal(s + 1, 32 * 32 * 9, 0, 0.05)),
+                                      lambda I, F: orf.conv2d(I.reshape(1, 32, 12, 12), F.reshape(32, 32, 3, 3)), 1e-5, False),
+        "conv3x3_f32_64x8x16_16_l": (lambda s: (fill_normal(s, 64 * 128, 0, 1), fill_normal(s + 1, 16 * 64 * 9, 0, 0.05)),
+                                     lambda I, F: orf.conv2d(I.reshape(1, 64, 8, 16), F.reshape(16, 64, 3, 3)), 1e-5, False),
         "maxpool3x3s2_f32_4x16x16": (lambda s: (fill_normal(s, 4 * 256, -3, 1), z),        # all-negative: padding must not win
                                      lambda I, F: orf.maxpool2d(I.reshape(1, 4, 16, 16)), 0.0, False),
         "gemm_bf16_128x64x1792": (lambda s: (f32_to_bf16(fill_normal(s, 128 * 64, 0, 1)), f32_to_bf16(fill_normal(s + 1, 1792 * 64, 0, 0.1))),
@@ -96,6 +102,8 @@ FUSIONS = [
     ("gemm_gelu_f32_64x192x288_d", "layernorm_8x256", "bfuse", "_c4"),
     ("gemm_gelu_f32_64x192x288_pc", "layernorm_8x256", "bfuse", "_c4"),
     ("gemm_bf16_256x320x1792_r", "rmsnorm_rope_bf16_6x1024", "hfuse", ""),
+    ("conv3x3_f32_32x12x12_32_l", "bias_relu_4096", "hfuse", ""),
+    ("conv3x3_f32_64x8x16_16_l", "layernorm_8x256", "bfuse", "_c4"),
 ]
 
 
