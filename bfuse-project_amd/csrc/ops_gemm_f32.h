@@ -34,12 +34,18 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 enum Epilogue : int { kEpiNone = 0, kEpiGeluTanh = 1 };
 
 // 0.5*x*(1+tanh(0.797885*(x+0.044715*x^3))) with the constants of the reference's GPT-2 dump
-// (files/gpt2.txt:67-74).
+// (files/gpt2.txt:67-74), evaluated as x / (1 + exp(-2u)): 0.5*(1 + tanh u) is the logistic
+// function of 2u, which has no cancellation for negative x and needs one v_exp_f32 and one
+// v_rcp_f32 (both ~1 ulp) instead of the library tanh's several dozen instructions -- the
+// epilogue runs on SIMDs whose issue slots other workgroups' MFMAs are competing for.
+// exp2 overflows to +inf for very negative x (result -0, the limit) and flushes to 0 for very
+// positive x (result x).
 __device__ __forceinline__ float gelu_tanh(float x)
 {
     const float x3 = x * x * x;
     const float u = 0.797885f * (x + 0.044715f * x3);
-    return (0.5f * x) * (tanhf(u) + 1.0f);
+    const float e = __builtin_amdgcn_exp2f(u * -2.885390081777927f);   // exp(-2u) = 2^(-2u log2 e)
+    return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 
 template <int M_, int N_, int K_, int BM_, int BN_, int KS_, int EPI_ = kEpiNone, int NBUF_ = 2, int SCHED_ = 1>
