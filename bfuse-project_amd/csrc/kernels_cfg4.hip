@@ -68,3 +68,8 @@ BFUSE_BFUSE_KERNEL(softmax_causal_12x512x512, Softmax4, gemm_gelu_f32_512x768x30
 BFUSE_BFUSE_KERNEL(softmax_causal_12x512x512_b4, Softmax4b, gemm_gelu_f32_512x768x3072_dh, GemmFcDh, _c256, bfuse::kChunked, 256, 1)
 BFUSE_HFUSE_KERNEL(softmax_causal_12x512x512_r3, Softmax4x3, gemm_gelu_f32_512x768x3072_dh, GemmFcDh)
 BFUSE_BFUSE_RT_KERNEL(softmax_causal_12x512x512, Softmax4, gemm_gelu_f32_512x768x3072_dh, GemmFcDh)
+using GemmFcDh2 = GemmF32Dma<512, 3072, 768, 32, 96, 4, kEpiGeluTanh, 2>;   // two ring stages: 32 KB, so that more softmax workgroups fit beside two of these
+BFUSE_KERNEL(gemm_gelu_f32_512x768x3072_dh2, GemmFcDh2, ({{512, 768, 1, 1}, 4}), ({{768, 3072, 1, 1}, 4}), ({{512, 3072, 1, 1}, 4}))
+BFUSE_BFUSE_KERNEL(softmax_causal_12x512x512, Softmax4, gemm_gelu_f32_512x768x3072_dh2, GemmFcDh2, _c512, bfuse::kChunked, 512, 1)
+BFUSE_BFUSE_KERNEL(softmax_causal_12x512x512, Softmax4, gemm_gelu_f32_512x768x3072_dh2, GemmFcDh2, _c256, bfuse::kChunked, 256, 1)
+BFUSE_BFUSE_RT_KERNEL(softmax_causal_12x512x512, Softmax4, gemm_gelu_f32_512x768x3072_dh2, GemmFcDh2)

@@ -185,12 +185,16 @@ struct SoftmaxCausal {
 #pragma unroll
             for (int c = 0; c < VEC; ++c) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) v[b][c][e] = expf(v[b][c][e] - m);  // exp(-inf) == 0 for masked columns
+                for (int e = 0; e < 4; ++e)   // exp(x - m) = 2^((x - m) log2 e): one v_exp_f32; masked columns give 2^-inf == 0
+                    v[b][c][e] = __builtin_amdgcn_exp2f((v[b][c][e] - m) * 1.4426950408889634f);
                 s += (v[b][c][0] + v[b][c][1]) + (v[b][c][2] + v[b][c][3]);
             }
             s = wave_sum(s);
+            // one division per row, one multiplication per element: under fusion these instructions
+            // compete for issue slots with the other side's MFMAs (an IEEE division is ~10 of them)
+            const float rs = 1.0f / s;
 #pragma unroll
-            for (int c = 0; c < VEC; ++c) y[c * 64 + lane] = v[b][c] / s;
+            for (int c = 0; c < VEC; ++c) y[c * 64 + lane] = v[b][c] * rs;
         }
     }
 

@@ -147,7 +147,9 @@ PAIRS: Dict[int, Pair] = {
              ("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072_dh", "bfuse", "_c256"),
              ("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072_dh", "bfuse", "_c512"),
              ("softmax_causal_12x512x512_b4", "gemm_gelu_f32_512x768x3072_dh", "bfuse", "_c256"),
-             ("softmax_causal_12x512x512_r3", "gemm_gelu_f32_512x768x3072_dh", "hfuse", "")], _pair4_inputs,
+             ("softmax_causal_12x512x512_r3", "gemm_gelu_f32_512x768x3072_dh", "hfuse", ""),
+             ("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072_dh2", "bfuse", "_c256"),
+             ("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072_dh2", "bfuse", "_c512")], _pair4_inputs,
             bytes1=2 * 12 * 512 * 512 * 4, bytes2=(512 * 768 + 768 * 3072 + 512 * 3072) * 4,
             flops=2 * 512 * 768 * 3072, bound="mfma", peak=157.3, dtype="f32", tol=1e-5),
     5: Pair(5, "GEMM bf16 [512x4096].[14336x4096]^T (fp32 acc) || RMSNorm+RoPE [512x4096] bf16, bfuse",
@@ -177,7 +179,7 @@ HEADLINE = {
     1: ("gemm_f32_512x512x512", "bias_relu_1048576", "hfuse", ""),
     2: ("gemm_f32_512x768x2304_d", "layernorm_512x768_w1", "bfuse", "_r"),
     3: ("conv3x3_f32_64x56x56_64", "maxpool3x3s2_f32_64x112x112", "bfuse", "_c256"),
-    4: ("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072_dh", "bfuse", "_c512"),
+    4: ("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072_dh2", "bfuse", "_c256"),
     5: ("gemm_bf16_512x4096x14336_p", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
 }
 
@@ -189,6 +191,6 @@ MEASURED_TRAFFIC = {
     "gemm_f32_512x512x512_bias_relu_1048576_fused_hfuse": 23_190_000,
     "gemm_f32_512x768x2304_d_layernorm_512x768_w1_fused_bfuse_r": 28_530_000,
     "conv3x3_f32_64x56x56_64_maxpool3x3s2_f32_64x112x112_fused_bfuse_c256": 11_060_000,
-    "softmax_causal_12x512x512_gemm_gelu_f32_512x768x3072_dh_fused_bfuse_c512": 47_770_000,
+    "softmax_causal_12x512x512_gemm_gelu_f32_512x768x3072_dh2_fused_bfuse_c256": 47_740_000,
     "gemm_bf16_512x4096x14336_p_rmsnorm_rope_bf16_512x4096_fused_bfuse_c256": 174_820_000,
 }
