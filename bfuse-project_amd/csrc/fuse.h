@@ -152,10 +152,16 @@ __device__ __forceinline__ void hfuse_body(const void* I1, const void* F1, void*
     __syncthreads();
     int local = 0;
     const int kernel_id = map_thread(plan, (int)blockIdx.x, (int)threadIdx.x, &local);
+    // A side whose partner has no barriers keeps the hardware barrier: s_barrier counts the waves
+    // of the workgroup that are still alive, the partner's waves never take part and leave when
+    // they are done, so the worst case is that this side's first barrier waits for them.  Only when
+    // BOTH sides synchronise do they need barriers of their own (the LDS arrival counters).
     if (kernel_id == 0) {
-        A::run((int)blockIdx.x, local, ss.a, I1, F1, O1, GroupSync{&ss.arrive[0], (unsigned)(round_up(A::THREADS, kWaveSize) / kWaveSize), 0u});
+        if constexpr (!B::HAS_BARRIERS) A::run((int)blockIdx.x, local, ss.a, I1, F1, O1, BlockSync{});
+        else A::run((int)blockIdx.x, local, ss.a, I1, F1, O1, GroupSync{&ss.arrive[0], (unsigned)(round_up(A::THREADS, kWaveSize) / kWaveSize), 0u});
     } else if (kernel_id == 1) {
-        B::run((int)blockIdx.x, local, ss.b, I2, F2, O2, GroupSync{&ss.arrive[1], (unsigned)(round_up(B::THREADS, kWaveSize) / kWaveSize), 0u});
+        if constexpr (!A::HAS_BARRIERS) B::run((int)blockIdx.x, local, ss.b, I2, F2, O2, BlockSync{});
+        else B::run((int)blockIdx.x, local, ss.b, I2, F2, O2, GroupSync{&ss.arrive[1], (unsigned)(round_up(B::THREADS, kWaveSize) / kWaveSize), 0u});
     }
 }
 

@@ -99,3 +99,6 @@ BFUSE_KERNEL(gemm_gelu_f32_64x192x288_pc, GemmS7, ({{64, 192, 1, 1}, 4}), ({{192
 BFUSE_BFUSE_KERNEL(gemm_gelu_f32_64x192x288_pc, GemmS7, layernorm_8x256, LayerNormS, _c4, bfuse::kChunked, 4, 1)
 BFUSE_HFUSE_KERNEL(conv3x3_f32_32x12x12_32_l, ConvL2, bias_relu_4096, BiasReluS)
 BFUSE_BFUSE_KERNEL(conv3x3_f32_64x8x16_16_l, ConvL3, layernorm_8x256, LayerNormS, _c4, bfuse::kChunked, 4, 1)
+// both sides synchronise: the LDS-staged GEMM's fence-free barriers and the split-K GEMM's reduction
+// barriers each become LDS arrival counters of their own side
+BFUSE_HFUSE_KERNEL(gemm_f32_128x160x192_l, GemmS4, gemm_gelu_f32_64x192x288_d, GemmS6)

@@ -104,7 +104,7 @@ struct Conv3x3F32 {
         float* __restrict__ Y = static_cast<float*>(O);
         const Dims3 vb = delinearize(vblock, GRID);
         const int p0 = vb.x * (16 * PB), co0 = vb.y * BM;
-        const int wave = tid >> 6, lane = tid & 63;
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;   // wave-uniform: addresses built on it stay in scalar registers
         int py[PB], px[PB];
 #pragma unroll
         for (int pb = 0; pb < PB; ++pb) {

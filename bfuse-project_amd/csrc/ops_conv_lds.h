@@ -76,7 +76,7 @@ struct Conv3x3F32Lds {
         const Dims3 vb = delinearize(vblock, GRID);
         const int p0 = vb.x * TP, co0 = vb.y * BM;
         const int y_lo = p0 / W;                       // first image row of the tile; staged row 0 is y_lo - 1
-        const int wave = tid >> 6, lane = tid & 63;
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;   // wave-uniform: addresses built on it stay in scalar registers
         const int li = lane & 15, kq = lane >> 4;
         unsigned char* const tile = sm.t + wave * TILE_BYTES;
 

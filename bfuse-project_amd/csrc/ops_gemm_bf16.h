@@ -264,21 +264,27 @@ struct GemmBf16NTDma {
     // that needs one of them, which throws away the read-ahead; written as asm it cannot see
     // them, and each MFMA group waits only for the fragments it uses (LDS reads of a wave
     // return in order, so "at most n outstanding" identifies which have landed).
-    template <int OFF>
+    // Operand addresses: one base register per (32-k substep, operand) and stage pair; the 16-row
+    // block and the stage are immediate offsets (+16 rows = +2048 bytes leaves the swizzle key alone)
+    struct Addr {
+        int a[BK / 32][(NSTG + 1) / 2], b[BK / 32][(NSTG + 1) / 2];   // [..][h]: base of stage 2h
+    };
+    static_assert(STAGE_BYTES + ((TM > TN ? TM : TN) - 1) * 2048 + 2048 <= 65536, "stage + block offsets are 16-bit immediates");
+    template <int IMM>
     __device__ static __forceinline__ bf16x8 lds_read(int addr)
     {
         bf16x8 r;
 #if defined(__HIP_DEVICE_COMPILE__)
-        if constexpr (OFF < 65536) {
-            asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
-        } else {
-            asm volatile("ds_read_b128 %0, %1" : "=v"(r) : "v"(addr + OFF));
-        }
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(IMM));
 #else
         r = bf16x8{};
 #endif
         return r;
     }
+    template <int U, int KS, int BLK>
+    __device__ static __forceinline__ bf16x8 read_a(const Addr& ad) { return lds_read<(U % 2) * STAGE_BYTES + BLK * 2048>(ad.a[KS][U / 2]); }
+    template <int U, int KS, int BLK>
+    __device__ static __forceinline__ bf16x8 read_b(const Addr& ad) { return lds_read<(U % 2) * STAGE_BYTES + BLK * 2048>(ad.b[KS][U / 2]); }
     template <int N_OUT>
     __device__ static __forceinline__ void wait_lds(bf16x8& b, bf16x8 (&a)[TM])
     {
@@ -307,24 +313,37 @@ struct GemmBf16NTDma {
         return n;
     }
 
+    template <int U, int KS, int A>
+    __device__ static __forceinline__ void read_a_all(bf16x8 (&af)[TM], const Addr& ad)
+    {
+        if constexpr (A < TM) {
+            af[A] = read_a<U, KS, A>(ad);
+            read_a_all<U, KS, A + 1>(af, ad);
+        }
+    }
+    template <int U, int P>
+    __device__ static __forceinline__ void read_b_first(bf16x8 (&bq)[RING], const Addr& ad)
+    {
+        if constexpr (P < PD) {
+            bq[P] = read_b<U, P / TN, P % TN>(ad);
+            read_b_first<U, P + 1>(bq, ad);
+        }
+    }
     template <int U, int ST>
-    __device__ static __forceinline__ void step_chain(f32x4 (&acc)[TM][TN], bf16x8 (&af)[BK / 32][TM], bf16x8 (&bq)[RING],
-                                                      const int (&a_ad)[BK / 32][TM], const int (&b_ad)[BK / 32][TN])
+    __device__ static __forceinline__ void step_chain(f32x4 (&acc)[TM][TN], bf16x8 (&af)[BK / 32][TM], bf16x8 (&bq)[RING], const Addr& ad)
     {
         if constexpr (ST < STEPS) {
             constexpr int ks = ST / TN, b = ST % TN;
-            constexpr int OFF = U * STAGE_BYTES;
             wait_lds<allowed(ST)>(bq[ST % RING], af[ks]);
 #pragma unroll
             for (int a = 0; a < TM; ++a)
                 acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[ks][a], bq[ST % RING], acc[a][b], 0, 0, 0);
-            if constexpr (ST + PD < STEPS) bq[(ST + PD) % RING] = lds_read<OFF>(b_ad[(ST + PD) / TN][(ST + PD) % TN]);
+            if constexpr (ST + PD < STEPS) bq[(ST + PD) % RING] = read_b<U, (ST + PD) / TN, (ST + PD) % TN>(ad);
             if constexpr (b == 1 && ks + 1 < BK / 32) {
-#pragma unroll
-                for (int a = 0; a < TM; ++a) af[ks + 1][a] = lds_read<OFF>(a_ad[ks + 1][a]);
+                read_a_all<U, ks + 1, 0>(af[ks + 1], ad);
             }
             __builtin_amdgcn_sched_barrier(0);
-            step_chain<U, ST + 1>(acc, af, bq, a_ad, b_ad);
+            step_chain<U, ST + 1>(acc, af, bq, ad);
         }
     }
 
@@ -343,21 +362,17 @@ struct GemmBf16NTDma {
 
     // LOADS: this wave also issues loads (no producer waves); otherwise it only meets the producers
     template <int U, bool LOADS, class Sync>
-    __device__ static __forceinline__ void k_step(int kt, f32x4 (&acc)[TM][TN], const int (&a_ad)[BK / 32][TM],
-                                                  const int (&b_ad)[BK / 32][TN], const Src& src,
+    __device__ static __forceinline__ void k_step(int kt, f32x4 (&acc)[TM][TN], const Addr& ad, const Src& src,
                                                   unsigned lds, bool full, Sync& sync)
     {
         if (kt >= NKT) return;
         if constexpr (LOADS) load_step<U>(kt, src, lds, full, sync);
         else sync.raw();
-        constexpr int OFF = U * STAGE_BYTES;
         bf16x8 af[BK / 32][TM], bq[RING];
-#pragma unroll
-        for (int a = 0; a < TM; ++a) af[0][a] = lds_read<OFF>(a_ad[0][a]);
-#pragma unroll
-        for (int p = 0; p < PD; ++p) bq[p] = lds_read<OFF>(b_ad[p / TN][p % TN]);
+        read_a_all<U, 0, 0>(af[0], ad);
+        read_b_first<U, 0>(bq, ad);
         __builtin_amdgcn_sched_barrier(0);
-        step_chain<U, 0>(acc, af, bq, a_ad, b_ad);
+        step_chain<U, 0>(acc, af, bq, ad);
     }
 
     template <class Sync>
@@ -417,32 +432,19 @@ struct GemmBf16NTDma {
             return;
         }
 
-        // byte offset inside a stage of every operand fragment this lane reads (K-substep ks,
-        // block a / b), with the chunk swizzle folded in: loop invariant
-        int a_rd[BK / 32][TM], b_rd[BK / 32][TN];
+        // LDS byte address of this lane's fragment of block 0 in stage 2h, for each 32-k substep, with
+        // the chunk swizzle folded in: loop invariant
+        const unsigned lds_base = (unsigned)(unsigned long long)(lds_u8*)sm.t;
+        Addr ad;
 #pragma unroll
         for (int ks = 0; ks < BK / 32; ++ks) {
             const int c = ks * 4 + kq;
+            const int arow = wm * WM + li, brow = BM + wn * WN + li;
 #pragma unroll
-            for (int a = 0; a < TM; ++a) {
-                const int row = wm * WM + a * 16 + li;
-                a_rd[ks][a] = row * 128 + ((c ^ ((row >> 1) & 7)) << 4);
+            for (int h = 0; h < (NSTG + 1) / 2; ++h) {
+                ad.a[ks][h] = (int)lds_base + 2 * h * STAGE_BYTES + arow * 128 + ((c ^ ((arow >> 1) & 7)) << 4);
+                ad.b[ks][h] = (int)lds_base + 2 * h * STAGE_BYTES + brow * 128 + ((c ^ ((brow >> 1) & 7)) << 4);
             }
-#pragma unroll
-            for (int b = 0; b < TN; ++b) {
-                const int row = BM + wn * WN + b * 16 + li;
-                b_rd[ks][b] = row * 128 + ((c ^ ((row >> 1) & 7)) << 4);
-            }
-        }
-
-        const unsigned lds_base = (unsigned)(unsigned long long)(lds_u8*)sm.t;
-        int a_ad[BK / 32][TM], b_ad[BK / 32][TN];  // absolute LDS byte addresses in stage 0
-#pragma unroll
-        for (int ks = 0; ks < BK / 32; ++ks) {
-#pragma unroll
-            for (int a = 0; a < TM; ++a) a_ad[ks][a] = a_rd[ks][a] + (int)lds_base;
-#pragma unroll
-            for (int b = 0; b < TN; ++b) b_ad[ks][b] = b_rd[ks][b] + (int)lds_base;
         }
 
         // K-steps are taken NSTG at a time so that the LDS stage of each is a compile-time constant;
@@ -451,10 +453,10 @@ struct GemmBf16NTDma {
         // fully unrolled short loop is where the register allocator runs out
 #pragma unroll 1
         for (int kt0 = 0; kt0 < NKT; kt0 += NSTG) {
-            k_step<0, PW == 0>(kt0, acc, a_ad, b_ad, src, lds, full, sync);
-            if constexpr (NSTG > 1) k_step<1, PW == 0>(kt0 + 1, acc, a_ad, b_ad, src, lds, full, sync);
-            if constexpr (NSTG > 2) k_step<2, PW == 0>(kt0 + 2, acc, a_ad, b_ad, src, lds, full, sync);
-            if constexpr (NSTG > 3) k_step<3, PW == 0>(kt0 + 3, acc, a_ad, b_ad, src, lds, full, sync);
+            k_step<0, PW == 0>(kt0, acc, ad, src, lds, full, sync);
+            if constexpr (NSTG > 1) k_step<1, PW == 0>(kt0 + 1, acc, ad, src, lds, full, sync);
+            if constexpr (NSTG > 2) k_step<2, PW == 0>(kt0 + 2, acc, ad, src, lds, full, sync);
+            if constexpr (NSTG > 3) k_step<3, PW == 0>(kt0 + 3, acc, ad, src, lds, full, sync);
         }
         sync();  // all waves are done reading the last stage before the tile buffer overwrites it
 

@@ -160,7 +160,7 @@ struct GemmF32 {
         float* __restrict__ C = static_cast<float*>(O);
         const Dims3 vb = delinearize(vblock, GRID);
         const int m0 = vb.y * BM, n0 = vb.x * BN;
-        const int wave = tid >> 6, lane = tid & 63;
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;   // wave-uniform: addresses built on it stay in scalar registers
         const int kbeg = wave * KW;
 
         f32x4 acc[TM][4 * G4 + G1];

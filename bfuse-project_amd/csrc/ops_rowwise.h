@@ -103,7 +103,7 @@ struct LayerNorm {
     __device__ static __forceinline__ void run(int vblock, int tid, Smem&, const void* I, const void* F,
                                                void* O, Sync)
     {
-        const int wave = tid >> 6, lane = tid & 63;
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;   // wave-uniform: addresses built on it stay in scalar registers
         const int row = vblock * WAVES + wave;
         const f32x4* __restrict__ x = static_cast<const f32x4*>(I) + (size_t)row * (D / 4);
         const f32x4* __restrict__ gamma = static_cast<const f32x4*>(F);
@@ -202,7 +202,7 @@ struct SoftmaxCausal {
     __device__ static __forceinline__ void run(int vblock, int tid, Smem&, const void* I, const void*,
                                                void* O, Sync)
     {
-        const int wave = tid >> 6, lane = tid & 63;
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;   // wave-uniform: addresses built on it stay in scalar registers
         // consecutive waves take consecutive rows; a wave's RPW rows are WAVES*GRID apart so
         // that every pass over the grid touches one contiguous slab of the matrix
         constexpr int stride = GRID.size() * WAVES;
@@ -251,7 +251,7 @@ struct RmsNormRope {
     __device__ static __forceinline__ void run(int vblock, int tid, Smem&, const void* I, const void* F,
                                                void* O, Sync)
     {
-        const int wave = tid >> 6, lane = tid & 63;
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;   // wave-uniform: addresses built on it stay in scalar registers
         const int pos = vblock * WAVES + wave;
         const unsigned short* __restrict__ x = static_cast<const unsigned short*>(I) + (size_t)pos * D;
         const unsigned short* __restrict__ w = static_cast<const unsigned short*>(F);
@@ -259,35 +259,44 @@ struct RmsNormRope {
         const float* __restrict__ sinv = reinterpret_cast<const float*>(static_cast<const char*>(F) + SIN_OFFSET) + (size_t)pos * HD;
         unsigned short* __restrict__ y = static_cast<unsigned short*>(O) + (size_t)pos * D;
 
-        float lo[SLOTS][8], hi[SLOTS][8];
+        // the row stays in registers as it was loaded (bf16, four registers per octet) and is widened
+        // where it is used: half the registers of an fp32 copy
+        u16x8 xl[SLOTS], xh[SLOTS];
         float ss = 0.f;
 #pragma unroll
         for (int s = 0; s < SLOTS; ++s) {
             const int slot = s * 64 + lane;
             const int base = (slot / OCT) * HD + (slot % OCT) * 8;
-            unpack(*reinterpret_cast<const u16x8*>(x + base), lo[s]);
-            unpack(*reinterpret_cast<const u16x8*>(x + base + HALF), hi[s]);
+            xl[s] = *reinterpret_cast<const u16x8*>(x + base);
+            xh[s] = *reinterpret_cast<const u16x8*>(x + base + HALF);
+            float lo[8], hi[8];
+            unpack(xl[s], lo);
+            unpack(xh[s], hi);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) ss += lo[s][e] * lo[s][e] + hi[s][e] * hi[s][e];
+            for (int e = 0; e < 8; ++e) ss += lo[e] * lo[e] + hi[e] * hi[e];
         }
         const float r = 1.0f / sqrtf(wave_sum(ss) / (float)D + 1e-5f);
 #pragma unroll
         for (int s = 0; s < SLOTS; ++s) {
-            const int slot = s * 64 + lane;
-            const int j = (slot % OCT) * 8;
-            const int base = (slot / OCT) * HD + j;
-            float wl[8], wh[8];
-            unpack(*reinterpret_cast<const u16x8*>(w + base), wl);
-            unpack(*reinterpret_cast<const u16x8*>(w + base + HALF), wh);
-            u16x8 ol, oh;
+            {
+                const int slot = s * 64 + lane;
+                const int j = (slot % OCT) * 8;
+                const int base = (slot / OCT) * HD + j;
+                float wl[8], wh[8], lo[8], hi[8];
+                unpack(*reinterpret_cast<const u16x8*>(w + base), wl);
+                unpack(*reinterpret_cast<const u16x8*>(w + base + HALF), wh);
+                unpack(xl[s], lo);
+                unpack(xh[s], hi);
+                u16x8 ol, oh;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const float tl = wl[e] * (lo[s][e] * r), th = wh[e] * (hi[s][e] * r);
-                ol[e] = to_bf16(tl * cosv[j + e] + (-th) * sinv[j + e]);
-                oh[e] = to_bf16(th * cosv[j + HALF + e] + tl * sinv[j + HALF + e]);
+                for (int e = 0; e < 8; ++e) {
+                    const float tl = wl[e] * (lo[e] * r), th = wh[e] * (hi[e] * r);
+                    ol[e] = to_bf16(tl * cosv[j + e] + (-th) * sinv[j + e]);
+                    oh[e] = to_bf16(th * cosv[j + HALF + e] + tl * sinv[j + HALF + e]);
+                }
+                *reinterpret_cast<u16x8*>(y + base) = ol;
+                *reinterpret_cast<u16x8*>(y + base + HALF) = oh;
             }
-            *reinterpret_cast<u16x8*>(y + base) = ol;
-            *reinterpret_cast<u16x8*>(y + base + HALF) = oh;
         }
     }
 };

@@ -102,6 +102,7 @@ FUSIONS = [
     ("gemm_gelu_f32_64x192x288_d", "layernorm_8x256", "bfuse", "_c4"),
     ("gemm_gelu_f32_64x192x288_pc", "layernorm_8x256", "bfuse", "_c4"),
     ("gemm_bf16_256x320x1792_r", "rmsnorm_rope_bf16_6x1024", "hfuse", ""),
+    ("gemm_f32_128x160x192_l", "gemm_gelu_f32_64x192x288_d", "hfuse", ""),   # both sides synchronise: LDS arrival counters
     ("conv3x3_f32_32x12x12_32_l", "bias_relu_4096", "hfuse", ""),
     ("conv3x3_f32_64x8x16_16_l", "layernorm_8x256", "bfuse", "_c4"),
 ]
