@@ -7,14 +7,22 @@
 //   GemmF32Dma  global -> LDS  (global_load_lds_dwordx4 into a ring PRIVATE to the wave)
 //                      -> VGPR (ds_read_b128 / b64 in MFMA layout)
 //
-// Measured on MI355X, the global->VGPR path delivers ~30 B/clk per CU and the direct-to-LDS
-// path ~52 B/clk; a 32 x 144 tile over K = 768 needs 540 KB per CU, which keeps the first path
-// busy enough that the single in-order wave per SIMD stalls at load issue.  Staging through
-// LDS costs LDS reads instead (250 B/clk per CU available) and takes the look-ahead out of
-// the register file.  Because no operand is shared between waves the ring needs NO barrier:
-// a wave waits for its own loads with s_waitcnt vmcnt(n) and for its own LDS reads with
-// s_waitcnt lgkmcnt(0); both are written by hand because the compiler would order every LDS
-// read after every outstanding direct-to-LDS load.
+// What the road buys is an inner loop made of MFMAs and almost nothing else.  Measured on
+// MI355X with single instructions dealt between the MFMAs of the issuing wave: one vector-ALU
+// instruction costs ~20 clocks of MFMA issue, an LDS read with an immediate offset ~12, an LDS
+// read whose address needs a v_add ~36, a global load with its 64-bit address arithmetic
+// 70-110.  So here
+//   * the ring slot, the fragment and the stage are immediate offsets on three base registers
+//     (the loop is unrolled over 2 fragment buffers x NSTG slots, the tail stages peeled with
+//     compile-time flags: no branch, no address arithmetic in a stage);
+//   * the loads are dma_load_lds_b128 (wave.h): a wave-uniform base in scalar registers, advanced
+//     by scalar adds, plus a constant per-lane offset;
+//   * the memory operations are dealt one or two per MFMA group.
+// A 32 x 144 tile gives 36 MFMAs : 6 loads : 8 LDS reads per 8-k stage and the loop runs at the
+// pipe rate (32.6 clocks per MFMA measured inside the kernel).  Because no operand is shared
+// between waves the ring needs NO barrier: a wave waits for its own loads with
+// s_waitcnt vmcnt(n) and for its own LDS reads with s_waitcnt lgkmcnt(0), both by hand (the
+// loads are asm, the compiler does not count them).
 //
 // Stage = 8 k.  Per wave and stage the ring slot holds A[BM][8] (rows of 32 bytes) followed by
 // B[8][BN].  Lane (i = lane % 16, kq = lane / 16) reads A[i][2kq], A[i][2kq+1] with one 64-bit
@@ -34,9 +42,9 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 //
 // PW_ = 1 adds one producer wave per k-range: it issues that range's direct-to-LDS loads and the
-// compute wave issues only LDS reads and MFMAs (a global load costs the issuing wave ~110 clocks
-// in which it cannot issue an MFMA; a wave that only loads does not disturb an MFMA wave on the
-// same SIMD).  Producer and compute waves meet at one workgroup barrier per K-stage.
+// compute wave issues only LDS reads and MFMAs.  Producer and compute waves meet at one workgroup
+// barrier per K-stage, which costs about what the six loads per stage did: no faster, kept as a
+// tested variant.
 template <int M_, int N_, int K_, int BM_, int BN_, int KS_, int EPI_ = kEpiNone, int NSTG_ = 3, int PW_ = 0>
 struct GemmF32Dma {
     static constexpr int M = M_, N = N_, K = K_, BM = BM_, BN = BN_, KS = KS_, EPI = EPI_, NSTG = NSTG_;
