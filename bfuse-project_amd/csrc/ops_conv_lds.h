@@ -8,7 +8,7 @@
 // Conv3x3F32 fetches it from global memory tap by tap: 16 scalar loads with a border test and
 // 4 weight loads per 16 MFMAs.  Measured on MI355X, every vector-ALU instruction a wave issues
 // between its MFMAs costs ~20 clocks of MFMA issue and a global load with its address
-// arithmetic 70-110, so that loop spends three quarters of its time not multiplying.  Here a wave
+// arithmetic 30-40, so that loop spends most of its time not multiplying.  Here a wave
 // first copies the 16 channels x (rows the tile touches + 2) x (W + 2) patch it needs into a
 // zero-padded LDS tile of its own -- once, before the loop, where issue slots are free -- in the
 // layout [channel quad kq][position][4 channels].  In the loop the B operand of a tap is then ONE

@@ -176,11 +176,12 @@ struct GemmBf16NT {
 // (still under 60 % of the ~250 B/clk the LDS delivers to eight waves) for a 1.5x higher
 // MFMA issue ceiling.
 //
-// Producer waves (PW_ > 0): measured on MI355X, every global load a wave issues -- to VGPRs or
-// direct to LDS -- keeps that wave from issuing anything else for ~110-125 clocks, an LDS read
-// for ~26; a wave that only issues loads leaves an MFMA wave on the same SIMD undisturbed.  With
-// PW_ extra waves the direct-to-LDS loads are issued by them and the WGM_ x WGN_ compute waves
-// issue only LDS reads and MFMAs.  All waves take part in every barrier.
+// Producer waves (PW_ > 0): measured on MI355X, a load issued between two MFMAs of the same wave
+// takes 8-14 clocks out of its MFMA stream when its base is in scalar registers (30-40 with the
+// 64-bit vector address arithmetic the compiler emits), an LDS read ~12; the same loads issued by
+// another wave of the SIMD cost the MFMA wave nothing.  With PW_ extra waves the direct-to-LDS
+// loads are issued by them and the WGM_ x WGN_ compute waves issue only LDS reads and MFMAs.  All
+// waves take part in every barrier.
 template <int M_, int N_, int K_, int BM_, int BN_, int NSTG_ = 3, int PD_ = 4, int WGM_ = 2, int WGN_ = 2, int PW_ = 0>
 struct GemmBf16NTDma {
     static constexpr int M = M_, N = N_, K = K_, BM = BM_, BN = BN_, NSTG = NSTG_;

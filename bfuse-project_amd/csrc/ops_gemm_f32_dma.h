@@ -10,8 +10,8 @@
 // What the road buys is an inner loop made of MFMAs and almost nothing else.  Measured on
 // MI355X with single instructions dealt between the MFMAs of the issuing wave: one vector-ALU
 // instruction costs ~20 clocks of MFMA issue, an LDS read with an immediate offset ~12, an LDS
-// read whose address needs a v_add ~36, a global load with its 64-bit address arithmetic
-// 70-110.  So here
+// read whose address needs a v_add ~37, a load with the 64-bit vector address arithmetic the
+// compiler emits 30-40, a direct-to-LDS load with a scalar base 8-14.  So here
 //   * the ring slot, the fragment and the stage are immediate offsets on three base registers
 //     (the loop is unrolled over 2 fragment buffers x NSTG slots, the tail stages peeled with
 //     compile-time flags: no branch, no address arithmetic in a stage);
