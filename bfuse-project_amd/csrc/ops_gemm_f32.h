@@ -80,24 +80,32 @@ struct GemmF32 {
         float b1[G1 > 0 ? G1 : 1][4];  // [group][t]
     };
 
+    // Every address is a wave-uniform part (tile origin, k, the row block, the k-step t: scalar
+    // registers) plus this lane's constant 32-bit offset: the loads then take the scalar-base form and
+    // no vector instruction is spent on addresses between the MFMAs.
     __device__ static __forceinline__ void load_stage(Frag& f, const float* __restrict__ A,
                                                       const float* __restrict__ B, int m0, int n0,
                                                       int k, int lane)
     {
         const int i = lane & 15, kq = lane >> 4;
+        const unsigned a_off = (unsigned)(i * K + 4 * kq) * 4u;            // bytes
+        const unsigned b_off = (unsigned)(4 * kq * N + 4 * i) * 4u;
+        const unsigned b1_off = (unsigned)(4 * kq * N + i) * 4u;
+        const char* a_ub = reinterpret_cast<const char*>(A + (size_t)m0 * K + k);
+        const char* b_ub = reinterpret_cast<const char*>(B + (size_t)k * N + n0);
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm)
-            f.a[tm] = *reinterpret_cast<const f32x4*>(A + (size_t)(m0 + tm * 16 + i) * K + k + 4 * kq);
+            f.a[tm] = *reinterpret_cast<const f32x4*>(a_ub + (size_t)tm * 16 * K * 4 + a_off);
 #pragma unroll
         for (int g = 0; g < G4; ++g)
 #pragma unroll
             for (int t = 0; t < 4; ++t)
-                f.b4[g][t] = *reinterpret_cast<const f32x4*>(B + (size_t)(k + 4 * kq + t) * N + n0 + g * 64 + 4 * i);
+                f.b4[g][t] = *reinterpret_cast<const f32x4*>(b_ub + ((size_t)t * N + g * 64) * 4 + b_off);
 #pragma unroll
         for (int g = 0; g < G1; ++g)
 #pragma unroll
             for (int t = 0; t < 4; ++t)
-                f.b1[g][t] = B[(size_t)(k + 4 * kq + t) * N + n0 + G4 * 64 + g * 16 + i];
+                f.b1[g][t] = *reinterpret_cast<const float*>(b_ub + ((size_t)t * N + G4 * 64 + g * 16) * 4 + b1_off);
     }
 
     __device__ static __forceinline__ void mma_stage(f32x4 (&acc)[TM][4 * G4 + G1], const Frag& f)
