@@ -367,7 +367,7 @@ struct GemmF32Dma {
             f32x4(*part)[TMR * NB][64] = reinterpret_cast<f32x4(*)[TMR * NB][64]>(sm.t);
 #pragma unroll
             for (int r = 0; r < ROUNDS; ++r) {
-                sync();   // round 0: rings dead; later rounds: the previous round's sums have been read
+                sync();   // first pass: the rings are dead; later passes: the previous sums have been read
                 if (!producer) {
 #pragma unroll
                     for (int tm = 0; tm < TMR; ++tm)
