@@ -150,4 +150,8 @@ def choose_fusion(a: KernelInfo, b: KernelInfo, lds_a: int, lds_b: int, cus: int
     rounds_a, rounds_b = -(-ga // (cus * na)), -(-gb // (cus * nb))
     return {"hfuse_ok": hfuse_ok, "prefer": "hfuse" if hfuse_ok and ga == gb else "bfuse",
             "wg_per_cu": (na, nb), "rounds": (rounds_a, rounds_b),
-            "chunk": 8 * max(1, min(ga, gb) // 8 and 1), "ratio_M": max(1, max(ga, gb) // max(1, min(ga, gb)))}
+            # one chunk per CU round when a grid covers the chip (measured best on MI355X: the
+            # compute-bound side lands one workgroup per CU and the other side is dealt on top);
+            # below that, a multiple of 8 keeps every side spread over the eight XCDs
+            "chunk": cus if max(ga, gb) >= cus else 8,
+            "ratio_M": max(1, max(ga, gb) // max(1, min(ga, gb)))}
