@@ -119,3 +119,45 @@ def test_pair5_gemm_every_output_element_exact_on_selector_inputs():
             got = op.run_kernel(0, A16, W).reshape(M, N)
         bad = np.nonzero(got != want)
         assert bad[0].size == 0, f"{name}: {bad[0].size} wrong elements, first at row {bad[0][0]} col {bad[1][0]}"
+
+
+@pytest.mark.parametrize("number,M,K,N,gemm_side", [(2, 512, 768, 2304, 0), (1, 512, 512, 512, 0)])
+def test_fp32_gemm_every_output_element_exact_on_selector_inputs(number, M, K, N, gemm_side):
+    """Selector inputs check every output index of the full-size fp32 GEMMs exactly, whatever the
+    K split: with one 1.0 per row of A at column k(r), C[r, n] = B[k(r), n] -- all other products are
+    exact zeros and every partial sum is exact -- so a wrong row, column, k-range or fragment shows
+    as a wrong element.  Run for each built implementation of the side."""
+    pair = PAIRS[number]
+    I1, B, I2, F2 = pair.inputs()
+    rng = np.random.default_rng(number)
+    k = rng.integers(0, K, M)
+    A = np.zeros((M, K), np.float32)
+    A[np.arange(M), k] = 1.0
+    want = B.reshape(K, N)[k, :]
+    for name in sorted({k1 for (k1, _) in fusions(pair)}):
+        _say(f"[pair {number}] selector inputs through {name}")
+        with bf.Operation(name, pair.k2) as op:
+            got = op.run_kernel(0, A.ravel(), B).reshape(M, N)
+        bad = np.nonzero(got != want)
+        assert bad[0].size == 0, f"{name}: {bad[0].size} wrong elements, first at row {bad[0][0]} col {bad[1][0]}"
+
+
+def test_pair4_gemm_gelu_every_output_element_on_selector_inputs():
+    """The same for pair 4's GEMM + tanh-GELU (side 2): C[r, n] = gelu(B[k(r), n]); the epilogue uses
+    the device's exp2 and reciprocal, so elements are compared within the pair's tolerance."""
+    pair = PAIRS[4]
+    I1, F1, _, B = pair.inputs()
+    M, K, N = 512, 768, 3072
+    rng = np.random.default_rng(4)
+    k = rng.integers(0, K, M)
+    A = np.zeros((M, K), np.float32)
+    A[np.arange(M), k] = 1.0
+    x = B.reshape(K, N)[k, :].astype(np.float64)
+    want = 0.5 * x * (1.0 + np.tanh(0.797885 * (x + 0.044715 * x ** 3)))
+    scale = max(float(np.sqrt((want ** 2).mean())), 1e-30)
+    for name in sorted({k2 for (_, k2) in fusions(pair)}):
+        _say(f"[pair 4] selector inputs through {name}")
+        with bf.Operation(pair.k1, name) as op:
+            got = op.run_kernel(1, A.ravel(), B).reshape(M, N).astype(np.float64)
+        err = np.abs(got - want) / np.maximum(np.abs(want), scale)
+        assert err.max() <= pair.tol, f"{name}: max rel err {err.max():.3e} at {np.unravel_index(err.argmax(), err.shape)}"
