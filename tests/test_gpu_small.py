@@ -182,3 +182,25 @@ def test_special_values():
         xf = bf16_to_f32(x).reshape(6, 1024).astype(np.float64)
         n0 = xf[0] / np.sqrt(np.mean(xf[0] ** 2) + 1e-5)            # position 0: rotation is the identity
         np.testing.assert_allclose(out[0], n0, rtol=1e-2, atol=1e-2 * np.sqrt(np.mean(n0 ** 2)))
+
+
+def test_gelu_epilogue_over_the_whole_range():
+    """tanh-GELU is evaluated as x / (1 + exp(-2u)) with the device's exp2 and reciprocal: check it
+    from -60 to 60 (exp2 overflows to inf on one side and flushes to 0 on the other) through a
+    selector GEMM, C[r, n] = gelu(B[k(r), n]), for each small GELU kernel."""
+    for name, (M, K, N) in {"gemm_gelu_f32_64x192x288_d": (64, 192, 288), "gemm_gelu_f32_64x192x288_pc": (64, 192, 288),
+                            "gemm_gelu_f32_96x128x192": (96, 128, 192)}.items():
+        rng = np.random.default_rng(7)
+        k = rng.integers(0, K, M)
+        A = np.zeros((M, K), np.float32)
+        A[np.arange(M), k] = 1.0
+        B = np.concatenate([np.linspace(-60.0, 60.0, K * N - 6), [0.0, -0.0, 1e-30, -1e-30, 88.0, -88.0]]).astype(np.float32)
+        B = rng.permutation(B).reshape(K, N)
+        x = B[k, :].astype(np.float64)
+        want = 0.5 * x * (1.0 + np.tanh(0.797885 * (x + 0.044715 * x ** 3)))
+        _say(f"[small] GELU range through {name}")
+        with bf.Operation(name, "bias_relu_4096") as op:
+            got = op.run_kernel(0, A.ravel(), B.ravel()).reshape(M, N).astype(np.float64)
+        assert np.isfinite(got).all()
+        err = np.abs(got - want) / np.maximum(np.abs(want), 1.0)
+        assert err.max() <= 1e-5, f"{name}: max err {err.max():.3e} at x = {x.ravel()[err.argmax()]}"
