@@ -116,7 +116,7 @@ __device__ __forceinline__ void bfuse_rt_body(const BlockPlan& plan, const void*
         if (tid < 2) sh.arrive[next][tid] = 0u;
         __syncthreads();  // every wave has left the previous iteration: its LDS contents are dead
         int virt = 0;
-        const int kernel_id = map_block(plan, id, &virt);
+        const int kernel_id = map_block(plan, id, &virt);   // scalar: the plan is a kernel argument
         if (kernel_id == 0 && tid < A::THREADS) {
             if constexpr (A::THREADS == T) A::run(virt, tid, sh.u.a, I1, F1, O1, BlockSync{});
             else A::run(virt, tid, sh.u.a, I1, F1, O1, GroupSync{&sh.arrive[set][0], (unsigned)(A::THREADS / kWaveSize), 0u});
@@ -183,7 +183,7 @@ struct KernelEntry {
     std::string side[2];    // fused: names of the two standalone kernels
     int pattern, p0, p1;    // bfuse: dispatch pattern and its parameters
     unsigned (*read_sync_timeouts)();  // device counter of GroupSync give-ups in this module
-    int (*set_plan)(const BlockPlan*); // bfuse_rt: copies a plan into the kernel's device-side plan (0 = ok)
+    int (*set_plan)(const BlockPlan*); // bfuse_rt: per-kernel hook called when a plan is installed (0 = ok); the plan itself travels as a kernel argument
 };
 
 std::vector<KernelEntry>& registry();
@@ -275,21 +275,19 @@ KernelEntry make_fused_entry(const char* name, const void* func, int kind, const
             #K1 "_" #K2 "_fused_hfuse", (const void*)&K1##_##K2##_fused_hfuse, bfuse::kHfuse, #K1, #K2, \
             OP1::HAS_BARRIERS || OP2::HAS_BARRIERS, -1, 0, 0, &bfuse_module_read_sync_timeouts));
 
-// The plan sits in device memory next to the kernel; the host writes it with an ordinary
-// (stream-ordered) copy before launching.
+// The plan is the kernel's seventh argument, passed by value: it arrives with the kernel arguments
+// (scalar loads that hit at once) instead of costing every workgroup a chain of dependent loads
+// from device memory before it can start.  The host keeps the installed plan and appends it at launch.
 #define BFUSE_BFUSE_RT_KERNEL(K1, OP1, K2, OP2)                                                      \
-    static __device__ bfuse::BlockPlan plan_##K1##_##K2##_rt;                                        \
     extern "C" __global__ __launch_bounds__((bfuse::BfuseRtPair<OP1, OP2>::THREADS), bfuse::kMinWavesPerEu)                 \
     void K1##_##K2##_fused_bfuse_rt(const void* __restrict__ I1, const void* __restrict__ F1,        \
                                     void* __restrict__ O1, const void* __restrict__ I2,              \
-                                    const void* __restrict__ F2, void* __restrict__ O2)              \
+                                    const void* __restrict__ F2, void* __restrict__ O2,              \
+                                    const bfuse::BlockPlan plan)                                     \
     {                                                                                               \
-        bfuse::bfuse_rt_body<OP1, OP2>(plan_##K1##_##K2##_rt, I1, F1, O1, I2, F2, O2);               \
+        bfuse::bfuse_rt_body<OP1, OP2>(plan, I1, F1, O1, I2, F2, O2);                                \
     }                                                                                               \
-    static int set_plan_##K1##_##K2##_rt(const bfuse::BlockPlan* p)                                  \
-    {                                                                                               \
-        return hipMemcpyToSymbol(HIP_SYMBOL(plan_##K1##_##K2##_rt), p, sizeof(*p)) == hipSuccess ? 0 : 1; \
-    }                                                                                               \
+    static int set_plan_##K1##_##K2##_rt(const bfuse::BlockPlan*) { return 0; }                      \
     static bfuse::Registrar reg_##K1##_##K2##_bfuse_rt([] {                                          \
         bfuse::KernelEntry e = bfuse::make_fused_entry<bfuse::BfuseRtPair<OP1, OP2>>(                \
             #K1 "_" #K2 "_fused_bfuse_rt", (const void*)&K1##_##K2##_fused_bfuse_rt, bfuse::kBfuseRt, #K1, #K2, \

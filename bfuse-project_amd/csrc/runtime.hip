@@ -200,7 +200,10 @@ int launch6(const void* func, const unsigned* grid, const unsigned* block, hipSt
             hipEvent_t ev0 = nullptr, hipEvent_t ev1 = nullptr)
 {
     Side &a = g.side[0], &b = g.side[1];
-    void* args[6] = {&a.buf[0], &a.buf[1], &a.buf[2], &b.buf[0], &b.buf[1], &b.buf[2]};
+    void* args[7] = {&a.buf[0], &a.buf[1], &a.buf[2], &b.buf[0], &b.buf[1], &b.buf[2], nullptr};
+    // a run-time-plan kernel takes its installed plan by value as a seventh argument
+    auto it = installed_plans().find(func);
+    if (it != installed_plans().end()) args[6] = &it->second;
     if (ev0 || ev1)
         HIP_TRY(hipExtLaunchKernel(func, d3(grid), d3(block), args, 0, stream, ev0, ev1, 0));
     else

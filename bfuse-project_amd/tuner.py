@@ -65,7 +65,7 @@ def static_choice(a: KernelHandle, b: KernelHandle, cus: int = 256) -> dict:
     return config.choose_fusion(ka, kb, max(a.lds_bytes, 0), max(b.lds_bytes, 0), cus)
 
 
-def autotune(op: Operation, candidates: Optional[Sequence[Candidate]] = None, warmup: int = 3, reps: int = 30,
+def autotune(op: Operation, candidates: Optional[Sequence[Candidate]] = None, warmup: int = 20, reps: int = 100,
              cus: int = 256) -> List[dict]:
     """Times every candidate plan of the pair's run-time-plan kernel over the buffers `op` holds
     (upload operands first).  Returns rows sorted by mean GPU time; row 0 is the choice."""
