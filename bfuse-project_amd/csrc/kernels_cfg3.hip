@@ -30,3 +30,4 @@ using Conv64L = Conv3x3F32Lds<64, 64, 56, 56, 16, 4, 4>;    // 196 workgroups, 7
 BFUSE_KERNEL(conv3x3_f32_64x56x56_64_l, Conv64L, ({{1, 64, 56, 56}, 4}), ({{64, 64, 3, 3}, 4}), ({{1, 64, 56, 56}, 4}))
 BFUSE_BFUSE_KERNEL(conv3x3_f32_64x56x56_64_l, Conv64L, maxpool3x3s2_f32_64x112x112, Pool, _c256, bfuse::kChunked, 256, 1)
 BFUSE_HFUSE_KERNEL(conv3x3_f32_64x56x56_64_l, Conv64L, maxpool3x3s2_f32_64x112x112, Pool)
+BFUSE_BFUSE_RT_KERNEL(conv3x3_f32_64x56x56_64_l, Conv64L, maxpool3x3s2_f32_64x112x112, Pool)

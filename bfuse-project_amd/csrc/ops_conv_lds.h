@@ -46,11 +46,13 @@ struct Conv3x3F32Lds {
     static constexpr int SPAN = (TP + W - 2) / W + 1;   // image rows TP consecutive pixels can touch
     static constexpr int R = SPAN + 2, WP = W + 2;      // staged rows / columns, one of padding on each side
     static constexpr int NPOS = R * WP;
-    static constexpr int PLANE = NPOS * 16;             // bytes of one channel quad: [position][4 channels]
+    // bytes of one channel quad, [position][4 channels], padded to 16 (mod 256): the four planes then
+    // start one 16-byte slot apart in the banks, which is what makes the staging writes below conflict-free
+    static constexpr int PLANE = (NPOS * 16 + 255) / 256 * 256 + 16;
     static constexpr int TILE_BYTES = 4 * PLANE;
     static constexpr int CPR = W / 4;                   // 16-byte chunks per image row
-    static constexpr int NQ = R * CPR * 16;             // chunk loads per group: rows x chunks x channels
-    static constexpr int NLD = (NQ + 63) / 64;
+    static constexpr int NCH = R * CPR;                 // 16-byte chunks per channel of the patch (contiguous in memory)
+    static constexpr int NLD = (NCH + 3) / 4;           // wave-level loads per group: 16 channels x 4 consecutive chunks each
     static constexpr int NZ = (TILE_BYTES + 1023) / 1024;
     static_assert(CI % 16 == 0 && CO % BM == 0 && BM % 16 == 0, "channel tiling");
     static_assert(HW % TP == 0 && NGROUP % KS == 0 && W % 4 == 0, "pixel / reduction tiling");
@@ -113,23 +115,27 @@ struct Conv3x3F32Lds {
 #pragma unroll
                 for (int j = 0; j < 9; ++j) aw[tm][j] = src[j];
             }
-            // stage the patch: chunk q = (channel cl, row r, 16-byte chunk c), chunk fastest, so that a wave-level
-            // load covers whole image rows (224-byte segments) instead of 64 separate cache lines
+            // stage the patch: lane = 4 * channel + (chunk % 4), i.e. a wave-level load takes four
+            // consecutive 16-byte chunks (64 bytes) of each of the 16 channels.  The four values of a chunk
+            // go to four consecutive positions of the channel's plane; with this lane order the 64 lanes of
+            // each of those stores fall in 64 different banks (channel % 4 -> word, channel / 4 -> plane,
+            // one slot apart, chunk % 4 -> 64 bytes apart)
+            const int cl = lane >> 2, c4 = lane & 3;
             f32x4 v[NLD];
 #pragma unroll
             for (int j = 0; j < NLD; ++j) {
-                const int q = j * 64 + lane;
-                const int c = q % CPR, r = (q / CPR) % R, cl = q / (CPR * R);
+                const int cc = j * 4 + c4;                 // chunk within the channel's R x W patch
+                const int r = cc / CPR, c = cc % CPR;
                 const int yy = y_lo - 1 + r;
-                const bool ok = q < NQ && yy >= 0 && yy < H;
+                const bool ok = cc < NCH && yy >= 0 && yy < H;
                 v[j] = ok ? *reinterpret_cast<const f32x4*>(X + (size_t)(ci0 + cl) * HW + yy * W + 4 * c) : f32x4{0.f, 0.f, 0.f, 0.f};
             }
 #pragma unroll
             for (int j = 0; j < NLD; ++j) {
-                const int q = j * 64 + lane;
-                const int c = q % CPR, r = (q / CPR) % R, cl = q / (CPR * R);
+                const int cc = j * 4 + c4;
+                const int r = cc / CPR, c = cc % CPR;
                 const int yy = y_lo - 1 + r;
-                if (q < NQ && yy >= 0 && yy < H) {
+                if (cc < NCH && yy >= 0 && yy < H) {
                     float* dst = reinterpret_cast<float*>(tile + (cl / 4) * PLANE + (r * WP + 1 + 4 * c) * 16) + cl % 4;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) dst[4 * e] = v[j][e];
