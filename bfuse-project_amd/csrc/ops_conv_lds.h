@@ -20,11 +20,11 @@
 // The tile is private to the wave, so the K loop has no barrier; consecutive pixels of a block
 // are consecutive 16-byte slots of a plane, so the reads are free of bank conflicts.
 //
-// Measured on the ResNet shape (64 -> 64 channels, 56 x 56, 196 workgroups): the loop drops to
-// 2.4 us, but the kernel only from 8.0 to 7.7 us -- filter rows 1.4 us and the patch 2.9 us now
-// come first (110 KB per workgroup through the ~30 B/clk global->VGPR path, 22 x the unique data
-// over the grid), the reduction and stores take 0.75 us, and ~1.7 us is launch.  At this problem
-// size the convolution is bounded by getting started, not by its inner loop.
+// Measured on the ResNet shape (64 -> 64 channels, 56 x 56, 196 workgroups; in-kernel clocks): filter
+// rows 1.5 us and patch 1.4 us (overlapping), loop 2.2 us (the MFMA pipe rate), reduction and stores
+// 0.85 us, ~1.5 us launch: 6.3-6.9 us against 8.0-8.2 for the global-memory kernel.  The lane order of
+// the staging matters as much as the loop: with the chunk index fastest the scattered 4-byte LDS
+// stores were 16-way bank conflicts and the patch alone took 2.9 us.
 #pragma once
 #include <hip/hip_runtime.h>
 

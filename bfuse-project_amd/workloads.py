@@ -190,7 +190,7 @@ HEADLINE = {
 MEASURED_TRAFFIC = {
     "gemm_f32_512x512x512_bias_relu_1048576_fused_hfuse": 23_190_000,
     "gemm_f32_512x768x2304_d_layernorm_512x768_w1_fused_bfuse_r": 28_530_000,
-    "conv3x3_f32_64x56x56_64_l_maxpool3x3s2_f32_64x112x112_fused_bfuse_c256": 11_060_000,
+    "conv3x3_f32_64x56x56_64_l_maxpool3x3s2_f32_64x112x112_fused_bfuse_c256": 12_320_000,
     "softmax_causal_12x512x512_gemm_gelu_f32_512x768x3072_dh2_fused_bfuse_c256": 47_740_000,
     "gemm_bf16_512x4096x14336_p_rmsnorm_rope_bf16_512x4096_fused_bfuse_c256": 174_820_000,
 }
