@@ -17,8 +17,12 @@
 // lane's 4 channels x 9 taps of one filter row, 36 consecutive floats -- sits in registers for
 // the whole group.  Loop body per tap: PB reads, 4*TM*PB MFMAs, no vector ALU.
 //
-// The tile is private to the wave, so the K loop has no barrier; consecutive pixels of a block
-// are consecutive 16-byte slots of a plane, so the reads are free of bank conflicts.
+// The tile is private to the wave, so the K loop has no barrier.  Consecutive pixels of a block
+// are consecutive 16-byte slots of a plane; the planes start one slot apart (see PLANE), which a
+// 128-bit read pays for with a second pass (measured 8 clocks per wave-level read instead of 5.3:
+// the hardware pairs lanes of two neighbouring quarter-waves in one pass, so only planes a
+// multiple of 256 bytes apart read conflict-free).  The loop needs a quarter of the LDS read rate
+// even so, whereas the staging stores, which the shift makes conflict-free, are on the critical path.
 //
 // Measured on the ResNet shape (64 -> 64 channels, 56 x 56, 196 workgroups; in-kernel clocks): filter
 // rows 1.5 us and patch 1.4 us (overlapping), loop 2.2 us (the MFMA pipe rate), reduction and stores
@@ -48,6 +52,7 @@ struct Conv3x3F32Lds {
     static constexpr int NPOS = R * WP;
     // bytes of one channel quad, [position][4 channels], padded to 16 (mod 256): the four planes then
     // start one 16-byte slot apart in the banks, which is what makes the staging writes below conflict-free
+    // (and the tap reads two-way conflicted: the cheaper side of the trade, see the header)
     static constexpr int PLANE = (NPOS * 16 + 255) / 256 * 256 + 16;
     static constexpr int TILE_BYTES = 4 * PLANE;
     static constexpr int CPR = W / 4;                   // 16-byte chunks per image row
