@@ -159,7 +159,8 @@ PAIRS: Dict[int, Pair] = {
              ("gemm_bf16_512x4096x14336_v", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
              ("gemm_bf16_512x4096x14336_w8", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
              ("gemm_bf16_512x4096x14336_r", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
-             ("gemm_bf16_512x4096x14336_p", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256")], _pair5_inputs,
+             ("gemm_bf16_512x4096x14336_p", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
+             ("gemm_bf16_512x4096x14336_x", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256")], _pair5_inputs,
             bytes1=(512 * 4096 + 4096 * 14336 + 512 * 14336) * 2, bytes2=2 * 512 * 4096 * 2 + 4096 * 2,
             flops=2 * 512 * 4096 * 14336, bound="mfma", peak=2500.0, dtype="bf16", tol=1e-2),
 }
