@@ -5,6 +5,8 @@
 // clock the chip actually ran at; with operand values that toggle bits (random, as in a real
 // GEMM) the power management holds a dense bf16 stream well below the boost clock, and that
 // clock -- not the 2.4 GHz behind the published peak -- bounds any bf16 GEMM on this part.
+// The bf16 stream is run with both instruction shapes (16x16x32: two A x seven B fragments;
+// 32x32x16: one A x seven B), figures per 16384 flop so that they compare.
 //
 //   hipcc --offload-arch=gfx950 -O3 -o mfma_clock_probe mfma_clock.hip && ./mfma_clock_probe
 #include <hip/hip_runtime.h>
@@ -14,7 +16,8 @@
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef short bf16x8 __attribute__((ext_vector_type(8)));
 
-enum Mode { kBf16Const, kBf16Random, kF32Const, kF32Random };
+enum Mode { kBf16Const, kBf16Random, kF32Const, kF32Random, kBf16x32Const, kBf16x32Random };
+typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 __device__ unsigned mix(unsigned x)
 {
@@ -28,7 +31,10 @@ template <int MODE>
 __global__ __launch_bounds__(512) void mfma_stream(float* out, unsigned long long* stamps, int iters)
 {
     constexpr bool kBf16 = MODE == kBf16Const || MODE == kBf16Random;
-    constexpr bool kRandom = MODE == kBf16Random || MODE == kF32Random;
+    constexpr bool k32 = MODE == kBf16x32Const || MODE == kBf16x32Random;
+    constexpr bool kRandom = MODE == kBf16Random || MODE == kF32Random || MODE == kBf16x32Random;
+    f32x16 big[7];
+    for (int j = 0; j < 7; ++j) for (int e = 0; e < 16; ++e) big[j][e] = 0.f;
     f32x4 acc[2][7];
     for (int i = 0; i < 2; ++i)
         for (int j = 0; j < 7; ++j) acc[i][j] = f32x4{0, 0, 0, 0};
@@ -45,6 +51,10 @@ __global__ __launch_bounds__(512) void mfma_stream(float* out, unsigned long lon
     }
     const unsigned long long c0 = clock64(), w0 = wall_clock64();
     for (int it = 0; it < iters; ++it) {
+        if constexpr (k32) {
+#pragma unroll
+            for (int j = 0; j < 7; ++j) big[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], b[j], big[j], 0, 0, 0);
+        } else
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -59,6 +69,7 @@ __global__ __launch_bounds__(512) void mfma_stream(float* out, unsigned long lon
         stamps[2 * blockIdx.x + 1] = w1 - w0;
     }
     f32x4 s = {0, 0, 0, 0};
+    for (int j = 0; j < 7; ++j) s[0] += big[j][0] + big[j][15];
     for (int i = 0; i < 2; ++i)
         for (int j = 0; j < 7; ++j) s += acc[i][j];
     if (s[0] == 12345.678f) out[threadIdx.x] = s[1];   // keeps the accumulators alive; never true in practice
@@ -113,6 +124,8 @@ int main()
     for (int rep = 0; rep < 2 && !rc; ++rep) {
         rc |= run<kBf16Const>("bf16 16x16x32, constant operands", out, stamps, 20000, 16384.0, 16);
         rc |= run<kBf16Random>("bf16 16x16x32, random operands", out, stamps, 20000, 16384.0, 16);
+        rc |= run<kBf16x32Const>("bf16 32x32x16, constant operands", out, stamps, 20000, 16384.0, 16);
+        rc |= run<kBf16x32Random>("bf16 32x32x16, random operands", out, stamps, 20000, 16384.0, 16);
         rc |= run<kF32Const>("f32 16x16x4, constant operands", out, stamps, 10000, 2048.0, 32);
         rc |= run<kF32Random>("f32 16x16x4, random operands", out, stamps, 10000, 2048.0, 32);
     }
