@@ -17,7 +17,7 @@ using namespace bfuse;
 
 BFUSE_MODULE_PROLOGUE()
 
-using GemmS1 = GemmF32<64, 48, 32, 16, 48, 1>;                        // one wave, 16-column groups only
+using GemmS1 = GemmF32<64, 48, 32, 16, 48, 1>;                        // one wave, a 32- and a 16-column group
 using GemmS2 = GemmF32<96, 192, 128, 32, 64, 2, kEpiGeluTanh, 3>;     // 2 waves, GELU, 3 register stages
 using GemmS3 = GemmF32<32, 144, 256, 32, 144, 4>;                     // the 64+64+16 column split, one tile
 using GemmS4 = GemmF32Lds<128, 192, 160, 64, 96, 48, kEpiNone, 3>;          // LDS-staged, 2x2 tiles, five K-steps

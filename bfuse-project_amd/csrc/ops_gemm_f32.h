@@ -17,8 +17,9 @@
 //     B[k+4kq+t][n0+4j .. n0+4j+3] (t = 0..3) with one 128-bit load each.  Component e of
 //     those vectors feeds 16x16 block e of the group, whose column j therefore is global
 //     column n0+4j+e: after the MFMAs a lane holds four consecutive columns of a row and
-//     stores them with one 128-bit store.  A trailing group of 16 columns (BN % 64 == 16)
-//     uses 32-bit loads/stores.
+//     stores them with one 128-bit store.  A trailing group of 32 columns works the same way
+//     with 64-bit loads and two blocks (lane j: columns 2j, 2j+1), a trailing group of 16
+//     columns uses 32-bit loads/stores.
 //   * lane (i = lane%16, kq) loads A[m0+i][k+4kq .. k+4kq+3]; component t is the A operand of
 //     MFMA step t, matching B row k+4kq+t above (the instruction sums over kq).
 #pragma once
@@ -30,6 +31,7 @@
 namespace bfuse {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 enum Epilogue : int { kEpiNone = 0, kEpiGeluTanh = 1 };
 
@@ -53,7 +55,9 @@ struct GemmF32 {
     static constexpr int M = M_, N = N_, K = K_, BM = BM_, BN = BN_, KS = KS_, EPI = EPI_;
     static constexpr int TM = BM / 16;          // 16-row blocks per tile
     static constexpr int G4 = BN / 64;          // 64-column groups
-    static constexpr int G1 = (BN % 64) / 16;   // trailing 16-column groups
+    static constexpr int G2 = (BN % 64) / 32;   // trailing 32-column group
+    static constexpr int G1 = (BN % 32) / 16;   // trailing 16-column group
+    static constexpr int NB = 4 * G4 + 2 * G2 + G1;   // 16 x 16 accumulator blocks per row block
     static constexpr int KW = K / KS;           // k-range of one wave
     static constexpr int STAGE = 16;            // k per stage (one 128-bit A load)
     static constexpr int NSTAGE = KW / STAGE;
@@ -67,16 +71,17 @@ struct GemmF32 {
     static constexpr Dims3 BLOCK{64 * KS, 1, 1};
     static constexpr int THREADS = 64 * KS;
     static constexpr bool HAS_BARRIERS = KS > 1;
-    static constexpr int NUNIT = TM * (G4 + G1);  // reduction / store units (one column group of one row block)
+    static constexpr int NUNIT = TM * (G4 + G2 + G1);  // reduction / store units (one column group of one row block)
 
     // partial tiles of every wave, in accumulator layout
     struct Smem {
-        f32x4 part[KS > 1 ? KS : 1][KS > 1 ? TM * (4 * G4 + G1) : 1][64];
+        f32x4 part[KS > 1 ? KS : 1][KS > 1 ? TM * NB : 1][64];
     };
 
     struct Frag {
         f32x4 a[TM];
         f32x4 b4[G4 > 0 ? G4 : 1][4];  // [group][t] -> 4 columns
+        f32x2 b2[G2 > 0 ? G2 : 1][4];  // [group][t] -> 2 columns
         float b1[G1 > 0 ? G1 : 1][4];  // [group][t]
     };
 
@@ -90,6 +95,7 @@ struct GemmF32 {
         const int i = lane & 15, kq = lane >> 4;
         const unsigned a_off = (unsigned)(i * K + 4 * kq) * 4u;            // bytes
         const unsigned b_off = (unsigned)(4 * kq * N + 4 * i) * 4u;
+        const unsigned b2_off = (unsigned)(4 * kq * N + 2 * i) * 4u;
         const unsigned b1_off = (unsigned)(4 * kq * N + i) * 4u;
         const char* a_ub = reinterpret_cast<const char*>(A + (size_t)m0 * K + k);
         const char* b_ub = reinterpret_cast<const char*>(B + (size_t)k * N + n0);
@@ -102,13 +108,18 @@ struct GemmF32 {
             for (int t = 0; t < 4; ++t)
                 f.b4[g][t] = *reinterpret_cast<const f32x4*>(b_ub + ((size_t)t * N + g * 64) * 4 + b_off);
 #pragma unroll
+        for (int g = 0; g < G2; ++g)
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                f.b2[g][t] = *reinterpret_cast<const f32x2*>(b_ub + ((size_t)t * N + G4 * 64 + g * 32) * 4 + b2_off);
+#pragma unroll
         for (int g = 0; g < G1; ++g)
 #pragma unroll
             for (int t = 0; t < 4; ++t)
-                f.b1[g][t] = *reinterpret_cast<const float*>(b_ub + ((size_t)t * N + G4 * 64 + g * 16) * 4 + b1_off);
+                f.b1[g][t] = *reinterpret_cast<const float*>(b_ub + ((size_t)t * N + G4 * 64 + G2 * 32 + g * 16) * 4 + b1_off);
     }
 
-    __device__ static __forceinline__ void mma_stage(f32x4 (&acc)[TM][4 * G4 + G1], const Frag& f)
+    __device__ static __forceinline__ void mma_stage(f32x4 (&acc)[TM][NB], const Frag& f)
     {
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
@@ -121,9 +132,15 @@ struct GemmF32 {
                         acc[tm][4 * g + e] = __builtin_amdgcn_mfma_f32_16x16x4f32(
                             f.a[tm][t], f.b4[g][t][e], acc[tm][4 * g + e], 0, 0, 0);
 #pragma unroll
+                for (int g = 0; g < G2; ++g)
+#pragma unroll
+                    for (int e = 0; e < 2; ++e)
+                        acc[tm][4 * G4 + 2 * g + e] = __builtin_amdgcn_mfma_f32_16x16x4f32(
+                            f.a[tm][t], f.b2[g][t][e], acc[tm][4 * G4 + 2 * g + e], 0, 0, 0);
+#pragma unroll
                 for (int g = 0; g < G1; ++g)
-                    acc[tm][4 * G4 + g] = __builtin_amdgcn_mfma_f32_16x16x4f32(
-                        f.a[tm][t], f.b1[g][t], acc[tm][4 * G4 + g], 0, 0, 0);
+                    acc[tm][4 * G4 + 2 * G2 + g] = __builtin_amdgcn_mfma_f32_16x16x4f32(
+                        f.a[tm][t], f.b1[g][t], acc[tm][4 * G4 + 2 * G2 + g], 0, 0, 0);
             }
         }
     }
@@ -150,13 +167,25 @@ struct GemmF32 {
             *reinterpret_cast<f32x4*>(C + (size_t)(m0 + tm * 16 + 4 * rg + v) * N + n0 + g * 64 + 4 * j) = o;
         }
     }
+    __device__ static __forceinline__ void store_group2(float* __restrict__ C, int m0, int n0, int tm,
+                                                        int g, const f32x4 (&blk)[2], int lane)
+    {
+        const int j = lane & 15, rg = lane >> 4;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            f32x2 o;
+            o[0] = epilogue(blk[0][v]);
+            o[1] = epilogue(blk[1][v]);
+            *reinterpret_cast<f32x2*>(C + (size_t)(m0 + tm * 16 + 4 * rg + v) * N + n0 + G4 * 64 + g * 32 + 2 * j) = o;
+        }
+    }
     __device__ static __forceinline__ void store_group1(float* __restrict__ C, int m0, int n0, int tm,
                                                         int g, const f32x4& blk, int lane)
     {
         const int j = lane & 15, rg = lane >> 4;
 #pragma unroll
         for (int v = 0; v < 4; ++v)
-            C[(size_t)(m0 + tm * 16 + 4 * rg + v) * N + n0 + G4 * 64 + g * 16 + j] = epilogue(blk[v]);
+            C[(size_t)(m0 + tm * 16 + 4 * rg + v) * N + n0 + G4 * 64 + G2 * 32 + g * 16 + j] = epilogue(blk[v]);
     }
 
     template <class Sync>
@@ -171,11 +200,11 @@ struct GemmF32 {
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;   // wave-uniform: addresses built on it stay in scalar registers
         const int kbeg = wave * KW;
 
-        f32x4 acc[TM][4 * G4 + G1];
+        f32x4 acc[TM][NB];
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm)
 #pragma unroll
-            for (int c = 0; c < 4 * G4 + G1; ++c) acc[tm][c] = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int c = 0; c < NB; ++c) acc[tm][c] = f32x4{0.f, 0.f, 0.f, 0.f};
 
         Frag buf[NBUF];
 #pragma unroll
@@ -207,10 +236,14 @@ struct GemmF32 {
                     store_group4(C, m0, n0, tm, g, blk, lane);
                 }
 #pragma unroll
-                for (int g = 0; g < G1; ++g) store_group1(C, m0, n0, tm, g, acc[tm][4 * G4 + g], lane);
+                for (int g = 0; g < G2; ++g) {
+                    const f32x4 blk[2] = {acc[tm][4 * G4 + 2 * g], acc[tm][4 * G4 + 2 * g + 1]};
+                    store_group2(C, m0, n0, tm, g, blk, lane);
+                }
+#pragma unroll
+                for (int g = 0; g < G1; ++g) store_group1(C, m0, n0, tm, g, acc[tm][4 * G4 + 2 * G2 + g], lane);
             }
         } else {
-            constexpr int NB = 4 * G4 + G1;
 #pragma unroll
             for (int tm = 0; tm < TM; ++tm)
 #pragma unroll
@@ -221,7 +254,7 @@ struct GemmF32 {
             for (int u0 = 0; u0 < NUNIT; u0 += KS) {
                 const int u = u0 + wave;
                 if (u < NUNIT) {
-                    const int tm = u / (G4 + G1), g = u % (G4 + G1);
+                    const int tm = u / (G4 + G2 + G1), g = u % (G4 + G2 + G1);
                     if (g < G4) {
                         f32x4 blk[4];
 #pragma unroll
@@ -232,11 +265,22 @@ struct GemmF32 {
                             blk[e] = s;
                         }
                         store_group4(C, m0, n0, tm, g, blk, lane);
-                    } else {
-                        f32x4 s = sm.part[0][tm * NB + 4 * G4 + (g - G4)][lane];
+                    } else if (g < G4 + G2) {
+                        f32x4 blk[2];
 #pragma unroll
-                        for (int w = 1; w < KS; ++w) s += sm.part[w][tm * NB + 4 * G4 + (g - G4)][lane];
-                        store_group1(C, m0, n0, tm, g - G4, s, lane);
+                        for (int e = 0; e < 2; ++e) {
+                            f32x4 s = sm.part[0][tm * NB + 4 * G4 + 2 * (g - G4) + e][lane];
+#pragma unroll
+                            for (int w = 1; w < KS; ++w) s += sm.part[w][tm * NB + 4 * G4 + 2 * (g - G4) + e][lane];
+                            blk[e] = s;
+                        }
+                        store_group2(C, m0, n0, tm, g - G4, blk, lane);
+                    } else {
+                        const int b = 4 * G4 + 2 * G2 + (g - G4 - G2);
+                        f32x4 s = sm.part[0][tm * NB + b][lane];
+#pragma unroll
+                        for (int w = 1; w < KS; ++w) s += sm.part[w][tm * NB + b][lane];
+                        store_group1(C, m0, n0, tm, g - G4 - G2, s, lane);
                     }
                 }
             }

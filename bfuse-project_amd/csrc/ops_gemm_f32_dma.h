@@ -38,8 +38,6 @@
 
 namespace bfuse {
 
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-
 //
 // PW_ = 1 adds one producer wave per k-range: it issues that range's direct-to-LDS loads and the
 // compute wave issues only LDS reads and MFMAs.  Producer and compute waves meet at one workgroup
