@@ -23,9 +23,7 @@ BFUSE_BFUSE_RT_KERNEL(gemm_f32_512x512x512, Gemm512, bias_relu_1048576, BiasRelu
 // four and eight waves split K (one or two per SIMD): the 128-thread split of the configuration leaves two SIMDs idle
 using Gemm512K4 = GemmF32<512, 512, 512, 16, 64, 4>;
 using Gemm512K8 = GemmF32<512, 512, 512, 16, 64, 8>;
-using Gemm512K4s = GemmF32<512, 512, 512, 16, 64, 4, kEpiNone, 2, 0>;
 BFUSE_KERNEL(gemm_f32_512x512x512_k4, Gemm512K4, ({{512, 512, 1, 1}, 4}), ({{512, 512, 1, 1}, 4}), ({{512, 512, 1, 1}, 4}))
 BFUSE_KERNEL(gemm_f32_512x512x512_k8, Gemm512K8, ({{512, 512, 1, 1}, 4}), ({{512, 512, 1, 1}, 4}), ({{512, 512, 1, 1}, 4}))
-BFUSE_KERNEL(gemm_f32_512x512x512_k4s, Gemm512K4s, ({{512, 512, 1, 1}, 4}), ({{512, 512, 1, 1}, 4}), ({{512, 512, 1, 1}, 4}))
 BFUSE_HFUSE_KERNEL(gemm_f32_512x512x512_k4, Gemm512K4, bias_relu_1048576, BiasRelu1M)
 BFUSE_HFUSE_KERNEL(gemm_f32_512x512x512_k8, Gemm512K8, bias_relu_1048576, BiasRelu1M)

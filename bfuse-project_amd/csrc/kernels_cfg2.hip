@@ -22,10 +22,6 @@ using LnBert1 = LayerNorm<512, 768, 1, 1>;
 BFUSE_KERNEL(layernorm_512x768_w2, LnBert2, ({{512, 768, 1, 1}, 4}), ({{2, 768, 1, 1}, 4}), ({{512, 768, 1, 1}, 4}))
 BFUSE_KERNEL(layernorm_512x768_w1, LnBert1, ({{512, 768, 1, 1}, 4}), ({{2, 768, 1, 1}, 4}), ({{512, 768, 1, 1}, 4}))
 
-using GemmQkvS0 = GemmF32<512, 2304, 768, 32, 144, 4, kEpiNone, 2, 0>;
-using GemmQkvS0p3 = GemmF32<512, 2304, 768, 32, 144, 4, kEpiNone, 3, 0>;
-BFUSE_KERNEL(gemm_f32_512x768x2304_s0, GemmQkvS0, ({{512, 768, 1, 1}, 4}), ({{768, 2304, 1, 1}, 4}), ({{512, 2304, 1, 1}, 4}))
-BFUSE_KERNEL(gemm_f32_512x768x2304_s0p3, GemmQkvS0p3, ({{512, 768, 1, 1}, 4}), ({{768, 2304, 1, 1}, 4}), ({{512, 2304, 1, 1}, 4}))
 BFUSE_BFUSE_KERNEL(gemm_f32_512x768x2304, GemmQkv, layernorm_512x768_w2, LnBert2, _r, bfuse::kRanges, 0, 0)
 BFUSE_BFUSE_KERNEL(gemm_f32_512x768x2304, GemmQkv, layernorm_512x768_w1, LnBert1, _r, bfuse::kRanges, 0, 0)
 BFUSE_HFUSE_KERNEL(gemm_f32_512x768x2304, GemmQkv, layernorm_512x768_w2, LnBert2)

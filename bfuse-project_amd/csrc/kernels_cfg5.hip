@@ -14,23 +14,19 @@ BFUSE_MODULE_PROLOGUE()
 using GemmGate = GemmBf16NTDma<512, 14336, 4096, 128, 224, 3, 4>;   // 4 x 64 = 256 workgroups, direct-to-LDS ring
 using GemmGate8 = GemmBf16NTDma<512, 14336, 4096, 128, 224, 3, 4, 4, 2>;   // same tiles, eight waves of 32 x 112 (two per SIMD)
 using GemmGateP = GemmBf16NTDma<512, 14336, 4096, 128, 224, 3, 4, 4, 2, 4>;   // eight compute waves + four producer waves that issue the loads
-using GemmGateP4 = GemmBf16NTDma<512, 14336, 4096, 128, 224, 3, 4, 2, 2, 4>;  // four compute waves (64 x 112) + four producer waves
 using GemmGateX = GemmBf16NT32<512, 14336, 4096, 128, 224, 3, 3, 4>;   // 32x32x16 MFMAs: waves of 32 x 128 and 32 x 96, four producer waves
 using GemmGateR = GemmBf16NTRing<512, 14336, 4096, 128, 224, 7, 4, 2>;     // 32-k stages in a ring of seven, barrier inside the stage, continuous MFMA stream
 using GemmGateV = GemmBf16NT<512, 14336, 4096, 128, 224>;           // same tiles, operands staged through VGPRs
 using NormRope1 = RmsNormRope<512, 32, 128, 1>;             // 512 one-wave workgroups
-using NormRope2 = RmsNormRope<512, 32, 128, 2>;             // 256 two-wave workgroups: one per GEMM tile under thread-level fusion
 using NormRope4 = RmsNormRope<512, 32, 128, 4>;             // 128 four-wave workgroups
 
 BFUSE_KERNEL(gemm_bf16_512x4096x14336, GemmGate, ({{512, 4096, 1, 1}, 2}), ({{14336, 4096, 1, 1}, 2}), ({{512, 14336, 1, 1}, 2}))
 BFUSE_KERNEL(gemm_bf16_512x4096x14336_w8, GemmGate8, ({{512, 4096, 1, 1}, 2}), ({{14336, 4096, 1, 1}, 2}), ({{512, 14336, 1, 1}, 2}))
 BFUSE_KERNEL(gemm_bf16_512x4096x14336_p, GemmGateP, ({{512, 4096, 1, 1}, 2}), ({{14336, 4096, 1, 1}, 2}), ({{512, 14336, 1, 1}, 2}))
-BFUSE_KERNEL(gemm_bf16_512x4096x14336_p4, GemmGateP4, ({{512, 4096, 1, 1}, 2}), ({{14336, 4096, 1, 1}, 2}), ({{512, 14336, 1, 1}, 2}))
 BFUSE_KERNEL(gemm_bf16_512x4096x14336_x, GemmGateX, ({{512, 4096, 1, 1}, 2}), ({{14336, 4096, 1, 1}, 2}), ({{512, 14336, 1, 1}, 2}))
 BFUSE_KERNEL(gemm_bf16_512x4096x14336_r, GemmGateR, ({{512, 4096, 1, 1}, 2}), ({{14336, 4096, 1, 1}, 2}), ({{512, 14336, 1, 1}, 2}))
 BFUSE_KERNEL(gemm_bf16_512x4096x14336_v, GemmGateV, ({{512, 4096, 1, 1}, 2}), ({{14336, 4096, 1, 1}, 2}), ({{512, 14336, 1, 1}, 2}))
 BFUSE_KERNEL(rmsnorm_rope_bf16_512x4096, NormRope1, ({{512, 4096, 1, 1}, 2}), ({{(int)NormRope1::F_BYTES, 1, 1, 1}, 1}), ({{512, 4096, 1, 1}, 2}))
-BFUSE_KERNEL(rmsnorm_rope_bf16_512x4096_w2, NormRope2, ({{512, 4096, 1, 1}, 2}), ({{(int)NormRope2::F_BYTES, 1, 1, 1}, 1}), ({{512, 4096, 1, 1}, 2}))
 BFUSE_KERNEL(rmsnorm_rope_bf16_512x4096_w4, NormRope4, ({{512, 4096, 1, 1}, 2}), ({{(int)NormRope4::F_BYTES, 1, 1, 1}, 1}), ({{512, 4096, 1, 1}, 2}))
 
 BFUSE_BFUSE_KERNEL(gemm_bf16_512x4096x14336, GemmGate, rmsnorm_rope_bf16_512x4096, NormRope1, , bfuse::kZigzag, 1, 1)
