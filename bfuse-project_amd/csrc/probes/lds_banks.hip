@@ -18,11 +18,11 @@ typedef __attribute__((address_space(3))) unsigned char lds_u8;
 enum Op { kR32, kR64, kR128, kW32, kW64, kW128 };
 
 template <int OP>
-__global__ __launch_bounds__(256) void hammer(const unsigned* __restrict__ offs, unsigned long long* stamps, float* out, int iters)
+__global__ __launch_bounds__(1024) void hammer(const unsigned* __restrict__ offs, unsigned long long* stamps, float* out, int iters)
 {
     __shared__ __attribute__((aligned(1024))) unsigned char lds[65536];
     const int lane = threadIdx.x & 63;
-    for (int i = threadIdx.x; i < 65536 / 4; i += 256) reinterpret_cast<float*>(lds)[i] = 0.f;
+    for (int i = threadIdx.x; i < 65536 / 4; i += blockDim.x) reinterpret_cast<float*>(lds)[i] = 0.f;
     __syncthreads();
     const unsigned a = (unsigned)(size_t)(lds_u8*)lds + offs[lane];
     f32x4 v[8];
@@ -61,7 +61,7 @@ __global__ __launch_bounds__(256) void hammer(const unsigned* __restrict__ offs,
 static unsigned* d_offs; static unsigned long long* d_stamps; static float* d_out;
 
 template <int OP>
-int run(const char* label, int width, const std::function<unsigned(int)>& f)
+int run(const char* label, int width, const std::function<unsigned(int)>& f, int waves = 4)
 {
     unsigned h[64];
     for (int l = 0; l < 64; ++l) {
@@ -70,29 +70,31 @@ int run(const char* label, int width, const std::function<unsigned(int)>& f)
     }
     CHECK(hipMemcpy(d_offs, h, sizeof(h), hipMemcpyHostToDevice));
     constexpr int kIters = 2000;
-    hammer<OP><<<1, 256>>>(d_offs, d_stamps, d_out, 200);
+    hammer<OP><<<1, 64 * waves>>>(d_offs, d_stamps, d_out, 200);
     CHECK(hipDeviceSynchronize());
-    hammer<OP><<<1, 256>>>(d_offs, d_stamps, d_out, kIters);
+    hammer<OP><<<1, 64 * waves>>>(d_offs, d_stamps, d_out, kIters);
     CHECK(hipDeviceSynchronize());
-    unsigned long long s[4];
-    CHECK(hipMemcpy(s, d_stamps, sizeof(s), hipMemcpyDeviceToHost));
+    unsigned long long s[16];
+    CHECK(hipMemcpy(s, d_stamps, sizeof(unsigned long long) * waves, hipMemcpyDeviceToHost));
     double m = 0;
-    for (int i = 0; i < 4; ++i) m = s[i] > m ? (double)s[i] : m;
-    // four waves share the LDS: clocks per instruction of the CU's LDS
-    std::printf("%-74s %6.2f clk / wave instruction\n", label, m / (kIters * 8.0 * 4.0));
+    for (int i = 0; i < waves; ++i) m = s[i] > m ? (double)s[i] : m;
+    // the waves share the LDS: clocks per instruction of the CU's LDS
+    std::printf("%-74s %6.2f clk / wave instruction\n", label, m / (kIters * 8.0 * waves));
     return 0;
 }
 
 int main()
 {
     CHECK(hipMalloc(&d_offs, 256));
-    CHECK(hipMalloc(&d_stamps, 64));
+    CHECK(hipMalloc(&d_stamps, 256));
     CHECK(hipMalloc(&d_out, 4096));
     int rc = 0;
     auto li = [](int l) { return l & 15; };
     auto kq = [](int l) { return l >> 4; };
     // ---- 128-bit reads
     rc |= run<kR128>("b128 read   contiguous: lane*16", 16, [&](int l) { return l * 16u; });
+    rc |= run<kR128>("b128 read   contiguous, 8 waves", 16, [&](int l) { return l * 16u; }, 8);
+    rc |= run<kR128>("b128 read   contiguous, 12 waves", 16, [&](int l) { return l * 16u; }, 12);
     rc |= run<kR128>("b128 read   all lanes one address", 16, [&](int l) { return 0u; });
     rc |= run<kR128>("b128 read   lane*32 (every other slot)", 16, [&](int l) { return l * 32u; });
     for (unsigned pitch : {1024u, 1152u, 1536u, 1024u + 16, 1024u + 32, 1024u + 64, 1024u + 128})
@@ -123,6 +125,7 @@ int main()
     rc |= run<kW32>("b32 write   conv staging, chunk index fastest: cl = lane%16", 4, [&](int l) { int cl = l & 15, c4 = l >> 4; return (cl / 4) * 3072u + c4 * 64u + (cl % 4) * 4u; });
     rc |= run<kW64>("b64 write   contiguous: lane*8", 8, [&](int l) { return l * 8u; });
     rc |= run<kW128>("b128 write  contiguous: lane*16", 16, [&](int l) { return l * 16u; });
+    rc |= run<kW128>("b128 write  contiguous, 8 waves", 16, [&](int l) { return l * 16u; }, 8);
     rc |= run<kW128>("b128 write  lane*32", 16, [&](int l) { return l * 32u; });
     return rc;
 }
