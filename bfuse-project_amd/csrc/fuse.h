@@ -29,6 +29,7 @@
 
 #include <cstring>
 #include <string>
+#include <type_traits>
 #include <vector>
 
 #include "dispatch.h"
@@ -128,6 +129,12 @@ __device__ __forceinline__ void bfuse_rt_body(const BlockPlan& plan, const void*
     }
 }
 
+// does the operator take a workgroup barrier inside its main loop (it says so with LOOP_BARRIERS)?
+template <class Op, class = void>
+struct loop_barriers : std::false_type {};
+template <class Op>
+struct loop_barriers<Op, std::void_t<decltype(Op::LOOP_BARRIERS)>> : std::bool_constant<Op::LOOP_BARRIERS> {};
+
 template <class A, class B>
 struct HfusePair {
     static constexpr LaunchDims dims[2] = {{A::GRID, A::BLOCK}, {B::GRID, B::BLOCK}};
@@ -152,15 +159,17 @@ __device__ __forceinline__ void hfuse_body(const void* I1, const void* F1, void*
     __syncthreads();
     int local = 0;
     const int kernel_id = map_thread(plan, (int)blockIdx.x, (int)threadIdx.x, &local);
-    // A side whose partner has no barriers keeps the hardware barrier: s_barrier counts the waves
+    // A side whose partner has no barriers can keep the hardware barrier: s_barrier counts the waves
     // of the workgroup that are still alive, the partner's waves never take part and leave when
-    // they are done, so the worst case is that this side's first barrier waits for them.  Only when
-    // BOTH sides synchronise do they need barriers of their own (the LDS arrival counters).
+    // they are done -- so this side's FIRST barrier waits until they have left.  That is free for a
+    // side that synchronises only in its epilogue (the split-K GEMMs, the convolutions) and would
+    // serialise the two sides if the barrier sat in the K loop: such a side (LOOP_BARRIERS), and
+    // both sides whenever both synchronise, get barriers of their own (the LDS arrival counters).
     if (kernel_id == 0) {
-        if constexpr (!B::HAS_BARRIERS) A::run((int)blockIdx.x, local, ss.a, I1, F1, O1, BlockSync{});
+        if constexpr (!B::HAS_BARRIERS && !loop_barriers<A>::value) A::run((int)blockIdx.x, local, ss.a, I1, F1, O1, BlockSync{});
         else A::run((int)blockIdx.x, local, ss.a, I1, F1, O1, GroupSync{&ss.arrive[0], (unsigned)(round_up(A::THREADS, kWaveSize) / kWaveSize), 0u});
     } else if (kernel_id == 1) {
-        if constexpr (!A::HAS_BARRIERS) B::run((int)blockIdx.x, local, ss.b, I2, F2, O2, BlockSync{});
+        if constexpr (!A::HAS_BARRIERS && !loop_barriers<B>::value) B::run((int)blockIdx.x, local, ss.b, I2, F2, O2, BlockSync{});
         else B::run((int)blockIdx.x, local, ss.b, I2, F2, O2, GroupSync{&ss.arrive[1], (unsigned)(round_up(B::THREADS, kWaveSize) / kWaveSize), 0u});
     }
 }

@@ -61,6 +61,7 @@ struct GemmBf16NT {
     static constexpr Dims3 GRID{MT * NT, 1, 1};
     static constexpr Dims3 BLOCK{THREADS, 1, 1};
     static constexpr bool HAS_BARRIERS = true;
+    static constexpr bool LOOP_BARRIERS = true;   // one workgroup barrier per K-stage, not only in the epilogue
 
     static constexpr int STAGE_ELEMS = (BM + BN) * PITCH;
     static constexpr int EPI_ELEMS = BM * CPITCH;
@@ -211,6 +212,7 @@ struct GemmBf16NTDma {
     static constexpr Dims3 GRID{MT * NT, 1, 1};
     static constexpr Dims3 BLOCK{THREADS, 1, 1};
     static constexpr bool HAS_BARRIERS = true;
+    static constexpr bool LOOP_BARRIERS = true;   // one workgroup barrier per K-stage, not only in the epilogue
     static constexpr int EPI_BYTES = BM * CPITCH * 2;
     struct Smem {
         __attribute__((aligned(1024))) unsigned char t[((NSTG * STAGE_BYTES > EPI_BYTES) ? NSTG * STAGE_BYTES : EPI_BYTES)];

@@ -64,6 +64,7 @@ struct GemmBf16NTRing {
     static constexpr Dims3 GRID{MT * NT, 1, 1};
     static constexpr Dims3 BLOCK{THREADS, 1, 1};
     static constexpr bool HAS_BARRIERS = true;
+    static constexpr bool LOOP_BARRIERS = true;   // one workgroup barrier per K-stage, not only in the epilogue
     static constexpr int EPI_BYTES = BM * CPITCH * 2;
     static_assert(NSTG * STAGE_BYTES <= 160 * 1024 && EPI_BYTES <= 160 * 1024, "LDS");
     struct Smem {

@@ -60,6 +60,7 @@ struct GemmBf16NT32 {
     static constexpr Dims3 GRID = Base::GRID;
     static constexpr Dims3 BLOCK = Base::BLOCK;
     static constexpr bool HAS_BARRIERS = true;
+    static constexpr bool LOOP_BARRIERS = true;   // one workgroup barrier per K-stage, not only in the epilogue
     using Smem = typename Base::Smem;
     using Src = typename Base::Src;
     typedef __attribute__((address_space(3))) unsigned char lds_u8;

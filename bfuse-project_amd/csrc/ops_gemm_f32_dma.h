@@ -74,6 +74,7 @@ struct GemmF32Dma {
     static constexpr Dims3 BLOCK{64 * NW, 1, 1};
     static constexpr int THREADS = 64 * NW;
     static constexpr bool HAS_BARRIERS = NW > 1;
+    static constexpr bool LOOP_BARRIERS = PW_ > 0;   // producer mode: one workgroup barrier per K-stage
     static constexpr int NUNIT = TM * (G4 + G1);
     static constexpr int RING_BYTES = KS * WAVE_BYTES;
     // The partial tiles meet in LDS in ROUNDS rounds of TMR row blocks each, so that the reduction

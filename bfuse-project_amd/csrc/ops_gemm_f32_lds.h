@@ -49,6 +49,7 @@ struct GemmF32Lds {
     static constexpr Dims3 GRID{N / BN, M / BM, 1};
     static constexpr Dims3 BLOCK{THREADS, 1, 1};
     static constexpr bool HAS_BARRIERS = true;
+    static constexpr bool LOOP_BARRIERS = true;   // one workgroup barrier per K-stage, not only in the epilogue
 
     struct Smem {
         __attribute__((aligned(1024))) unsigned char t[NSTG * STAGE_BYTES];
