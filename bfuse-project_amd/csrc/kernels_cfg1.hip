@@ -20,10 +20,7 @@ BFUSE_BFUSE_KERNEL(gemm_f32_512x512x512, Gemm512, bias_relu_1048576, BiasRelu1M,
 BFUSE_BFUSE_KERNEL(gemm_f32_512x512x512, Gemm512, bias_relu_1048576, BiasRelu1M, _c8, bfuse::kChunked, 8, 1)
 // the same pair with its dispatch plan as run-time data and persistent workgroups
 BFUSE_BFUSE_RT_KERNEL(gemm_f32_512x512x512, Gemm512, bias_relu_1048576, BiasRelu1M)
-// four and eight waves split K (one or two per SIMD): the 128-thread split of the configuration leaves two SIMDs idle
+// alternative GEMM side: four waves split K (one per SIMD); outside the configuration's 128/128 split
 using Gemm512K4 = GemmF32<512, 512, 512, 16, 64, 4>;
-using Gemm512K8 = GemmF32<512, 512, 512, 16, 64, 8>;
 BFUSE_KERNEL(gemm_f32_512x512x512_k4, Gemm512K4, ({{512, 512, 1, 1}, 4}), ({{512, 512, 1, 1}, 4}), ({{512, 512, 1, 1}, 4}))
-BFUSE_KERNEL(gemm_f32_512x512x512_k8, Gemm512K8, ({{512, 512, 1, 1}, 4}), ({{512, 512, 1, 1}, 4}), ({{512, 512, 1, 1}, 4}))
 BFUSE_HFUSE_KERNEL(gemm_f32_512x512x512_k4, Gemm512K4, bias_relu_1048576, BiasRelu1M)
-BFUSE_HFUSE_KERNEL(gemm_f32_512x512x512_k8, Gemm512K8, bias_relu_1048576, BiasRelu1M)

@@ -2,32 +2,22 @@
 // zig-zag block-fused with a 3x3 stride-2 max-pool on [1,64,112,112].
 #include "fuse.h"
 #include "ops_conv.h"
-#include "ops_conv_lds.h"
+#include "ops_pool.h"
 
 using namespace bfuse;
 
 BFUSE_MODULE_PROLOGUE()
 
-// 16 output channels x 64 (or 32) pixels per workgroup; four waves take one 16-channel group each
-using Conv64 = Conv3x3F32<64, 64, 56, 56, 16, 4, 4>;     // 4 x 49 = 196 workgroups
-using Conv32 = Conv3x3F32<64, 64, 56, 56, 16, 2, 4>;     // 4 x 98 = 392 workgroups
-using Pool = MaxPool3x3S2<64, 112, 112, 256>;            // 196 workgroups
+// 16 output channels x 64 pixels per workgroup; four waves take one 16-channel group each
+using Conv64 = Conv3x3F32Lds<64, 64, 56, 56, 16, 4, 4>;    // 4 x 49 = 196 workgroups, 74 KB
+using Pool = MaxPool3x3S2<64, 112, 112, 256>;              // 196 workgroups
 
 BFUSE_KERNEL(conv3x3_f32_64x56x56_64, Conv64, ({{1, 64, 56, 56}, 4}), ({{64, 64, 3, 3}, 4}), ({{1, 64, 56, 56}, 4}))
-BFUSE_KERNEL(conv3x3_f32_64x56x56_64_h, Conv32, ({{1, 64, 56, 56}, 4}), ({{64, 64, 3, 3}, 4}), ({{1, 64, 56, 56}, 4}))
 BFUSE_KERNEL(maxpool3x3s2_f32_64x112x112, Pool, ({{1, 64, 112, 112}, 4}), ({{1, 1, 1, 1}, 4}), ({{1, 64, 56, 56}, 4}))
 
 BFUSE_BFUSE_KERNEL(conv3x3_f32_64x56x56_64, Conv64, maxpool3x3s2_f32_64x112x112, Pool, , bfuse::kZigzag, 1, 1)
 BFUSE_BFUSE_KERNEL(conv3x3_f32_64x56x56_64, Conv64, maxpool3x3s2_f32_64x112x112, Pool, _c8, bfuse::kChunked, 8, 1)
 BFUSE_BFUSE_KERNEL(conv3x3_f32_64x56x56_64, Conv64, maxpool3x3s2_f32_64x112x112, Pool, _c256, bfuse::kChunked, 256, 1)
 BFUSE_HFUSE_KERNEL(conv3x3_f32_64x56x56_64, Conv64, maxpool3x3s2_f32_64x112x112, Pool)
-BFUSE_BFUSE_KERNEL(conv3x3_f32_64x56x56_64_h, Conv32, maxpool3x3s2_f32_64x112x112, Pool, , bfuse::kZigzag, 1, 1)
-BFUSE_BFUSE_KERNEL(conv3x3_f32_64x56x56_64_h, Conv32, maxpool3x3s2_f32_64x112x112, Pool, _c8, bfuse::kChunked, 8, 1)
 // the same pair with its dispatch plan as run-time data and persistent workgroups
 BFUSE_BFUSE_RT_KERNEL(conv3x3_f32_64x56x56_64, Conv64, maxpool3x3s2_f32_64x112x112, Pool)
-// the image patch staged in per-wave LDS tiles: one 128-bit LDS read per tap and pixel block in the loop
-using Conv64L = Conv3x3F32Lds<64, 64, 56, 56, 16, 4, 4>;    // 196 workgroups, 74 KB
-BFUSE_KERNEL(conv3x3_f32_64x56x56_64_l, Conv64L, ({{1, 64, 56, 56}, 4}), ({{64, 64, 3, 3}, 4}), ({{1, 64, 56, 56}, 4}))
-BFUSE_BFUSE_KERNEL(conv3x3_f32_64x56x56_64_l, Conv64L, maxpool3x3s2_f32_64x112x112, Pool, _c256, bfuse::kChunked, 256, 1)
-BFUSE_HFUSE_KERNEL(conv3x3_f32_64x56x56_64_l, Conv64L, maxpool3x3s2_f32_64x112x112, Pool)
-BFUSE_BFUSE_RT_KERNEL(conv3x3_f32_64x56x56_64_l, Conv64L, maxpool3x3s2_f32_64x112x112, Pool)

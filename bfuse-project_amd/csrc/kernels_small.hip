@@ -5,12 +5,10 @@
 // different grid sizes under horizontal fusion, and the ratio / proportional block patterns.
 #include "fuse.h"
 #include "ops_conv.h"
-#include "ops_conv_lds.h"
 #include "ops_gemm_bf16.h"
-#include "ops_gemm_bf16_ring.h"
 #include "ops_gemm_f32.h"
-#include "ops_gemm_f32_lds.h"
 #include "ops_gemm_f32_dma.h"
+#include "ops_pool.h"
 #include "ops_rowwise.h"
 
 using namespace bfuse;
@@ -20,53 +18,39 @@ BFUSE_MODULE_PROLOGUE()
 using GemmS1 = GemmF32<64, 48, 32, 16, 48, 1>;                        // one wave, a 32- and a 16-column group
 using GemmS2 = GemmF32<96, 192, 128, 32, 64, 2, kEpiGeluTanh, 3>;     // 2 waves, GELU, 3 register stages
 using GemmS3 = GemmF32<32, 144, 256, 32, 144, 4>;                     // the 64+64+16 column split, one tile
-using GemmS4 = GemmF32Lds<128, 192, 160, 64, 96, 48, kEpiNone, 3>;          // LDS-staged, 2x2 tiles, five K-steps
+using GemmS5 = GemmF32Dma<128, 192, 160, 32, 96, 2>;                  // private LDS rings, two waves split K, ten 8-k stages each
+using GemmS6 = GemmF32Dma<64, 288, 192, 32, 144, 4, kEpiGeluTanh>;    // the 32x144 tile (partial last B load), four waves, GELU
 using BiasReluS = BiasRelu<4096, 64, 4>;
 using LayerNormS = LayerNorm<8, 256, 2, 1>;
 using SoftmaxS = SoftmaxCausal<2, 256, 2, 2, 2>;
-using ConvS1 = Conv3x3F32<16, 16, 8, 8, 16, 1, 1>;                     // one channel group, one wave
-using ConvS2 = Conv3x3F32<32, 32, 12, 12, 16, 1, 2>;                   // two channel groups on two waves
-using ConvS3 = Conv3x3F32<64, 16, 8, 16, 16, 2, 2>;                    // two groups per wave, two pixel blocks
-using ConvL1 = Conv3x3F32Lds<16, 16, 8, 8, 16, 1, 1>;                  // the same three shapes with the patch staged in LDS
-using ConvL2 = Conv3x3F32Lds<32, 32, 12, 12, 16, 1, 2>;
-using ConvL3 = Conv3x3F32Lds<64, 16, 8, 16, 16, 2, 2>;
+using ConvS1 = Conv3x3F32Lds<16, 16, 8, 8, 16, 1, 1>;                 // one channel group, one wave
+using ConvS2 = Conv3x3F32Lds<32, 32, 12, 12, 16, 1, 2>;               // two channel groups on two waves
+using ConvS3 = Conv3x3F32Lds<64, 16, 8, 16, 16, 2, 2>;                // two groups per wave, two pixel blocks
 using PoolS = MaxPool3x3S2<4, 16, 16, 64>;
-using GemmB1 = GemmBf16NT<128, 1792, 64, 128, 224>;                   // one K-step
-using GemmB2 = GemmBf16NT<256, 1792, 192, 128, 224>;                  // two M-tiles, three K-steps
-using GemmB3 = GemmBf16NTDma<256, 1792, 320, 128, 224, 3>;             // direct-to-LDS ring, five K-steps
-using GemmB5 = GemmBf16NTDma<256, 1792, 320, 128, 224, 3, 4, 4, 2>;       // the same with eight waves (uneven load groups per wave)
-using GemmB6 = GemmBf16NTRing<256, 1792, 320, 128, 224, 7, 4, 2>;         // ring of seven 32-k stages, ten K-steps, eight waves
-using GemmB7 = GemmBf16NTRing<256, 1792, 320, 128, 224, 4, 2, 2>;         // ring of four, four waves (four A fragments per wave)
-using GemmB8 = GemmBf16NTDma<256, 1792, 384, 128, 224, 3, 4, 4, 2, 4>;    // eight compute + four producer waves
-using GemmB4 = GemmBf16NTDma<128, 1792, 192, 128, 224, 2>;             // two stages, three K-steps
+using GemmB1 = GemmBf16NTDma<128, 1792, 64, 128, 224, 2>;             // one K-step
+using GemmB2 = GemmBf16NTDma<128, 1792, 192, 128, 224, 2>;            // two stages, three K-steps
+using GemmB3 = GemmBf16NTDma<256, 1792, 320, 128, 224, 3>;            // two M-tiles, ring of three, five K-steps
+using GemmB5 = GemmBf16NTDma<256, 1792, 320, 128, 224, 3, 4, 4, 2>;   // the same with eight waves (uneven load groups per wave)
+using GemmB8 = GemmBf16NTDma<256, 1792, 384, 128, 224, 3, 4, 4, 2, 4>;   // eight compute + four producer waves
 using NormRopeS = RmsNormRope<6, 8, 128, 2>;
 
 BFUSE_KERNEL(gemm_f32_64x32x48, GemmS1, ({{64, 32, 1, 1}, 4}), ({{32, 48, 1, 1}, 4}), ({{64, 48, 1, 1}, 4}))
 BFUSE_KERNEL(gemm_gelu_f32_96x128x192, GemmS2, ({{96, 128, 1, 1}, 4}), ({{128, 192, 1, 1}, 4}), ({{96, 192, 1, 1}, 4}))
 BFUSE_KERNEL(gemm_f32_32x256x144, GemmS3, ({{32, 256, 1, 1}, 4}), ({{256, 144, 1, 1}, 4}), ({{32, 144, 1, 1}, 4}))
-using GemmS5 = GemmF32Dma<128, 192, 160, 32, 96, 2>;                       // private LDS rings, two waves split K, ten 8-k stages each
-using GemmS6 = GemmF32Dma<64, 288, 192, 32, 144, 4, kEpiGeluTanh>;         // the 32x144 tile (partial last B load), four waves, GELU
 BFUSE_KERNEL(gemm_f32_128x160x192_d, GemmS5, ({{128, 160, 1, 1}, 4}), ({{160, 192, 1, 1}, 4}), ({{128, 192, 1, 1}, 4}))
 BFUSE_KERNEL(gemm_gelu_f32_64x192x288_d, GemmS6, ({{64, 192, 1, 1}, 4}), ({{192, 288, 1, 1}, 4}), ({{64, 288, 1, 1}, 4}))
-BFUSE_KERNEL(gemm_f32_128x160x192_l, GemmS4, ({{128, 160, 1, 1}, 4}), ({{160, 192, 1, 1}, 4}), ({{128, 192, 1, 1}, 4}))
 BFUSE_KERNEL(bias_relu_4096, BiasReluS, ({{4096, 1, 1, 1}, 4}), ({{4096, 1, 1, 1}, 4}), ({{4096, 1, 1, 1}, 4}))
 BFUSE_KERNEL(layernorm_8x256, LayerNormS, ({{8, 256, 1, 1}, 4}), ({{2, 256, 1, 1}, 4}), ({{8, 256, 1, 1}, 4}))
 BFUSE_KERNEL(softmax_causal_2x256x256, SoftmaxS, ({{2, 256, 256, 1}, 4}), ({{1, 1, 1, 1}, 4}), ({{2, 256, 256, 1}, 4}))
 BFUSE_KERNEL(conv3x3_f32_16x8x8_16, ConvS1, ({{1, 16, 8, 8}, 4}), ({{16, 16, 3, 3}, 4}), ({{1, 16, 8, 8}, 4}))
 BFUSE_KERNEL(conv3x3_f32_32x12x12_32, ConvS2, ({{1, 32, 12, 12}, 4}), ({{32, 32, 3, 3}, 4}), ({{1, 32, 12, 12}, 4}))
 BFUSE_KERNEL(conv3x3_f32_64x8x16_16, ConvS3, ({{1, 64, 8, 16}, 4}), ({{16, 64, 3, 3}, 4}), ({{1, 16, 8, 16}, 4}))
-BFUSE_KERNEL(conv3x3_f32_16x8x8_16_l, ConvL1, ({{1, 16, 8, 8}, 4}), ({{16, 16, 3, 3}, 4}), ({{1, 16, 8, 8}, 4}))
-BFUSE_KERNEL(conv3x3_f32_32x12x12_32_l, ConvL2, ({{1, 32, 12, 12}, 4}), ({{32, 32, 3, 3}, 4}), ({{1, 32, 12, 12}, 4}))
-BFUSE_KERNEL(conv3x3_f32_64x8x16_16_l, ConvL3, ({{1, 64, 8, 16}, 4}), ({{16, 64, 3, 3}, 4}), ({{1, 16, 8, 16}, 4}))
 BFUSE_KERNEL(maxpool3x3s2_f32_4x16x16, PoolS, ({{1, 4, 16, 16}, 4}), ({{1, 1, 1, 1}, 4}), ({{1, 4, 8, 8}, 4}))
 BFUSE_KERNEL(gemm_bf16_128x64x1792, GemmB1, ({{128, 64, 1, 1}, 2}), ({{1792, 64, 1, 1}, 2}), ({{128, 1792, 1, 1}, 2}))
-BFUSE_KERNEL(gemm_bf16_256x192x1792, GemmB2, ({{256, 192, 1, 1}, 2}), ({{1792, 192, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
-BFUSE_KERNEL(gemm_bf16_256x320x1792_d, GemmB3, ({{256, 320, 1, 1}, 2}), ({{1792, 320, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
+BFUSE_KERNEL(gemm_bf16_128x192x1792, GemmB2, ({{128, 192, 1, 1}, 2}), ({{1792, 192, 1, 1}, 2}), ({{128, 1792, 1, 1}, 2}))
+BFUSE_KERNEL(gemm_bf16_256x320x1792, GemmB3, ({{256, 320, 1, 1}, 2}), ({{1792, 320, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
 BFUSE_KERNEL(gemm_bf16_256x320x1792_w8, GemmB5, ({{256, 320, 1, 1}, 2}), ({{1792, 320, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
-BFUSE_KERNEL(gemm_bf16_256x320x1792_r, GemmB6, ({{256, 320, 1, 1}, 2}), ({{1792, 320, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
-BFUSE_KERNEL(gemm_bf16_256x320x1792_r4, GemmB7, ({{256, 320, 1, 1}, 2}), ({{1792, 320, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
 BFUSE_KERNEL(gemm_bf16_256x384x1792_p, GemmB8, ({{256, 384, 1, 1}, 2}), ({{1792, 384, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
-BFUSE_KERNEL(gemm_bf16_128x192x1792_d4, GemmB4, ({{128, 192, 1, 1}, 2}), ({{1792, 192, 1, 1}, 2}), ({{128, 1792, 1, 1}, 2}))
 BFUSE_KERNEL(rmsnorm_rope_bf16_6x1024, NormRopeS, ({{6, 1024, 1, 1}, 2}), ({{(int)NormRopeS::F_BYTES, 1, 1, 1}, 1}), ({{6, 1024, 1, 1}, 2}))
 
 // calibration kernel for the memory counters: 64 MiB read, 64 MiB written
@@ -82,23 +66,18 @@ BFUSE_BFUSE_KERNEL(conv3x3_f32_32x12x12_32, ConvS2, gemm_gelu_f32_96x128x192, Ge
 BFUSE_BFUSE_KERNEL(conv3x3_f32_32x12x12_32, ConvS2, gemm_gelu_f32_96x128x192, GemmS2, _p1, bfuse::kProportional, 1, 1)
 BFUSE_BFUSE_KERNEL(conv3x3_f32_32x12x12_32, ConvS2, gemm_gelu_f32_96x128x192, GemmS2, _c4, bfuse::kChunked, 4, 1)
 BFUSE_BFUSE_KERNEL(layernorm_8x256, LayerNormS, softmax_causal_2x256x256, SoftmaxS, , bfuse::kZigzag, 1, 1)
-BFUSE_BFUSE_KERNEL(gemm_bf16_256x192x1792, GemmB2, rmsnorm_rope_bf16_6x1024, NormRopeS, _c8, bfuse::kChunked, 8, 1)
+BFUSE_BFUSE_KERNEL(gemm_bf16_256x320x1792, GemmB3, rmsnorm_rope_bf16_6x1024, NormRopeS, _c8, bfuse::kChunked, 8, 1)
 BFUSE_HFUSE_KERNEL(maxpool3x3s2_f32_4x16x16, PoolS, layernorm_8x256, LayerNormS)
-// the direct-to-LDS GEMM under horizontal fusion: its fence-free barrier becomes the LDS-counter one
-BFUSE_HFUSE_KERNEL(gemm_f32_128x160x192_l, GemmS4, bias_relu_4096, BiasReluS)
-BFUSE_HFUSE_KERNEL(gemm_bf16_256x320x1792_r, GemmB6, rmsnorm_rope_bf16_6x1024, NormRopeS)
+// a side with a barrier in its K loop under horizontal fusion: its fence-free barriers become the LDS-counter one
+BFUSE_HFUSE_KERNEL(gemm_bf16_256x320x1792_w8, GemmB5, rmsnorm_rope_bf16_6x1024, NormRopeS)
 // run-time plans / persistent workgroups: equal and unequal workgroup widths, barrier-bearing sides
 BFUSE_BFUSE_RT_KERNEL(conv3x3_f32_32x12x12_32, ConvS2, gemm_gelu_f32_96x128x192, GemmS2)
 BFUSE_BFUSE_RT_KERNEL(layernorm_8x256, LayerNormS, softmax_causal_2x256x256, SoftmaxS)
-BFUSE_BFUSE_RT_KERNEL(gemm_bf16_256x320x1792_d, GemmB3, rmsnorm_rope_bf16_6x1024, NormRopeS)
-BFUSE_BFUSE_RT_KERNEL(gemm_f32_128x160x192_l, GemmS4, bias_relu_4096, BiasReluS)
+BFUSE_BFUSE_RT_KERNEL(gemm_bf16_256x320x1792_w8, GemmB5, rmsnorm_rope_bf16_6x1024, NormRopeS)
+BFUSE_BFUSE_RT_KERNEL(gemm_f32_128x160x192_d, GemmS5, bias_relu_4096, BiasReluS)
 BFUSE_HFUSE_KERNEL(gemm_f32_128x160x192_d, GemmS5, bias_relu_4096, BiasReluS)
 BFUSE_BFUSE_KERNEL(gemm_gelu_f32_64x192x288_d, GemmS6, layernorm_8x256, LayerNormS, _c4, bfuse::kChunked, 4, 1)
-using GemmS7 = GemmF32Dma<64, 288, 192, 32, 144, 4, kEpiGeluTanh, 3, 1>;   // four compute + four producer waves
-BFUSE_KERNEL(gemm_gelu_f32_64x192x288_pc, GemmS7, ({{64, 192, 1, 1}, 4}), ({{192, 288, 1, 1}, 4}), ({{64, 288, 1, 1}, 4}))
-BFUSE_BFUSE_KERNEL(gemm_gelu_f32_64x192x288_pc, GemmS7, layernorm_8x256, LayerNormS, _c4, bfuse::kChunked, 4, 1)
-BFUSE_HFUSE_KERNEL(conv3x3_f32_32x12x12_32_l, ConvL2, bias_relu_4096, BiasReluS)
-BFUSE_BFUSE_KERNEL(conv3x3_f32_64x8x16_16_l, ConvL3, layernorm_8x256, LayerNormS, _c4, bfuse::kChunked, 4, 1)
-// both sides synchronise: the LDS-staged GEMM's fence-free barriers and the split-K GEMM's reduction
-// barriers each become LDS arrival counters of their own side
-BFUSE_HFUSE_KERNEL(gemm_f32_128x160x192_l, GemmS4, gemm_gelu_f32_64x192x288_d, GemmS6)
+BFUSE_HFUSE_KERNEL(conv3x3_f32_32x12x12_32, ConvS2, bias_relu_4096, BiasReluS)
+BFUSE_BFUSE_KERNEL(conv3x3_f32_64x8x16_16, ConvS3, layernorm_8x256, LayerNormS, _c4, bfuse::kChunked, 4, 1)
+// both sides synchronise (each split-K GEMM's reduction barriers): each side gets LDS arrival counters of its own
+BFUSE_HFUSE_KERNEL(gemm_f32_128x160x192_d, GemmS5, gemm_gelu_f32_64x192x288_d, GemmS6)

@@ -38,12 +38,9 @@
 
 namespace bfuse {
 
-//
-// PW_ = 1 adds one producer wave per k-range: it issues that range's direct-to-LDS loads and the
-// compute wave issues only LDS reads and MFMAs.  Producer and compute waves meet at one workgroup
-// barrier per K-stage, which costs about what the six loads per stage did: no faster, kept as a
-// tested variant.
-template <int M_, int N_, int K_, int BM_, int BN_, int KS_, int EPI_ = kEpiNone, int NSTG_ = 3, int PW_ = 0>
+// (One producer wave per k-range issuing the loads was tried: it has to meet its compute wave at a
+// workgroup barrier per K-stage, which costs about what the six loads per stage did -- no faster.)
+template <int M_, int N_, int K_, int BM_, int BN_, int KS_, int EPI_ = kEpiNone, int NSTG_ = 3>
 struct GemmF32Dma {
     static constexpr int M = M_, N = N_, K = K_, BM = BM_, BN = BN_, KS = KS_, EPI = EPI_, NSTG = NSTG_;
     static constexpr int TM = BM / 16;
@@ -66,15 +63,12 @@ struct GemmF32Dma {
     static_assert(NSTG >= 2 && NSTAGE >= NSTG, "pipeline shape");
     static_assert((NSTG - 1) * LPS <= 63, "vmcnt range");
     static_assert(NSTG * STAGE_BYTES + BN * 8 + 1024 < 65536, "fragment offsets are 16-bit immediates");
-    static_assert(!(PW_ && KS_ == 1), "producer waves go with a K split");
 
     static constexpr Dims3 GRID{N / BN, M / BM, 1};
-    static constexpr int PW = PW_;
-    static constexpr int NW = KS * (1 + PW_);   // waves in the workgroup
+    static constexpr int NW = KS;   // waves in the workgroup
     static constexpr Dims3 BLOCK{64 * NW, 1, 1};
     static constexpr int THREADS = 64 * NW;
     static constexpr bool HAS_BARRIERS = NW > 1;
-    static constexpr bool LOOP_BARRIERS = PW_ > 0;   // producer mode: one workgroup barrier per K-stage
     static constexpr int NUNIT = TM * (G4 + G1);
     static constexpr int RING_BYTES = KS * WAVE_BYTES;
     // The partial tiles meet in LDS in ROUNDS rounds of TMR row blocks each, so that the reduction
@@ -122,7 +116,7 @@ struct GemmF32Dma {
     template <int I>
     __device__ static __forceinline__ void issue_one(const Ctx& c, int slot, int s)
     {
-        const unsigned dst = c.ring + slot * STAGE_BYTES;   // `slot` is a constant wherever a compute wave calls this
+        const unsigned dst = c.ring + slot * STAGE_BYTES;   // `slot` is a compile-time constant at every call
         if constexpr (I < A_LOADS) {
             dma_load_lds_b128(c.a_voff[I], c.a_ub + (size_t)s * (STAGE * 4), dst + I * 1024);
         } else {
@@ -191,9 +185,9 @@ struct GemmF32Dma {
     __device__ static __forceinline__ void mem_op(int s, Frag& nxt, const Ctx& c)
     {
         if constexpr (OP < LPS) {
-            if constexpr (REFILL && !PW) issue_one<OP>(c, SLOT, s + NSTG);
+            if constexpr (REFILL) issue_one<OP>(c, SLOT, s + NSTG);
         } else if constexpr (OP == LPS) {
-            if constexpr (NEXT && !PW) {
+            if constexpr (NEXT) {
                 if constexpr (REFILL) wait_vm<(NSTG - 1) * LPS>();
                 else wait_vm<0>();
             }
@@ -233,12 +227,9 @@ struct GemmF32Dma {
     // s+NSTG (REFILL: that stage exists), read stage s+1 into `nxt` (NEXT), multiply -- the
     // memory operations dealt between the MFMA groups.  Slot and both flags are compile-time: the
     // body has no branch and no address arithmetic in it.
-    template <int SLOT, bool REFILL, bool NEXT, class Sync>
-    __device__ static __forceinline__ void step(int s, f32x4 (&acc)[TM][NB], Frag& cur, Frag& nxt, const Ctx& c, Sync& sync)
+    template <int SLOT, bool REFILL, bool NEXT>
+    __device__ static __forceinline__ void step(int s, f32x4 (&acc)[TM][NB], Frag& cur, Frag& nxt, const Ctx& c)
     {
-        // barrier of stage s (producer mode): stage s+1 is in LDS (the producers waited for it)
-        // and every compute wave holds stage s in registers, so its slot can be refilled
-        if constexpr (PW) sync.raw();
         groups<0, SLOT, REFILL, NEXT>(s, acc, cur, nxt, c);
         wait_reads(nxt);
     }
@@ -247,22 +238,22 @@ struct GemmF32Dma {
     // bring both back to where they started.
     static constexpr int UNR = NSTG % 2 == 0 ? NSTG : 2 * NSTG;
     static constexpr int MAIN = NSTAGE > NSTG ? ((NSTAGE - NSTG) / UNR) * UNR : 0;   // stages in the rolled loop: all refill
-    template <int J, class Sync>
-    __device__ static __forceinline__ void main_chain(int s0, f32x4 (&acc)[TM][NB], Frag& f0, Frag& f1, const Ctx& c, Sync& sync)
+    template <int J>
+    __device__ static __forceinline__ void main_chain(int s0, f32x4 (&acc)[TM][NB], Frag& f0, Frag& f1, const Ctx& c)
     {
         if constexpr (J < UNR) {
-            if constexpr (J % 2 == 0) step<J % NSTG, true, true>(s0 + J, acc, f0, f1, c, sync);
-            else step<J % NSTG, true, true>(s0 + J, acc, f1, f0, c, sync);
-            main_chain<J + 1>(s0, acc, f0, f1, c, sync);
+            if constexpr (J % 2 == 0) step<J % NSTG, true, true>(s0 + J, acc, f0, f1, c);
+            else step<J % NSTG, true, true>(s0 + J, acc, f1, f0, c);
+            main_chain<J + 1>(s0, acc, f0, f1, c);
         }
     }
-    template <int S, class Sync>
-    __device__ static __forceinline__ void tail_chain(f32x4 (&acc)[TM][NB], Frag& f0, Frag& f1, const Ctx& c, Sync& sync)
+    template <int S>
+    __device__ static __forceinline__ void tail_chain(f32x4 (&acc)[TM][NB], Frag& f0, Frag& f1, const Ctx& c)
     {
         if constexpr (S < NSTAGE) {
-            if constexpr (S % 2 == 0) step<S % NSTG, (S + NSTG < NSTAGE), (S + 1 < NSTAGE)>(S, acc, f0, f1, c, sync);
-            else step<S % NSTG, (S + NSTG < NSTAGE), (S + 1 < NSTAGE)>(S, acc, f1, f0, c, sync);
-            tail_chain<S + 1>(acc, f0, f1, c, sync);
+            if constexpr (S % 2 == 0) step<S % NSTG, (S + NSTG < NSTAGE), (S + 1 < NSTAGE)>(S, acc, f0, f1, c);
+            else step<S % NSTG, (S + NSTG < NSTAGE), (S + 1 < NSTAGE)>(S, acc, f1, f0, c);
+            tail_chain<S + 1>(acc, f0, f1, c);
         }
     }
 
@@ -283,12 +274,10 @@ struct GemmF32Dma {
         const int m0 = vb.y * BM, n0 = vb.x * BN;
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
         const int li = lane & 15, kq = lane >> 4;
-        const bool producer = PW && wave >= KS;
-        const int part = wave < KS ? wave : wave - KS;        // k-range this wave computes or loads
-        const int kbeg = part * KW;
+        const int kbeg = wave * KW;        // k-range this wave accumulates
 
         Ctx c;
-        c.ring = (unsigned)(unsigned long long)(lds_u8*)sm.t + (unsigned)part * WAVE_BYTES;
+        c.ring = (unsigned)(unsigned long long)(lds_u8*)sm.t + (unsigned)wave * WAVE_BYTES;
         c.a_ub = reinterpret_cast<const char*>(A + (size_t)m0 * K + kbeg);
         c.b_ub = reinterpret_cast<const char*>(B + (size_t)kbeg * N + n0);
         // A slot: [BM][8] floats; a wave-level load covers 32 rows (two lanes per 32-byte row)
@@ -316,37 +305,16 @@ struct GemmF32Dma {
             for (int b = 0; b < NB; ++b) acc[tm][b] = f32x4{0.f, 0.f, 0.f, 0.f};
 
         // stages 0 .. NSTG-1 go out; stage 0's fragments are read before the loop
-        if (producer) {
-            // the producer's whole K loop: same barriers as the compute waves, in the same order
+        {
+            Frag f0, f1;
 #pragma unroll
             for (int s = 0; s < NSTG; ++s) issue_all<0>(c, s, s);
             wait_vm<(NSTG - 1) * LPS>();
-            sync.raw();   // stage 0 is in LDS
-            int slot = 0;
-#pragma unroll 1
-            for (int s = 0; s < NSTAGE; ++s) {
-                if (s + 1 < NSTAGE) {
-                    if (s + NSTG - 1 < NSTAGE) wait_vm<(NSTG - 2) * LPS>();
-                    else wait_vm<0>();
-                }
-                sync.raw();
-                if (s + NSTG < NSTAGE) issue_all<0>(c, slot, s + NSTG);
-                slot = slot + 1 == NSTG ? 0 : slot + 1;
-            }
-        } else {
-            Frag f0, f1;
-            if constexpr (!PW) {
-#pragma unroll
-                for (int s = 0; s < NSTG; ++s) issue_all<0>(c, s, s);
-                wait_vm<(NSTG - 1) * LPS>();
-            } else {
-                sync.raw();   // stage 0 is in LDS
-            }
             read_stage<0>(f0, c);
             wait_reads(f0);
 #pragma unroll 1
-            for (int s0 = 0; s0 < MAIN; s0 += UNR) main_chain<0>(s0, acc, f0, f1, c, sync);
-            tail_chain<MAIN>(acc, f0, f1, c, sync);
+            for (int s0 = 0; s0 < MAIN; s0 += UNR) main_chain<0>(s0, acc, f0, f1, c);
+            tail_chain<MAIN>(acc, f0, f1, c);
         }
 
         if constexpr (KS == 1) {
@@ -367,14 +335,12 @@ struct GemmF32Dma {
 #pragma unroll
             for (int r = 0; r < ROUNDS; ++r) {
                 sync();   // first pass: the rings are dead; later passes: the previous sums have been read
-                if (!producer) {
 #pragma unroll
-                    for (int tm = 0; tm < TMR; ++tm)
+                for (int tm = 0; tm < TMR; ++tm)
 #pragma unroll
-                        for (int b = 0; b < NB; ++b) part[wave][tm * NB + b][lane] = acc[r * TMR + tm][b];
-                }
+                    for (int b = 0; b < NB; ++b) part[wave][tm * NB + b][lane] = acc[r * TMR + tm][b];
                 sync();
-                // every wave of the workgroup, producers included, finishes units
+                // every wave of the workgroup finishes units
 #pragma unroll
                 for (int u0 = 0; u0 < NUNIT / ROUNDS; u0 += NW) {
                     const int u = u0 + wave;

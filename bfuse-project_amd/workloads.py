@@ -103,64 +103,35 @@ PAIRS: Dict[int, Pair] = {
     1: Pair(1, "GEMM fp32 512x512x512 || ReLU(x+b) over 1Mi fp32, hfuse 128/128",
             "gemm_f32_512x512x512", "bias_relu_1048576", "hfuse",
             [("hfuse", ""), ("bfuse", ""), ("bfuse", "_c8")],
-            [("gemm_f32_512x512x512_k4", "bias_relu_1048576", "hfuse", ""),
-             ("gemm_f32_512x512x512_k8", "bias_relu_1048576", "hfuse", "")], _pair1_inputs,
+            [("gemm_f32_512x512x512_k4", "bias_relu_1048576", "hfuse", "")], _pair1_inputs,
             bytes1=3 * 512 * 512 * 4, bytes2=3 * 1048576 * 4, flops=2 * 512 ** 3,
             bound="hbm", peak=8000.0, dtype="f32", tol=1e-5),
     2: Pair(2, "GEMM fp32 [512x768].[768x2304] || LayerNorm [512x768], bfuse",
             "gemm_f32_512x768x2304", "layernorm_512x768", "bfuse",
-            [("bfuse", ""), ("bfuse", "_z2"), ("bfuse", "_c8"), ("bfuse", "_r")],
-            [("gemm_f32_512x768x2304", "layernorm_512x768_w2", "bfuse", "_r"),
-             ("gemm_f32_512x768x2304", "layernorm_512x768_w1", "bfuse", "_r"),
-             ("gemm_f32_512x768x2304", "layernorm_512x768_w2", "hfuse", ""),
-             ("gemm_f32_512x768x2304_d", "layernorm_512x768_w1", "bfuse", "_r"),
-             ("gemm_f32_512x768x2304_pc", "layernorm_512x768_w1", "bfuse", "_r")], _pair2_inputs,
+            [("bfuse", "_r"), ("bfuse", ""), ("bfuse", "_c8")],
+            [("gemm_f32_512x768x2304_v", "layernorm_512x768", "bfuse", "_r"),
+             ("gemm_f32_512x768x2304", "layernorm_512x768_w4", "bfuse", "_r")], _pair2_inputs,
             bytes1=(512 * 768 + 768 * 2304 + 512 * 2304) * 4, bytes2=(2 * 512 * 768 + 2 * 768) * 4,
             flops=2 * 512 * 768 * 2304, bound="mfma", peak=157.3, dtype="f32", tol=1e-5),
     3: Pair(3, "conv 3x3 s1 p1 [1,64,56,56]->64 fp32 || max-pool 3x3 s2 p1 [1,64,112,112], zig-zag bfuse",
             "conv3x3_f32_64x56x56_64", "maxpool3x3s2_f32_64x112x112", "bfuse",
-            [("bfuse", ""), ("bfuse", "_c8"), ("bfuse", "_c256"), ("hfuse", "")],
-            [("conv3x3_f32_64x56x56_64_h", "maxpool3x3s2_f32_64x112x112", "bfuse", ""),
-             ("conv3x3_f32_64x56x56_64_h", "maxpool3x3s2_f32_64x112x112", "bfuse", "_c8"),
-             ("conv3x3_f32_64x56x56_64_l", "maxpool3x3s2_f32_64x112x112", "bfuse", "_c256"),
-             ("conv3x3_f32_64x56x56_64_l", "maxpool3x3s2_f32_64x112x112", "hfuse", "")], _pair3_inputs,
+            [("bfuse", "_c256"), ("bfuse", ""), ("bfuse", "_c8"), ("hfuse", "")],
+            [], _pair3_inputs,
             bytes1=(64 * 56 * 56 * 2 + 64 * 64 * 9) * 4, bytes2=(64 * 112 * 112 + 64 * 56 * 56) * 4,
             flops=2 * 64 * 64 * 9 * 56 * 56, bound="mfma", peak=157.3, dtype="f32", tol=1e-5),
     4: Pair(4, "causal softmax 12x[512x512] fp32 || GEMM fp32 [512x768].[768x3072] + tanh-GELU, bfuse",
             "softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072", "bfuse",
-            [("bfuse", ""), ("bfuse", "_c256")],
-            [("softmax_causal_12x512x512_w1", "gemm_gelu_f32_512x768x3072", "bfuse", "_c256"),
-             ("softmax_causal_12x512x512_w1", "gemm_gelu_f32_512x768x3072_t32", "bfuse", "_c256"),
-             ("softmax_causal_12x512x512_b4", "gemm_gelu_f32_512x768x3072", "bfuse", "_c256"),
-             ("softmax_causal_12x512x512_b4", "gemm_gelu_f32_512x768x3072_h", "bfuse", "_c256"),
-             ("softmax_causal_12x512x512_b4", "gemm_gelu_f32_512x768x3072_h", "bfuse", "_c512"),
-             ("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072_h", "bfuse", "_c512"),
-             ("softmax_causal_12x512x512_b4", "gemm_gelu_f32_512x768x3072_h3", "bfuse", "_c512"),
-             ("softmax_causal_12x512x512_r3", "gemm_gelu_f32_512x768x3072_h", "hfuse", ""),
-             ("softmax_causal_12x512x512_r3", "gemm_gelu_f32_512x768x3072_h3", "hfuse", ""),
-             ("softmax_causal_12x512x512_r6", "gemm_gelu_f32_512x768x3072_l", "hfuse", ""),
-             ("softmax_causal_12x512x512_b4", "gemm_gelu_f32_512x768x3072_l", "bfuse", "_c256"),
-             ("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072_l", "bfuse", "_c256"),
-             ("softmax_causal_12x512x512_r6", "gemm_gelu_f32_512x768x3072", "hfuse", ""),
-             ("softmax_causal_12x512x512_r6", "gemm_gelu_f32_512x768x3072_t32", "hfuse", ""),
-             ("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072_d", "bfuse", "_c256"),
-             ("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072_dh", "bfuse", "_c256"),
-             ("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072_dh", "bfuse", "_c512"),
-             ("softmax_causal_12x512x512_b4", "gemm_gelu_f32_512x768x3072_dh", "bfuse", "_c256"),
-             ("softmax_causal_12x512x512_r3", "gemm_gelu_f32_512x768x3072_dh", "hfuse", ""),
-             ("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072_dh2", "bfuse", "_c256"),
-             ("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072_dh2", "bfuse", "_c512")], _pair4_inputs,
+            [("bfuse", "_c256"), ("bfuse", "_c512"), ("bfuse", "")],
+            [("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072_s3", "bfuse", "_c256"),
+             ("softmax_causal_12x512x512_r3", "gemm_gelu_f32_512x768x3072", "hfuse", "")], _pair4_inputs,
             bytes1=2 * 12 * 512 * 512 * 4, bytes2=(512 * 768 + 768 * 3072 + 512 * 3072) * 4,
             flops=2 * 512 * 768 * 3072, bound="mfma", peak=157.3, dtype="f32", tol=1e-5),
     5: Pair(5, "GEMM bf16 [512x4096].[14336x4096]^T (fp32 acc) || RMSNorm+RoPE [512x4096] bf16, bfuse",
             "gemm_bf16_512x4096x14336", "rmsnorm_rope_bf16_512x4096", "bfuse",
-            [("bfuse", ""), ("bfuse", "_c256")],
-            [("gemm_bf16_512x4096x14336", "rmsnorm_rope_bf16_512x4096_w4", "bfuse", "_c256"),
-             ("gemm_bf16_512x4096x14336_v", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
-             ("gemm_bf16_512x4096x14336_w8", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
-             ("gemm_bf16_512x4096x14336_r", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
-             ("gemm_bf16_512x4096x14336_p", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
-             ("gemm_bf16_512x4096x14336_x", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256")], _pair5_inputs,
+            [("bfuse", "_c256")],
+            [("gemm_bf16_512x4096x14336_w8", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
+             ("gemm_bf16_512x4096x14336_w8", "rmsnorm_rope_bf16_512x4096", "bfuse", ""),
+             ("gemm_bf16_512x4096x14336", "rmsnorm_rope_bf16_512x4096_w4", "bfuse", "_c256")], _pair5_inputs,
             bytes1=(512 * 4096 + 4096 * 14336 + 512 * 14336) * 2, bytes2=2 * 512 * 4096 * 2 + 4096 * 2,
             flops=2 * 512 * 4096 * 14336, bound="mfma", peak=2500.0, dtype="bf16", tol=1e-2),
 }
@@ -178,10 +149,19 @@ def fusions(pair: Pair):
 # headline fused variant of each pair: (k1, k2, kind, suffix)
 HEADLINE = {
     1: ("gemm_f32_512x512x512", "bias_relu_1048576", "hfuse", ""),
-    2: ("gemm_f32_512x768x2304_d", "layernorm_512x768_w1", "bfuse", "_r"),
-    3: ("conv3x3_f32_64x56x56_64_l", "maxpool3x3s2_f32_64x112x112", "bfuse", "_c256"),
-    4: ("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072_dh2", "bfuse", "_c256"),
-    5: ("gemm_bf16_512x4096x14336_p", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
+    2: ("gemm_f32_512x768x2304", "layernorm_512x768", "bfuse", "_r"),
+    3: ("conv3x3_f32_64x56x56_64", "maxpool3x3s2_f32_64x112x112", "bfuse", "_c256"),
+    4: ("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072", "bfuse", "_c256"),
+    5: ("gemm_bf16_512x4096x14336", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
+}
+
+# the pair whose block-fused kernel takes its dispatch plan at run time (`..._fused_bfuse_rt`), for the tuner
+RT_SIDES = {
+    1: ("gemm_f32_512x512x512", "bias_relu_1048576"),
+    2: ("gemm_f32_512x768x2304", "layernorm_512x768"),
+    3: ("conv3x3_f32_64x56x56_64", "maxpool3x3s2_f32_64x112x112"),
+    4: ("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072"),
+    5: ("gemm_bf16_512x4096x14336_w8", "rmsnorm_rope_bf16_512x4096"),
 }
 
 
@@ -190,8 +170,8 @@ HEADLINE = {
 # derivation and commands are in the profile summaries shipped with the repository).
 MEASURED_TRAFFIC = {
     "gemm_f32_512x512x512_bias_relu_1048576_fused_hfuse": 23_190_000,
-    "gemm_f32_512x768x2304_d_layernorm_512x768_w1_fused_bfuse_r": 28_530_000,
-    "conv3x3_f32_64x56x56_64_l_maxpool3x3s2_f32_64x112x112_fused_bfuse_c256": 12_320_000,
-    "softmax_causal_12x512x512_gemm_gelu_f32_512x768x3072_dh2_fused_bfuse_c256": 47_740_000,
-    "gemm_bf16_512x4096x14336_p_rmsnorm_rope_bf16_512x4096_fused_bfuse_c256": 174_820_000,
+    "gemm_f32_512x768x2304_layernorm_512x768_fused_bfuse_r": 28_530_000,
+    "conv3x3_f32_64x56x56_64_maxpool3x3s2_f32_64x112x112_fused_bfuse_c256": 12_320_000,
+    "softmax_causal_12x512x512_gemm_gelu_f32_512x768x3072_fused_bfuse_c256": 47_740_000,
+    "gemm_bf16_512x4096x14336_rmsnorm_rope_bf16_512x4096_fused_bfuse_c256": 174_820_000,
 }

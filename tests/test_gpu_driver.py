@@ -18,7 +18,7 @@ def _run(*args):
 def test_driver_modes_validate():
     if not os.path.exists(EXE):
         pytest.fail(f"{EXE} has not been built")
-    k1, k2 = "gemm_f32_512x768x2304", "layernorm_512x768_w1"
+    k1, k2 = "gemm_f32_512x768x2304", "layernorm_512x768"
     for mode, extra in (("0", []), ("1", []), ("2", []), ("5", []), ("4", ["-x", "_r"])):
         r = _run("-v", "-n", "5", *extra, mode, k1, k2)
         assert r.returncode == 0, r.stdout + r.stderr

@@ -14,16 +14,16 @@ import pytest
 import bfuse_project_amd as bf
 from bfuse_project_amd import patterns, tuner
 from bfuse_project_amd._lib import BfuseError
-from bfuse_project_amd.workloads import PAIRS, HEADLINE
+from bfuse_project_amd.workloads import PAIRS, RT_SIDES
 from tests.test_gpu_small import _cases
 
 pytestmark = pytest.mark.gpu
 
 SMALL = [
-    ("gemm_f32_128x160x192_l", "bias_relu_4096"),                 # 8-wave LDS GEMM (barriers) + narrower barrier-free side
+    ("gemm_f32_128x160x192_d", "bias_relu_4096"),                 # split-K GEMM (epilogue barriers) + barrier-free side
     ("conv3x3_f32_32x12x12_32", "gemm_gelu_f32_96x128x192"),      # both sides end in a barrier
     ("layernorm_8x256", "softmax_causal_2x256x256"),
-    ("gemm_bf16_256x320x1792_d", "rmsnorm_rope_bf16_6x1024"),     # fence-free barriers of the direct-to-LDS GEMM
+    ("gemm_bf16_256x320x1792_w8", "rmsnorm_rope_bf16_6x1024"),    # fence-free barriers of the direct-to-LDS GEMM
 ]
 PLANS = [("zigzag", 1, 1), ("zigzag", 2, 3), ("zigzag", 8, 1), ("chunked", 4, 1), ("chunked", 256, 1), ("proportional", 1, 1), ("ranges", 1, 1)]
 
@@ -92,7 +92,7 @@ def test_bad_plans_and_grids_are_refused():
 @pytest.mark.parametrize("number", [2, 4])
 def test_autotune_full_size(number):
     pair = PAIRS[number]
-    k1, k2, _, _ = HEADLINE[number]
+    k1, k2 = RT_SIDES[number]
     I1, F1, I2, F2 = pair.inputs()
     with bf.Operation(k1, k2) as op:
         O1, O2 = op.run_kernel(0, I1, F1), op.run_kernel(1, I2, F2)
