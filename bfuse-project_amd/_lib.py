@@ -52,6 +52,7 @@ class KernelInfoC(C.Structure):
 EXPORTS = [
     "bfuse_last_error", "bfuse_init", "bfuse_shutdown", "bfuse_device_info",
     "bfuse_plan_threads", "bfuse_plan_blocks", "bfuse_map_block", "bfuse_map_thread", "bfuse_map_blocks_device", "bfuse_probe_placement", "bfuse_set_plan",
+    "bfuse_set_sync_spin_limit",
     "bfuse_kernel_count", "bfuse_kernel_at", "bfuse_kernel_find",
     "bfuse_set_elem_bytes", "initialize_kernel1", "initialize_kernel2", "finalize_kernel1", "finalize_kernel2",
     "run_kernel1", "run_kernel2", "run_parallel", "run_fuse",
@@ -91,6 +92,7 @@ def lib():
         l.bfuse_map_thread.argtypes = [C.POINTER(ThreadPlanC), C.c_int, C.c_int, ip]
         l.bfuse_map_blocks_device.argtypes = [C.POINTER(BlockPlanC), C.c_int, C.c_int, vp, vp]
         l.bfuse_set_plan.argtypes = [vp, C.POINTER(BlockPlanC)]
+        l.bfuse_set_sync_spin_limit.argtypes = [vp, C.c_uint]
         l.bfuse_probe_placement.argtypes = [C.c_int, C.c_int, C.c_int, vp, vp, vp, vp, vp]
         l.bfuse_kernel_at.argtypes = [C.c_int, C.POINTER(KernelInfoC)]
         l.bfuse_kernel_find.argtypes = [C.c_char_p, C.POINTER(KernelInfoC)]

@@ -160,7 +160,16 @@ int main(int argc, char** argv)
     while ((c = getopt(argc, argv, "vhn:s:x:")) != -1) {
         switch (c) {
             case 'v': validation = true; break;
-            case 'n': num_iterations = (size_t)atoi(optarg); break;
+            case 'n': {
+                char* end = nullptr;
+                const long n = strtol(optarg, &end, 10);
+                if (!end || *end != '\0' || n < 1 || n > 100000) {
+                    fprintf(stderr, "-n must be a number from 1 to 100000, not '%s'\n", optarg);
+                    return EXIT_FAILURE;
+                }
+                num_iterations = (size_t)n;
+                break;
+            }
             case 's': seed = strtoull(optarg, nullptr, 0); break;
             case 'x': suffix = optarg; break;
             case 'h':
@@ -171,11 +180,13 @@ int main(int argc, char** argv)
         print_help(argv[0]);
         exit(0);
     }
-    const size_t T = (size_t)atoi(argv[optind]);
-    if (T > 5 || num_iterations < 1) {
-        fprintf(stderr, "T must be 0..5 and -n at least 1\n");
+    char* t_end = nullptr;
+    const long t_arg = strtol(argv[optind], &t_end, 10);
+    if (!t_end || *t_end != '\0' || t_arg < 0 || t_arg > 5) {
+        fprintf(stderr, "T must be 0..5, not '%s'\n", argv[optind]);
         return EXIT_FAILURE;
     }
+    const size_t T = (size_t)t_arg;
     CHECK(bfuse_init(0));
     const std::string k1 = resolve(argv[optind + 1], 0), k2 = resolve(argv[optind + 2], 1);
 
@@ -206,8 +217,18 @@ int main(int argc, char** argv)
             CHECK(run_kernel2(b.I.data(), b.F.data(), b.O.data(), b.ki.shape[0], b.ki.shape[1], b.ki.shape[2],
                               (bfuse_kernel3_fn)b.ki.func, b.ki.grid, b.ki.block, 0));
             break;
-        case BFUSE_MODE_PARALLEL:
         case BFUSE_MODE_SERIAL:
+            // kernel 1 then kernel 2 on ONE stream with no host synchronisation in between, over
+            // resident operands (the harness functions have no such call: upload, launch, download)
+            CHECK(bfuse_upload(1, a.I.data(), a.F.data()));
+            CHECK(bfuse_upload(2, b.I.data(), b.F.data()));
+            CHECK(bfuse_zero_output(1));
+            CHECK(bfuse_zero_output(2));
+            CHECK(bfuse_launch(BFUSE_MODE_SERIAL, a.ki.func, a.ki.grid, a.ki.block, b.ki.func, b.ki.grid, b.ki.block));
+            CHECK(bfuse_download(1, a.O.data()));
+            CHECK(bfuse_download(2, b.O.data()));
+            break;
+        case BFUSE_MODE_PARALLEL:
             CHECK(run_parallel(a.I.data(), a.F.data(), a.O.data(), b.I.data(), b.F.data(), b.O.data(), a.ki.shape[0],
                                a.ki.shape[1], a.ki.shape[2], b.ki.shape[0], b.ki.shape[1], b.ki.shape[2],
                                (bfuse_kernel3_fn)a.ki.func, (bfuse_kernel3_fn)b.ki.func, a.ki.grid, a.ki.block,

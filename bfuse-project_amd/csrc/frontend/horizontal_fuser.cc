@@ -515,7 +515,11 @@ string emit_bfuse(const vector<Kernel>& ks, const vector<KernelInfo>& infos, con
 const char* kSideBarrier = R"(// Barrier over the wavefronts of ONE side of a horizontally fused workgroup (gfx950 has no
 // partial-workgroup barrier): lane 0 of every wavefront of the side adds 1 to an LDS counter,
 // then the wavefront polls until the counter reaches waves * epoch.  The poll is bounded so
-// that the grid always drains.
+// that the grid always drains; a wait that gives up is counted in bfuse_sync_timeouts, which the
+// loader reads after the launch (a side that carried on unsynchronised has a wrong output).
+#ifndef BFUSE_SIDE_BARRIER_DEFINED
+#define BFUSE_SIDE_BARRIER_DEFINED
+extern "C" __device__ unsigned int bfuse_sync_timeouts = 0u;
 __device__ __forceinline__ void bfuse_side_barrier(unsigned int* counter, unsigned int waves, unsigned int* epoch)
 {
   *epoch += 1u;
@@ -525,10 +529,14 @@ __device__ __forceinline__ void bfuse_side_barrier(unsigned int* counter, unsign
   unsigned int spins = 0;
   while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < target) {
     __builtin_amdgcn_s_sleep(1);
-    if (++spins == (1u << 22)) break;
+    if (++spins == (1u << 22)) {
+      if ((threadIdx.x & 63) == 0) atomicAdd(&bfuse_sync_timeouts, 1u);
+      break;
+    }
   }
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 }
+#endif
 
 )";
 
@@ -539,10 +547,22 @@ string emit_hfuse(const vector<Kernel>& ks, const vector<KernelInfo>& infos, con
     LaunchDims dims[kMaxKernels];
     for (int i = 0; i < n; ++i) dims[i] = {infos[i].grid, infos[i].block};
     const ThreadPlan plan = plan_threads(n, dims, opt.pad);
+    // With thread ranges that are not whole wavefronts, lane 0 of a side's wavefront can belong to
+    // the other side, and every side barrier would give up.  Such a kernel is still written (its
+    // text and launch shape are what the reference's 32-thread padding produces, for comparison),
+    // but it refuses to compile.
+    bool any_barrier = false;
+    for (int i = 0; i < n; ++i) any_barrier = any_barrier || ks[i].body.find("__syncthreads") != string::npos;
+    const bool unsafe = opt.pad % kWaveSize != 0 && any_barrier;
     if (opt.pad % kWaveSize != 0)
-        cerr << "horizontal-fuser: warning: -w " << opt.pad << " lets one wavefront hold threads of two kernels; the side barrier assumes whole wavefronts\n";
+        cerr << "horizontal-fuser: warning: -w " << opt.pad << " lets one wavefront hold threads of two kernels"
+             << (unsafe ? "; " + fused_name + " synchronises, so its output is marked not to be compiled for gfx950\n" : "\n");
     stringstream o;
-    o << "#include <hip/hip_runtime.h>\n\n" << kSideBarrier;
+    o << "#include <hip/hip_runtime.h>\n\n";
+    if (unsafe)
+        o << "#error \"" << fused_name << ": thread ranges padded to " << opt.pad
+          << " are not whole 64-lane wavefronts; the per-side barrier needs -w 64 (or a multiple)\"\n\n";
+    o << kSideBarrier;
     o << "extern \"C\" __global__ __launch_bounds__(" << plan.fused_block << ") void " << fused_name << "(";
     bool first = true;
     for (int i = 0; i < n; ++i)

@@ -191,8 +191,15 @@ struct KernelEntry {
     TensorDesc io[3];       // single: I, F, O
     std::string side[2];    // fused: names of the two standalone kernels
     int pattern, p0, p1;    // bfuse: dispatch pattern and its parameters
-    unsigned (*read_sync_timeouts)();  // device counter of GroupSync give-ups in this module
+    unsigned (*read_sync_timeouts)();  // device counter of GroupSync give-ups in this module (read and reset)
+    int (*set_spin_limit)(unsigned);   // polls a side barrier of this module makes before it gives up (0 = ok)
     int (*set_plan)(const BlockPlan*); // bfuse_rt: per-kernel hook called when a plan is installed (0 = ok); the plan itself travels as a kernel argument
+};
+
+// per-module (translation unit) access to its own copies of the side-barrier device variables
+struct ModuleHooks {
+    unsigned (*read_sync_timeouts)();
+    int (*set_spin_limit)(unsigned);
 };
 
 std::vector<KernelEntry>& registry();
@@ -203,7 +210,7 @@ struct Registrar {
 
 template <class Op>
 KernelEntry make_single_entry(const char* name, const void* func, TensorDesc i, TensorDesc f, TensorDesc o,
-                              unsigned (*rst)())
+                              const ModuleHooks& hooks)
 {
     KernelEntry e{};
     e.name = name;
@@ -213,13 +220,14 @@ KernelEntry make_single_entry(const char* name, const void* func, TensorDesc i, 
     e.block[0] = Op::THREADS; e.block[1] = 1; e.block[2] = 1;
     e.has_barriers = Op::HAS_BARRIERS;
     e.io[0] = i; e.io[1] = f; e.io[2] = o;
-    e.read_sync_timeouts = rst;
+    e.read_sync_timeouts = hooks.read_sync_timeouts;
+    e.set_spin_limit = hooks.set_spin_limit;
     return e;
 }
 
 template <class Pair>
 KernelEntry make_fused_entry(const char* name, const void* func, int kind, const char* k1, const char* k2,
-                             bool barriers, int pattern, int p0, int p1, unsigned (*rst)())
+                             bool barriers, int pattern, int p0, int p1, const ModuleHooks& hooks)
 {
     KernelEntry e{};
     e.name = name;
@@ -230,7 +238,8 @@ KernelEntry make_fused_entry(const char* name, const void* func, int kind, const
     e.has_barriers = barriers;
     e.side[0] = k1; e.side[1] = k2;
     e.pattern = pattern; e.p0 = p0; e.p1 = p1;
-    e.read_sync_timeouts = rst;
+    e.read_sync_timeouts = hooks.read_sync_timeouts;
+    e.set_spin_limit = hooks.set_spin_limit;
     return e;
 }
 
@@ -244,7 +253,12 @@ KernelEntry make_fused_entry(const char* name, const void* func, int kind, const
         if (hipMemcpyFromSymbol(&v, HIP_SYMBOL(bfuse::g_sync_timeouts), sizeof(v)) != hipSuccess) return ~0u; \
         if (v) (void)hipMemcpyToSymbol(HIP_SYMBOL(bfuse::g_sync_timeouts), &z, sizeof(z));          \
         return v;                                                                                   \
-    }
+    }                                                                                               \
+    static int bfuse_module_set_spin_limit(unsigned polls)                                          \
+    {                                                                                               \
+        return hipMemcpyToSymbol(HIP_SYMBOL(bfuse::g_sync_spin_limit), &polls, sizeof(polls)) == hipSuccess ? 0 : -1; \
+    }                                                                                               \
+    static const bfuse::ModuleHooks bfuse_module_hooks{&bfuse_module_read_sync_timeouts, &bfuse_module_set_spin_limit};
 
 #define BFUSE_KERNEL(NAME, OP, IDESC, FDESC, ODESC)                                                  \
     extern "C" __global__ __launch_bounds__(OP::THREADS, bfuse::kMinWavesPerEu) void NAME(const void* __restrict__ I,       \
@@ -255,7 +269,7 @@ KernelEntry make_fused_entry(const char* name, const void* func, int kind, const
     }                                                                                               \
     static bfuse::Registrar reg_##NAME(bfuse::make_single_entry<OP>(                                \
         #NAME, (const void*)&NAME, bfuse::TensorDesc IDESC, bfuse::TensorDesc FDESC, bfuse::TensorDesc ODESC, \
-        &bfuse_module_read_sync_timeouts));
+        bfuse_module_hooks));
 
 #define BFUSE_BFUSE_KERNEL(K1, OP1, K2, OP2, SUFFIX, PATTERN, P0, P1)                                \
     extern "C" __global__ __launch_bounds__((bfuse::BfusePair<OP1, OP2, PATTERN, P0, P1>::THREADS), bfuse::kMinWavesPerEu)  \
@@ -269,7 +283,7 @@ KernelEntry make_fused_entry(const char* name, const void* func, int kind, const
         bfuse::make_fused_entry<bfuse::BfusePair<OP1, OP2, PATTERN, P0, P1>>(                        \
             #K1 "_" #K2 "_fused_bfuse" #SUFFIX, (const void*)&K1##_##K2##_fused_bfuse##SUFFIX,       \
             bfuse::kBfuse, #K1, #K2, OP1::HAS_BARRIERS || OP2::HAS_BARRIERS, PATTERN, P0, P1,        \
-            &bfuse_module_read_sync_timeouts));
+            bfuse_module_hooks));
 
 #define BFUSE_HFUSE_KERNEL(K1, OP1, K2, OP2)                                                         \
     extern "C" __global__ __launch_bounds__((bfuse::HfusePair<OP1, OP2>::THREADS), bfuse::kMinWavesPerEu)                  \
@@ -282,7 +296,7 @@ KernelEntry make_fused_entry(const char* name, const void* func, int kind, const
     static bfuse::Registrar reg_##K1##_##K2##_hfuse(                                                 \
         bfuse::make_fused_entry<bfuse::HfusePair<OP1, OP2>>(                                         \
             #K1 "_" #K2 "_fused_hfuse", (const void*)&K1##_##K2##_fused_hfuse, bfuse::kHfuse, #K1, #K2, \
-            OP1::HAS_BARRIERS || OP2::HAS_BARRIERS, -1, 0, 0, &bfuse_module_read_sync_timeouts));
+            OP1::HAS_BARRIERS || OP2::HAS_BARRIERS, -1, 0, 0, bfuse_module_hooks));
 
 // The plan is the kernel's seventh argument, passed by value: it arrives with the kernel arguments
 // (scalar loads that hit at once) instead of costing every workgroup a chain of dependent loads
@@ -300,7 +314,7 @@ KernelEntry make_fused_entry(const char* name, const void* func, int kind, const
     static bfuse::Registrar reg_##K1##_##K2##_bfuse_rt([] {                                          \
         bfuse::KernelEntry e = bfuse::make_fused_entry<bfuse::BfuseRtPair<OP1, OP2>>(                \
             #K1 "_" #K2 "_fused_bfuse_rt", (const void*)&K1##_##K2##_fused_bfuse_rt, bfuse::kBfuseRt, #K1, #K2, \
-            true, -1, 0, 0, &bfuse_module_read_sync_timeouts);                                       \
+            true, -1, 0, 0, bfuse_module_hooks);                                       \
         e.set_plan = &set_plan_##K1##_##K2##_rt;                                                     \
         return e;                                                                                   \
     }());

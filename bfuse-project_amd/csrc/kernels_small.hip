@@ -15,6 +15,35 @@ using namespace bfuse;
 
 BFUSE_MODULE_PROLOGUE()
 
+// Test operator for the side barrier's give-up path: the two waves of a workgroup swap their
+// values through LDS across one barrier, y[g] = x[partner of g] + f[g].  Under a side barrier
+// (GroupSync) wave 0 then takes ONE MORE barrier that wave 1 never reaches: the wait is bounded, so
+// it gives up, the kernel ends normally with the right output, and the host must report
+// BFUSE_ERR_SYNC.  Under the hardware barrier (standalone, block fusion) the body is well formed.
+template <int NBLOCKS_, int TAG_>
+struct SyncProbe {
+    static constexpr int THREADS = 128;
+    static constexpr Dims3 GRID{NBLOCKS_, 1, 1};
+    static constexpr Dims3 BLOCK{THREADS, 1, 1};
+    static constexpr bool HAS_BARRIERS = true;
+    struct Smem {
+        float v[THREADS];
+    };
+    template <class Sync>
+    __device__ static __forceinline__ void run(int vblock, int tid, Smem& sm, const void* I, const void* F, void* O, Sync sync)
+    {
+        const int g = vblock * THREADS + tid;
+        sm.v[tid] = static_cast<const float*>(I)[g];
+        sync();
+        static_cast<float*>(O)[g] = sm.v[tid ^ 64] + static_cast<const float*>(F)[g];
+        if constexpr (std::is_same<Sync, GroupSync>::value) {
+            if (tid < 64) sync();   // unmatched on purpose: bounded wait, then the give-up is recorded
+        }
+    }
+};
+using SyncProbeA = SyncProbe<4, 0>;
+using SyncProbeB = SyncProbe<6, 1>;
+
 using GemmS1 = GemmF32<64, 48, 32, 16, 48, 1>;                        // one wave, a 32- and a 16-column group
 using GemmS2 = GemmF32<96, 192, 128, 32, 64, 2, kEpiGeluTanh, 3>;     // 2 waves, GELU, 3 register stages
 using GemmS3 = GemmF32<32, 144, 256, 32, 144, 4>;                     // the 64+64+16 column split, one tile
@@ -81,3 +110,7 @@ BFUSE_HFUSE_KERNEL(conv3x3_f32_32x12x12_32, ConvS2, bias_relu_4096, BiasReluS)
 BFUSE_BFUSE_KERNEL(conv3x3_f32_64x8x16_16, ConvS3, layernorm_8x256, LayerNormS, _c4, bfuse::kChunked, 4, 1)
 // both sides synchronise (each split-K GEMM's reduction barriers): each side gets LDS arrival counters of its own
 BFUSE_HFUSE_KERNEL(gemm_f32_128x160x192_d, GemmS5, gemm_gelu_f32_64x192x288_d, GemmS6)
+// the give-up path of the side barrier, forced from the host with a small spin limit
+BFUSE_KERNEL(sync_probe_a, SyncProbeA, ({{512, 1, 1, 1}, 4}), ({{512, 1, 1, 1}, 4}), ({{512, 1, 1, 1}, 4}))
+BFUSE_KERNEL(sync_probe_b, SyncProbeB, ({{768, 1, 1, 1}, 4}), ({{768, 1, 1, 1}, 4}), ({{768, 1, 1, 1}, 4}))
+BFUSE_HFUSE_KERNEL(sync_probe_a, SyncProbeA, sync_probe_b, SyncProbeB)

@@ -66,7 +66,31 @@ struct State {
     Side side[2];
 } g;
 
-size_t shape_bytes(const int* s, int elem) { return (size_t)s[0] * s[1] * s[2] * s[3] * (size_t)elem; }
+// 0 for a shape with a dimension below 1 (callers refuse empty tensors)
+size_t shape_bytes(const int* s, int elem)
+{
+    for (int d = 0; d < 4; ++d)
+        if (s[d] < 1) return 0;
+    return (size_t)s[0] * s[1] * s[2] * s[3] * (size_t)elem;
+}
+
+// device memory and events that an early return must not leak
+struct DevBuf {
+    void* p = nullptr;
+    ~DevBuf() { if (p) (void)hipFree(p); }
+    template <class T> T* as() const { return static_cast<T*>(p); }
+};
+struct EventList {
+    std::vector<hipEvent_t> v;
+    explicit EventList(size_t n) : v(n, nullptr) {}
+    ~EventList() { for (auto e : v) if (e) (void)hipEventDestroy(e); }
+};
+
+// Fused kernels launched since the last synchronisation whose side barriers can give up, and code
+// objects launched from: their give-up counters are read at the next synchronisation, whichever
+// entry point performs it.
+std::vector<const void*> g_pending_fused;
+std::vector<int> g_pending_modules;
 
 int init_side(int idx, const int* I, const int* F, const int* O)
 {
@@ -75,12 +99,20 @@ int init_side(int idx, const int* I, const int* F, const int* O)
     Side& s = g.side[idx];
     if (s.live) return fail(BFUSE_ERR_STATE, "kernel%d is already initialized", idx + 1);
     const int* shp[3] = {I, F, O};
+    size_t bytes[3];
     for (int i = 0; i < 3; ++i) {
-        s.bytes[i] = shape_bytes(shp[i], s.elem[i]);
-        if (s.bytes[i] == 0) return fail(BFUSE_ERR_ARG, "empty tensor");
-        HIP_TRY(hipMalloc(&s.buf[i], s.bytes[i]));
+        bytes[i] = shape_bytes(shp[i], s.elem[i]);
+        if (bytes[i] == 0) return fail(BFUSE_ERR_ARG, "tensor %d of kernel%d is empty or has a dimension below 1", i, idx + 1);
     }
+    // all or nothing: a failure part-way leaves the side as it was
+    DevBuf tmp[3];
+    for (int i = 0; i < 3; ++i) HIP_TRY(hipMalloc(&tmp[i].p, bytes[i]));
     HIP_TRY(hipStreamCreate(&s.stream));
+    for (int i = 0; i < 3; ++i) {
+        s.buf[i] = tmp[i].p;
+        tmp[i].p = nullptr;
+        s.bytes[i] = bytes[i];
+    }
     s.live = true;
     return BFUSE_OK;
 }
@@ -204,6 +236,9 @@ int launch6(const void* func, const unsigned* grid, const unsigned* block, hipSt
     // a run-time-plan kernel takes its installed plan by value as a seventh argument
     auto it = installed_plans().find(func);
     if (it != installed_plans().end()) args[6] = &it->second;
+    bool known = false;
+    for (const void* f : g_pending_fused) known = known || f == func;
+    if (!known) g_pending_fused.push_back(func);
     if (ev0 || ev1)
         HIP_TRY(hipExtLaunchKernel(func, d3(grid), d3(block), args, 0, stream, ev0, ev1, 0));
     else
@@ -211,18 +246,43 @@ int launch6(const void* func, const unsigned* grid, const unsigned* block, hipSt
     return BFUSE_OK;
 }
 
-int sync_and_check(const void* fused_func)
+// kernels of a loaded code object report give-ups of their side barriers in this device variable
+// (the front end emits it next to every horizontally fused kernel)
+const char* const kModuleSyncCounter = "bfuse_sync_timeouts";
+std::vector<hipModule_t>& modules();
+
+// Device synchronisation, launch errors, and the side barriers' give-up counters of everything
+// launched since the last call: a barrier that gave up let its side run on unsynchronised, so
+// outputs and timings of that launch are not to be trusted.
+int sync_and_check()
 {
     HIP_TRY(hipDeviceSynchronize());
     HIP_TRY(hipGetLastError());
-    if (fused_func) {
-        const KernelEntry* e = entry_of(fused_func);
-        if (e && (e->kind == kHfuse || e->kind == kBfuseRt) && e->read_sync_timeouts) {
-            unsigned n = e->read_sync_timeouts();
-            if (n) return fail(BFUSE_ERR_SYNC, "%s: %u side-barrier waits gave up", e->name.c_str(), n);
+    int rc = BFUSE_OK;
+    for (const void* f : g_pending_fused) {
+        const KernelEntry* e = entry_of(f);
+        if (!e || !(e->kind == kHfuse || e->kind == kBfuseRt) || !e->read_sync_timeouts) continue;
+        const unsigned n = e->read_sync_timeouts();   // reads and resets
+        if (n && rc == BFUSE_OK) rc = fail(BFUSE_ERR_SYNC, "%s: %u side-barrier waits gave up", e->name.c_str(), n);
+    }
+    g_pending_fused.clear();
+    for (int id : g_pending_modules) {
+        if (id < 0 || id >= (int)modules().size() || !modules()[id]) continue;
+        hipDeviceptr_t dp = nullptr;
+        size_t bytes = 0;
+        if (hipModuleGetGlobal(&dp, &bytes, modules()[id], kModuleSyncCounter) != hipSuccess || bytes != sizeof(unsigned)) {
+            (void)hipGetLastError();   // a module without the counter has no side barriers
+            continue;
+        }
+        unsigned n = 0, z = 0;
+        HIP_TRY(hipMemcpy(&n, dp, sizeof(n), hipMemcpyDeviceToHost));
+        if (n) {
+            HIP_TRY(hipMemcpy(dp, &z, sizeof(z), hipMemcpyHostToDevice));
+            if (rc == BFUSE_OK) rc = fail(BFUSE_ERR_SYNC, "code object %d: %u side-barrier waits gave up", id, n);
         }
     }
-    return BFUSE_OK;
+    g_pending_modules.clear();
+    return rc;
 }
 
 int validate_mode(int mode, const void* fa, const unsigned* ga, const unsigned* ba, const void* fb,
@@ -315,6 +375,12 @@ inline double u01(unsigned long long seed, unsigned long long i)  // in (0,1)
     return ((double)(r >> 11) + 0.5) * (1.0 / 9007199254740992.0);
 }
 
+std::vector<hipModule_t>& modules()
+{
+    static std::vector<hipModule_t> m;
+    return m;
+}
+
 }  // namespace
 
 extern "C" {
@@ -405,17 +471,15 @@ int bfuse_map_blocks_device(const bfuse_block_plan* plan, int lo, int hi, int* k
     if (!g.inited) return fail(BFUSE_ERR_STATE, "bfuse_init has not been called");
     if (!plan || !kernel_out || !virt_out || hi <= lo) return fail(BFUSE_ERR_ARG, "bad argument");
     const int n = hi - lo;
-    int *dk = nullptr, *dv = nullptr;
-    HIP_TRY(hipMalloc(&dk, sizeof(int) * (size_t)n));
-    HIP_TRY(hipMalloc(&dv, sizeof(int) * (size_t)n));
+    DevBuf dk, dv;
+    HIP_TRY(hipMalloc(&dk.p, sizeof(int) * (size_t)n));
+    HIP_TRY(hipMalloc(&dv.p, sizeof(int) * (size_t)n));
     BlockPlan p;
     memcpy(&p, plan, sizeof(p));
-    hipLaunchKernelGGL(map_blocks_kernel, dim3((n + 255) / 256), dim3(256), 0, nullptr, p, lo, hi, dk, dv);
+    hipLaunchKernelGGL(map_blocks_kernel, dim3((n + 255) / 256), dim3(256), 0, nullptr, p, lo, hi, dk.as<int>(), dv.as<int>());
     HIP_TRY(hipGetLastError());
-    HIP_TRY(hipMemcpy(kernel_out, dk, sizeof(int) * (size_t)n, hipMemcpyDeviceToHost));
-    HIP_TRY(hipMemcpy(virt_out, dv, sizeof(int) * (size_t)n, hipMemcpyDeviceToHost));
-    HIP_TRY(hipFree(dk));
-    HIP_TRY(hipFree(dv));
+    HIP_TRY(hipMemcpy(kernel_out, dk.p, sizeof(int) * (size_t)n, hipMemcpyDeviceToHost));
+    HIP_TRY(hipMemcpy(virt_out, dv.p, sizeof(int) * (size_t)n, hipMemcpyDeviceToHost));
     return BFUSE_OK;
 }
 
@@ -425,11 +489,12 @@ int bfuse_probe_placement(int workgroups, int threads, int hold, unsigned* xcc, 
     if (!g.inited) return fail(BFUSE_ERR_STATE, "bfuse_init has not been called");
     if (workgroups < 1 || workgroups > (1 << 20) || threads < 64 || threads > 1024 || threads % 64 || hold < 0 || hold > 100000)
         return fail(BFUSE_ERR_ARG, "bad argument");
-    unsigned *d_hw = nullptr, *d_xcc = nullptr;
-    unsigned long long* d_t = nullptr;
-    HIP_TRY(hipMalloc(&d_hw, sizeof(unsigned) * (size_t)workgroups));
-    HIP_TRY(hipMalloc(&d_xcc, sizeof(unsigned) * (size_t)workgroups));
-    HIP_TRY(hipMalloc(&d_t, sizeof(unsigned long long) * (size_t)workgroups));
+    DevBuf b_hw, b_xcc, b_t;
+    HIP_TRY(hipMalloc(&b_hw.p, sizeof(unsigned) * (size_t)workgroups));
+    HIP_TRY(hipMalloc(&b_xcc.p, sizeof(unsigned) * (size_t)workgroups));
+    HIP_TRY(hipMalloc(&b_t.p, sizeof(unsigned long long) * (size_t)workgroups));
+    unsigned *d_hw = b_hw.as<unsigned>(), *d_xcc = b_xcc.as<unsigned>();
+    unsigned long long* d_t = b_t.as<unsigned long long>();
     hipLaunchKernelGGL(placement_kernel, dim3(workgroups), dim3(threads), 0, nullptr, d_hw, d_xcc, d_t, hold);
     HIP_TRY(hipGetLastError());
     std::vector<unsigned> hw((size_t)workgroups), xc((size_t)workgroups);
@@ -437,9 +502,6 @@ int bfuse_probe_placement(int workgroups, int threads, int hold, unsigned* xcc, 
     HIP_TRY(hipMemcpy(hw.data(), d_hw, sizeof(unsigned) * hw.size(), hipMemcpyDeviceToHost));
     HIP_TRY(hipMemcpy(xc.data(), d_xcc, sizeof(unsigned) * xc.size(), hipMemcpyDeviceToHost));
     HIP_TRY(hipMemcpy(ts.data(), d_t, sizeof(unsigned long long) * ts.size(), hipMemcpyDeviceToHost));
-    HIP_TRY(hipFree(d_hw));
-    HIP_TRY(hipFree(d_xcc));
-    HIP_TRY(hipFree(d_t));
     for (int i = 0; i < workgroups; ++i) {
         const unsigned h = hw[(size_t)i];  // gfx9 layout: wave 3:0, simd 5:4, pipe 7:6, cu 11:8, sh 12, se 15:13
         if (xcc) xcc[i] = xc[(size_t)i] & 0xFu;
@@ -489,6 +551,20 @@ int bfuse_set_plan(const void* func, const bfuse_block_plan* plan)
         return fail(BFUSE_ERR_HIP, "could not copy the plan to the device");
     }
     installed_plans()[func] = p;
+    return BFUSE_OK;
+}
+
+int bfuse_set_sync_spin_limit(const void* func, unsigned polls)
+{
+    if (!g.inited) return fail(BFUSE_ERR_STATE, "bfuse_init has not been called");
+    if (!func || polls < 1) return fail(BFUSE_ERR_ARG, "null kernel or a limit below 1");
+    const KernelEntry* e = entry_of(func);
+    if (!e || !e->set_spin_limit) return fail(BFUSE_ERR_ARG, "func is not a kernel of this library");
+    HIP_TRY(hipDeviceSynchronize());   // no launch may be polling with the old limit
+    if (e->set_spin_limit(polls)) {
+        (void)hipGetLastError();
+        return fail(BFUSE_ERR_HIP, "could not set the spin limit of %s's module", e->name.c_str());
+    }
     return BFUSE_OK;
 }
 
@@ -573,7 +649,7 @@ static int run_single(int idx, const void* I, const void* F, void* O, const int*
     HIP_TRY(hipMemcpy(s.buf[0], I, s.bytes[0], hipMemcpyHostToDevice));
     HIP_TRY(hipMemcpy(s.buf[1], F, s.bytes[1], hipMemcpyHostToDevice));
     if ((rc = launch3(func, grid, block, idx, nullptr))) return rc;
-    if ((rc = sync_and_check(nullptr))) return rc;
+    if ((rc = sync_and_check())) return rc;
     HIP_TRY(hipMemcpy(O, s.buf[2], s.bytes[2], hipMemcpyDeviceToHost));
     return BFUSE_OK;
 }
@@ -619,7 +695,7 @@ int run_parallel(const void* I1, const void* F1, void* O1, const void* I2, const
     if ((rc = validate_mode(BFUSE_MODE_PARALLEL, (const void*)func1, g1, b1, (const void*)func2, g2, b2))) return rc;
     if ((rc = upload_both(I1, F1, I2, F2))) return rc;
     if ((rc = enqueue_mode(BFUSE_MODE_PARALLEL, (const void*)func1, g1, b1, (const void*)func2, g2, b2, nullptr))) return rc;
-    if ((rc = sync_and_check(nullptr))) return rc;
+    if ((rc = sync_and_check())) return rc;
     return download_both(O1, O2);
 }
 
@@ -636,7 +712,7 @@ int run_fuse(const void* I1, const void* F1, void* O1, const void* I2, const voi
     if ((rc = validate_mode(mode, (const void*)func, grid, block, nullptr, nullptr, nullptr))) return rc;
     if ((rc = upload_both(I1, F1, I2, F2))) return rc;
     if ((rc = launch6((const void*)func, grid, block, nullptr))) return rc;
-    if ((rc = sync_and_check((const void*)func))) return rc;
+    if ((rc = sync_and_check())) return rc;
     return download_both(O1, O2);
 }
 
@@ -667,15 +743,18 @@ int bfuse_download(int side, void* O)
     Side& s = g.side[side - 1];
     if (!s.live) return fail(BFUSE_ERR_STATE, "kernel%d is not initialized", side);
     if (!O) return fail(BFUSE_ERR_ARG, "null host buffer");
-    HIP_TRY(hipDeviceSynchronize());
+    // the output is copied out even when a side barrier gave up (the caller may want to look at
+    // it), but the call then reports BFUSE_ERR_SYNC
+    const int rc = sync_and_check();
+    if (rc && rc != BFUSE_ERR_SYNC) return rc;
     HIP_TRY(hipMemcpy(O, s.buf[2], s.bytes[2], hipMemcpyDeviceToHost));
-    return BFUSE_OK;
+    return rc;
 }
 
 int bfuse_synchronize(void)
 {
     if (!g.inited) return fail(BFUSE_ERR_STATE, "bfuse_init has not been called");
-    return sync_and_check(nullptr);
+    return sync_and_check();
 }
 
 int bfuse_launch(int mode, const void* fa, const unsigned* ga, const unsigned* ba, const void* fb, const unsigned* gb,
@@ -696,13 +775,14 @@ int bfuse_time(int mode, const void* fa, const unsigned* ga, const unsigned* ba,
     for (int i = 0; i < warmup; ++i)
         if ((rc = enqueue_mode(mode, fa, ga, ba, fb, gb, bb, nullptr))) return rc;
     HIP_TRY(hipDeviceSynchronize());
-    std::vector<hipEvent_t> ev((size_t)reps * 4, nullptr);
+    EventList evl((size_t)reps * 4);
+    std::vector<hipEvent_t>& ev = evl.v;
     const int per = two ? 4 : 2;
     for (int r = 0; r < reps; ++r)
         for (int j = 0; j < per; ++j) HIP_TRY(hipEventCreate(&ev[(size_t)r * 4 + j]));
     for (int r = 0; r < reps; ++r)
         if ((rc = enqueue_mode(mode, fa, ga, ba, fb, gb, bb, &ev[(size_t)r * 4]))) return rc;
-    if ((rc = sync_and_check(mode == BFUSE_MODE_HFUSE ? fa : nullptr))) return rc;
+    if ((rc = sync_and_check())) return rc;
     for (int r = 0; r < reps; ++r) {
         hipEvent_t* e = &ev[(size_t)r * 4];
         float ms_a = 0.f;
@@ -722,8 +802,6 @@ int bfuse_time(int mode, const void* fa, const unsigned* ga, const unsigned* ba,
             us_total[r] = ((end_a > end_b ? end_a : end_b) - first) * 1000.f;
         }
     }
-    for (auto e : ev)
-        if (e) HIP_TRY(hipEventDestroy(e));
     return BFUSE_OK;
 }
 
@@ -737,28 +815,22 @@ int bfuse_time_batched(int mode, const void* fa, const unsigned* ga, const unsig
     for (int i = 0; i < warmup; ++i)
         if ((rc = enqueue_mode(mode, fa, ga, ba, fb, gb, bb, nullptr))) return rc;
     HIP_TRY(hipDeviceSynchronize());
-    hipEvent_t e0, e1;
+    EventList evl(2);
+    hipEvent_t &e0 = evl.v[0], &e1 = evl.v[1];
     HIP_TRY(hipEventCreate(&e0));
     HIP_TRY(hipEventCreate(&e1));
     HIP_TRY(hipEventRecord(e0, nullptr));
     for (int r = 0; r < reps; ++r)
         if ((rc = enqueue_mode(mode, fa, ga, ba, fb, gb, bb, nullptr))) return rc;
     HIP_TRY(hipEventRecord(e1, nullptr));
-    if ((rc = sync_and_check(mode == BFUSE_MODE_HFUSE ? fa : nullptr))) return rc;
+    if ((rc = sync_and_check())) return rc;
     float ms = 0.f;
     HIP_TRY(hipEventElapsedTime(&ms, e0, e1));
     *us_per_launch = ms * 1000.f / (float)reps;
-    HIP_TRY(hipEventDestroy(e0));
-    HIP_TRY(hipEventDestroy(e1));
     return BFUSE_OK;
 }
 
 // ---- kernels from a code object -------------------------------------------------------------
-static std::vector<hipModule_t>& modules()
-{
-    static std::vector<hipModule_t> m;
-    return m;
-}
 
 int bfuse_module_load(const char* path, int* module_id)
 {
@@ -786,9 +858,10 @@ int bfuse_module_unload(int id)
 {
     auto& ms = modules();
     if (id < 0 || id >= (int)ms.size() || !ms[id]) return fail(BFUSE_ERR_ARG, "unknown module %d", id);
+    const int rc = sync_and_check();   // nothing of the module may still run; its counter is read while it exists
     HIP_TRY(hipModuleUnload(ms[id]));
     ms[id] = nullptr;
-    return BFUSE_OK;
+    return rc;
 }
 
 int bfuse_module_launch(int id, const char* name, const unsigned* grid, const unsigned* block, int n_ptrs, int side,
@@ -822,21 +895,23 @@ int bfuse_module_launch(int id, const char* name, const unsigned* grid, const un
     }
     void* args[6];
     for (int i = 0; i < n_ptrs; ++i) args[i] = &ptrs[i];
-    hipEvent_t e0 = nullptr, e1 = nullptr;
+    EventList evl(2);
+    hipEvent_t &e0 = evl.v[0], &e1 = evl.v[1];
     if (us_out) {
         HIP_TRY(hipEventCreate(&e0));
         HIP_TRY(hipEventCreate(&e1));
     }
+    bool known = false;
+    for (int m : g_pending_modules) known = known || m == id;
+    if (!known) g_pending_modules.push_back(id);
     HIP_TRY(hipExtModuleLaunchKernel(fn, grid[0] * block[0], grid[1] * block[1], grid[2] * block[2], block[0], block[1],
                                      block[2], 0, nullptr, args, nullptr, e0, e1, 0));
     if (us_out) {
-        HIP_TRY(hipDeviceSynchronize());
-        HIP_TRY(hipGetLastError());
+        int rc = sync_and_check();
+        if (rc) return rc;
         float ms_ = 0.f;
         HIP_TRY(hipEventElapsedTime(&ms_, e0, e1));
         *us_out = ms_ * 1000.f;
-        HIP_TRY(hipEventDestroy(e0));
-        HIP_TRY(hipEventDestroy(e1));
     }
     return BFUSE_OK;
 }

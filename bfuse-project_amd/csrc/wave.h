@@ -90,34 +90,44 @@ struct BlockSync {
     }
 };
 
+// How many polls a side barrier makes before it gives up.  Device data so that the host can lower
+// it (bfuse_set_sync_spin_limit) -- read only by a wave that already has to wait.
+static __device__ unsigned int g_sync_spin_limit = 1u << 22;
+
 // Barrier over the waves of ONE side of a horizontally fused workgroup.  gfx950 has no
 // partial-workgroup barrier (s_barrier always spans the workgroup), so the side's waves
 // meet on an LDS counter: lane 0 of each wave adds 1, then the wave polls until the counter
 // reaches waves * epoch.  All waves of a workgroup are resident on one CU for the whole
 // kernel, so the wait cannot depend on a wave that has not been scheduled.  The poll is
 // bounded: a side whose waves disagree on the number of barriers gives up after
-// kSpinLimit polls, records it in g_sync_timeouts and carries on, so the grid always drains.
+// g_sync_spin_limit polls, records it in g_sync_timeouts and carries on, so the grid always
+// drains; the host reads the counter at its next synchronisation and reports BFUSE_ERR_SYNC.
 struct GroupSync {
     unsigned int* counter;  // in LDS, zeroed before the sides diverge
     unsigned int waves;
     unsigned int epoch;
-    static constexpr unsigned int kSpinLimit = 1u << 22;
+
+    __device__ __forceinline__ void poll(unsigned int target)
+    {
+        if (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) >= target) return;
+        const unsigned int limit = *(volatile unsigned int*)&g_sync_spin_limit;
+        unsigned int spins = 0;
+        do {
+            __builtin_amdgcn_s_sleep(1);
+            if (++spins >= limit) {
+                if ((threadIdx.x & 63) == 0) atomicAdd(&g_sync_timeouts, 1u);
+                break;
+            }
+        } while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < target);
+    }
 
     __device__ __forceinline__ void operator()()
     {
         ++epoch;
-        const unsigned int target = waves * epoch;
         // order this wave's earlier LDS writes before its arrival
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         if ((threadIdx.x & 63) == 0) atomicAdd(counter, 1u);
-        unsigned int spins = 0;
-        while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < target) {
-            __builtin_amdgcn_s_sleep(1);
-            if (++spins == kSpinLimit) {
-                if ((threadIdx.x & 63) == 0) atomicAdd(&g_sync_timeouts, 1u);
-                break;
-            }
-        }
+        poll(waves * epoch);
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     }
 
@@ -129,17 +139,9 @@ struct GroupSync {
     __device__ __forceinline__ void raw()
     {
         ++epoch;
-        const unsigned int target = waves * epoch;
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         if ((threadIdx.x & 63) == 0) atomicAdd(counter, 1u);
-        unsigned int spins = 0;
-        while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < target) {
-            __builtin_amdgcn_s_sleep(1);
-            if (++spins == kSpinLimit) {
-                if ((threadIdx.x & 63) == 0) atomicAdd(&g_sync_timeouts, 1u);
-                break;
-            }
-        }
+        poll(waves * epoch);
         asm volatile("" ::: "memory");
     }
 };

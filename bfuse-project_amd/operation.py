@@ -179,6 +179,10 @@ class Operation:
             raise ValueError("fused kernel handle required")
         return (fused.func, _u3(fused.grid), _u3(fused.block), None, None, None)
 
+    def set_sync_spin_limit(self, kernel: KernelHandle, polls: int):
+        """Polls a side barrier makes before it gives up, for every kernel of `kernel`'s module."""
+        _lib.check(self.l.bfuse_set_sync_spin_limit(kernel.func, polls))
+
     def launch(self, mode: str, fused: Optional[KernelHandle] = None):
         _lib.check(self.l.bfuse_launch(MODES[mode], *self._mode_args(mode, fused)))
 

@@ -26,7 +26,11 @@ enum {
     BFUSE_ERR_HIP = -2,      /* a HIP runtime call failed; replaces CHECK_CUDA's exit(EXIT_FAILURE),
                                 operation_cu.py:111-121 */
     BFUSE_ERR_STATE = -3,    /* called before bfuse_init / initialize_kernelN */
-    BFUSE_ERR_SYNC = -4      /* a horizontally fused side gave up waiting on its LDS barrier */
+    BFUSE_ERR_SYNC = -4      /* a side of a fused kernel gave up waiting on its LDS barrier: the kernel ran to its
+                                end, but that side carried on unsynchronised, so its output (and any timing of
+                                the launch) is not to be trusted.  Reported by the first call that synchronises
+                                after the launch: run_fuse, bfuse_synchronize, bfuse_download, bfuse_time,
+                                bfuse_time_batched, bfuse_module_launch with us_out, bfuse_module_unload */
 };
 const char* bfuse_last_error(void);
 
@@ -102,6 +106,12 @@ int bfuse_probe_placement(int workgroups, int threads, int hold, unsigned* xcc, 
 int bfuse_set_plan(const void* func, const bfuse_block_plan* plan);
 
 int bfuse_map_blocks_device(const bfuse_block_plan* plan, int lo, int hi, int* kernel_out, int* virt_out);
+
+/* Side barriers of horizontally fused and run-time-plan kernels (the replacement for the
+ * reference's `bar.sync id, n`, horizontal-fuser/src/Matchers.cc:288-320) poll an LDS counter a
+ * bounded number of times, then give up and report BFUSE_ERR_SYNC.  This sets the bound (polls,
+ * default 4194304) for every kernel built into the same module as `func`. */
+int bfuse_set_sync_spin_limit(const void* func, unsigned polls);
 
 /* ------------------------------------------------------------------------------------------
  * Kernel registry -- the role of the reference's generated macro.h tables

@@ -135,6 +135,14 @@ def test_hfuse_ranges(tmp_path):
     assert "warning" in r.stderr
     info = config.load_kernels_yaml(str(out32 / "hfuse_kernels.yaml"))["mm_tiled_ew_max_fused_hfuse"]
     assert info.BlockDim == (416, 1, 1)               # the reference's 32-thread padding: 256 + 160
+    # mm_tiled synchronises: with ranges that are not whole wavefronts its side barrier could never
+    # complete, so the kernel is written (for comparison with the reference) but refuses to compile
+    text32 = (out32 / "mm_tiled_ew_max_hfuse.hip").read_text()
+    assert text32.count("#error") == 1 and "not to be compiled" in r.stderr
+    assert "#error" not in text                       # whole wavefronts: compiles
+    # a give-up of the emitted barrier is counted where the loader can read it
+    assert 'extern "C" __device__ unsigned int bfuse_sync_timeouts' in text
+    assert "atomicAdd(&bfuse_sync_timeouts, 1u)" in text
 
 
 def test_errors(tmp_path):
