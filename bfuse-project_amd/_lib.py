@@ -51,7 +51,7 @@ class KernelInfoC(C.Structure):
 # every symbol include/bfuse_rt.h declares
 EXPORTS = [
     "bfuse_last_error", "bfuse_init", "bfuse_shutdown", "bfuse_device_info",
-    "bfuse_plan_threads", "bfuse_plan_blocks", "bfuse_map_block", "bfuse_map_thread", "bfuse_map_blocks_device", "bfuse_probe_placement", "bfuse_set_plan",
+    "bfuse_plan_threads", "bfuse_plan_blocks", "bfuse_map_block", "bfuse_map_thread", "bfuse_map_blocks_device", "bfuse_map_blocks_device_noalloc", "bfuse_probe_placement", "bfuse_set_plan",
     "bfuse_set_sync_spin_limit",
     "bfuse_kernel_count", "bfuse_kernel_at", "bfuse_kernel_find",
     "bfuse_set_elem_bytes", "initialize_kernel1", "initialize_kernel2", "finalize_kernel1", "finalize_kernel2",
@@ -91,6 +91,7 @@ def lib():
         l.bfuse_map_block.argtypes = [C.POINTER(BlockPlanC), C.c_int, ip]
         l.bfuse_map_thread.argtypes = [C.POINTER(ThreadPlanC), C.c_int, C.c_int, ip]
         l.bfuse_map_blocks_device.argtypes = [C.POINTER(BlockPlanC), C.c_int, C.c_int, vp, vp]
+        l.bfuse_map_blocks_device_noalloc.argtypes = [C.POINTER(BlockPlanC), C.c_int, C.c_int, vp, vp]
         l.bfuse_set_plan.argtypes = [vp, C.POINTER(BlockPlanC)]
         l.bfuse_set_sync_spin_limit.argtypes = [vp, C.c_uint]
         l.bfuse_probe_placement.argtypes = [C.c_int, C.c_int, C.c_int, vp, vp, vp, vp, vp]

@@ -92,6 +92,17 @@ struct EventList {
 std::vector<const void*> g_pending_fused;
 std::vector<int> g_pending_modules;
 
+// ---- staging memory of bfuse_map_blocks_device_noalloc ----------------------------------------
+// A fixed device array (kernel and block index of up to kNoAllocMaxIds fused blocks) that lives as
+// long as the process does.  `scratch` is only the host-side name of the symbol: the address a
+// kernel or a copy can use is looked up once per device (scratch_of) and kept.
+constexpr int kNoAllocMaxIds = BFUSE_NOALLOC_MAX_IDS;
+static __device__ __align__(256) int scratch[2 * kNoAllocMaxIds];
+constexpr int kMaxDevices = 64;
+int* g_scratch_ptr[kMaxDevices] = {};
+
+int scratch_of(int device, int** out);
+
 int init_side(int idx, const int* I, const int* F, const int* O)
 {
     if (!g.inited) return fail(BFUSE_ERR_STATE, "bfuse_init has not been called");
@@ -381,6 +392,22 @@ std::vector<hipModule_t>& modules()
     return m;
 }
 
+// Address of the staging array on `device` (which must be current): looked up on first use,
+// then kept -- every device holds its own copy of the array at its own address.
+int scratch_of(int device, int** out)
+{
+    if (device < 0 || device >= kMaxDevices) return fail(BFUSE_ERR_ARG, "device %d: at most %d devices are supported", device, kMaxDevices);
+    if (!g_scratch_ptr[device]) {
+        int* ptr = nullptr;
+        hipError_t st = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+        if (st != hipSuccess || !ptr)
+            return fail(BFUSE_ERR_HIP, "hipGetSymbolAddress(staging array) on device %d: %s", device, hipGetErrorString(st));
+        g_scratch_ptr[device] = ptr;
+    }
+    *out = g_scratch_ptr[device];
+    return BFUSE_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -396,6 +423,11 @@ int bfuse_init(int device)
                     st == hipSuccess ? "device count is 0" : hipGetErrorString(st));
     if (device < 0 || device >= n) return fail(BFUSE_ERR_ARG, "device %d out of range (0..%d)", device, n - 1);
     HIP_TRY(hipSetDevice(device));
+    // the allocation-free entry point's staging array: its address on this device, looked up now so
+    // that the entry point itself calls nothing that could allocate
+    int* sp = nullptr;
+    int rc = scratch_of(device, &sp);
+    if (rc) return rc;
     g.device = device;
     g.inited = true;
     return BFUSE_OK;
@@ -480,6 +512,32 @@ int bfuse_map_blocks_device(const bfuse_block_plan* plan, int lo, int hi, int* k
     HIP_TRY(hipGetLastError());
     HIP_TRY(hipMemcpy(kernel_out, dk.p, sizeof(int) * (size_t)n, hipMemcpyDeviceToHost));
     HIP_TRY(hipMemcpy(virt_out, dv.p, sizeof(int) * (size_t)n, hipMemcpyDeviceToHost));
+    return BFUSE_OK;
+}
+
+// The same evaluation with no allocation anywhere: the two tables are staged in the library's fixed
+// device array (first half kernel ids, second half virtual block ids) instead of buffers allocated
+// per call.  Every entry of [lo,hi) is written before it is copied out, so nothing has to be
+// cleared between calls; the array keeps the last call's contents, and two calls that overlap on
+// one device would race on it.
+int bfuse_map_blocks_device_noalloc(const bfuse_block_plan* plan, int lo, int hi, int* kernel_out, int* virt_out)
+{
+    if (!g.inited) return fail(BFUSE_ERR_STATE, "bfuse_init has not been called");
+    if (!plan || !kernel_out || !virt_out || hi <= lo) return fail(BFUSE_ERR_ARG, "bad argument");
+    const long long n = (long long)hi - (long long)lo;
+    if (n > kNoAllocMaxIds)
+        return fail(BFUSE_ERR_ARG, "bfuse_map_blocks_device_noalloc: %lld block ids requested, the fixed staging array holds %d; "
+                                   "split the range or use bfuse_map_blocks_device", n, kNoAllocMaxIds);
+    if (g.device < 0 || g.device >= kMaxDevices || !g_scratch_ptr[g.device])
+        return fail(BFUSE_ERR_STATE, "no staging array address for device %d", g.device);
+    int* dk = g_scratch_ptr[g.device];
+    int* dv = dk + kNoAllocMaxIds;
+    BlockPlan p;
+    memcpy(&p, plan, sizeof(p));
+    hipLaunchKernelGGL(map_blocks_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, nullptr, p, lo, hi, dk, dv);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipMemcpy(kernel_out, dk, sizeof(int) * (size_t)n, hipMemcpyDeviceToHost));
+    HIP_TRY(hipMemcpy(virt_out, dv, sizeof(int) * (size_t)n, hipMemcpyDeviceToHost));
     return BFUSE_OK;
 }
 

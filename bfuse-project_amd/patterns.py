@@ -78,6 +78,15 @@ class BlockPlan:
         _lib.check(_lib.lib().bfuse_map_blocks_device(C.byref(self.c), lo, hi, ks.ctypes.data, vs.ctypes.data))
         return ks, vs
 
+    def table_device_noalloc(self, lo=0, hi=None):
+        """table_device through the entry point that allocates nothing (fixed staging array,
+        at most BFUSE_NOALLOC_MAX_IDS = 262144 ids per call)."""
+        hi = self.fused_grid if hi is None else hi
+        ks = np.empty(max(hi - lo, 0), np.int32)
+        vs = np.empty(max(hi - lo, 0), np.int32)
+        _lib.check(_lib.lib().bfuse_map_blocks_device_noalloc(C.byref(self.c), lo, hi, ks.ctypes.data, vs.ctypes.data))
+        return ks, vs
+
     def segments(self) -> List[dict]:
         out = []
         for s in self.c.seg[: self.c.n_seg]:

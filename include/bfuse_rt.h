@@ -107,6 +107,16 @@ int bfuse_set_plan(const void* func, const bfuse_block_plan* plan);
 
 int bfuse_map_blocks_device(const bfuse_block_plan* plan, int lo, int hi, int* kernel_out, int* virt_out);
 
+/* bfuse_map_blocks_device without any allocation.  No counterpart in the reference: it is for
+ * callers that cannot allocate device memory where they call -- code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  Same arguments and results; the two tables are
+ * staged in a fixed device array of the library (2 x BFUSE_NOALLOC_MAX_IDS ints = 2 MiB per GPU,
+ * held until the process ends) whose address is looked up in bfuse_init.  hi - lo above
+ * BFUSE_NOALLOC_MAX_IDS is refused (BFUSE_ERR_ARG).  Calls on one GPU share that array: calls
+ * that overlap on one GPU race. */
+#define BFUSE_NOALLOC_MAX_IDS 262144
+int bfuse_map_blocks_device_noalloc(const bfuse_block_plan* plan, int lo, int hi, int* kernel_out, int* virt_out);
+
 /* Side barriers of horizontally fused and run-time-plan kernels (the replacement for the
  * reference's `bar.sync id, n`, horizontal-fuser/src/Matchers.cc:288-320) poll an LDS counter a
  * bounded number of times, then give up and report BFUSE_ERR_SYNC.  This sets the bound (polls,
