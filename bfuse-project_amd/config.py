@@ -150,8 +150,9 @@ def choose_fusion(a: KernelInfo, b: KernelInfo, lds_a: int, lds_b: int, cus: int
     rounds_a, rounds_b = -(-ga // (cus * na)), -(-gb // (cus * nb))
     return {"hfuse_ok": hfuse_ok, "prefer": "hfuse" if hfuse_ok and ga == gb else "bfuse",
             "wg_per_cu": (na, nb), "rounds": (rounds_a, rounds_b),
-            # one chunk per CU round when a grid covers the chip (measured best on MI355X: the
-            # compute-bound side lands one workgroup per CU and the other side is dealt on top);
-            # below that, a multiple of 8 keeps every side spread over the eight XCDs
-            "chunk": cus if max(ga, gb) >= cus else 8,
+            # one chunk per round over the CUs (measured best on MI355X: the compute-bound side lands
+            # one workgroup per CU and the other side is dealt on top).  A grid below the CU count
+            # is then a single contiguous range, which the hardware itself deals round-robin over
+            # the eight XCDs.
+            "chunk": cus,
             "ratio_M": max(1, max(ga, gb) // max(1, min(ga, gb)))}

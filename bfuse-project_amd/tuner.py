@@ -78,6 +78,61 @@ def autotune(op: Operation, candidates: Optional[Sequence[Candidate]] = None, wa
         h = op.set_plan(rt, plan, c.workgroups)
         t = op.time("bfuse", h, warmup=warmup, reps=reps)[0]
         rows.append({"label": c.label, "pattern": c.pattern, "p0": c.p0, "p1": c.p1, "workgroups": h.grid[0],
-                     "us_mean": float(np.mean(t)), "us_min": float(np.min(t)), "us_std": float(np.std(t))})
+                     "persistent": c.workgroups is not None,
+                     "us_mean": float(np.mean(t)), "us_median": float(np.median(t)), "us_min": float(np.min(t)),
+                     "us_std": float(np.std(t))})
     rows.sort(key=lambda r: r["us_mean"])
     return rows
+
+
+_PATTERN_NAMES = {0: "zigzag", 1: "proportional", 2: "chunked", 3: "ranges"}
+
+
+def _side_dims(k1: KernelHandle, k2: KernelHandle):
+    return [patterns.LaunchDims(tuple(k1.grid), tuple(k1.block)), patterns.LaunchDims(tuple(k2.grid), tuple(k2.block))]
+
+
+def built_variants(k1: str, k2: str) -> List[KernelHandle]:
+    """Every compile-time fused kernel (block or thread fusion) the library holds for the sides (k1, k2)."""
+    from .operation import list_kernels
+    return [k for k in list_kernels() if k.kind in (1, 2) and k.sides == (k1, k2)]
+
+
+def same_dispatch(plan_a, plan_b) -> bool:
+    """Do two block plans send every fused block id to the same (kernel, block)?  Plans built from
+    different patterns can coincide (chunk 256 over grids of at most 256 workgroups is plain ranges)."""
+    if plan_a.fused_grid != plan_b.fused_grid:
+        return False
+    ka, va = plan_a.table()
+    kb, vb = plan_b.table()
+    return bool(np.array_equal(ka, kb) and np.array_equal(va, vb))
+
+
+def static_plan(a: KernelHandle, b: KernelHandle, cus: int = 256, kinds: Sequence[str] = ("hfuse", "bfuse")) -> dict:
+    """The fusion the metadata alone selects, among the allowed kinds: thread-level fusion when the
+    footprints allow it and the grids match, else block fusion in chunks of `chunk` workgroups
+    (one chunk per round over the CUs).  Returns {"kind", "pattern", "p0", "p1", "static"}."""
+    st = static_choice(a, b, cus)
+    if "hfuse" in kinds and (st["prefer"] == "hfuse" or "bfuse" not in kinds):
+        if not st["hfuse_ok"]:
+            raise ValueError(f"{a.name} + {b.name}: thread-level fusion is not possible (barriers on both sides, threads or LDS)")
+        return {"kind": "hfuse", "pattern": None, "p0": 0, "p1": 0, "static": st}
+    return {"kind": "bfuse", "pattern": "chunked", "p0": int(st["chunk"]), "p1": 1, "static": st}
+
+
+def find_variant(k1: KernelHandle, k2: KernelHandle, choice: dict) -> Optional[KernelHandle]:
+    """The built compile-time kernel of (k1, k2) that realises `choice` (static_plan's or a row of
+    autotune): for block fusion, the one whose dispatch table equals the chosen plan's."""
+    built = built_variants(k1.name, k2.name)
+    if choice["kind"] == "hfuse":
+        hs = [k for k in built if k.kind == 2]
+        return hs[0] if hs else None
+    dims = _side_dims(k1, k2)
+    want = patterns.plan_blocks(choice["pattern"], dims, max(choice["p0"], 1), max(choice["p1"], 1))
+    for k in built:
+        if k.kind != 1:
+            continue
+        have = patterns.plan_blocks(_PATTERN_NAMES[k.pattern], dims, max(k.p0, 1), max(k.p1, 1))
+        if same_dispatch(want, have):
+            return k
+    return None

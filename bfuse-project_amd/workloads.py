@@ -155,6 +155,10 @@ HEADLINE = {
     5: ("gemm_bf16_512x4096x14336", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
 }
 
+# fusion kinds the configuration of each pair allows: pair 1 is "horizontally fused", pairs 2-5 are
+# "block-fused"; the chooser picks within them
+CONFIG_KINDS = {1: ("hfuse",), 2: ("bfuse",), 3: ("bfuse",), 4: ("bfuse",), 5: ("bfuse",)}
+
 # the pair whose block-fused kernel takes its dispatch plan at run time (`..._fused_bfuse_rt`), for the tuner
 RT_SIDES = {
     1: ("gemm_f32_512x512x512", "bias_relu_1048576"),
@@ -174,4 +178,13 @@ MEASURED_TRAFFIC = {
     "conv3x3_f32_64x56x56_64_maxpool3x3s2_f32_64x112x112_fused_bfuse_c256": 12_320_000,
     "softmax_causal_12x512x512_gemm_gelu_f32_512x768x3072_fused_bfuse_c256": 47_740_000,
     "gemm_bf16_512x4096x14336_rmsnorm_rope_bf16_512x4096_fused_bfuse_c256": 174_820_000,
+}
+
+# the profile summary each figure above was taken from
+TRAFFIC_SOURCE = {
+    "gemm_f32_512x512x512_bias_relu_1048576_fused_hfuse": "profiles/pair1_gemm_f32_bias_relu_hfuse.md",
+    "gemm_f32_512x768x2304_layernorm_512x768_fused_bfuse_r": "profiles/pair2_gemm_f32_layernorm_bfuse.md",
+    "conv3x3_f32_64x56x56_64_maxpool3x3s2_f32_64x112x112_fused_bfuse_c256": "profiles/pair3_conv3x3_maxpool_bfuse.md",
+    "softmax_causal_12x512x512_gemm_gelu_f32_512x768x3072_fused_bfuse_c256": "profiles/pair4_softmax_gemm_gelu_bfuse.md",
+    "gemm_bf16_512x4096x14336_rmsnorm_rope_bf16_512x4096_fused_bfuse_c256": "profiles/pair5_gemm_bf16_rmsnorm_rope_bfuse.md",
 }

@@ -14,7 +14,7 @@ import pytest
 import bfuse_project_amd as bf
 from bfuse_project_amd import patterns, tuner
 from bfuse_project_amd._lib import BfuseError
-from bfuse_project_amd.workloads import PAIRS, RT_SIDES
+from bfuse_project_amd.workloads import CONFIG_KINDS, HEADLINE, PAIRS, RT_SIDES
 from tests.test_gpu_small import _cases
 
 pytestmark = pytest.mark.gpu
@@ -89,21 +89,39 @@ def test_bad_plans_and_grids_are_refused():
             op.launch("bfuse", replace(h, block=(64, 1, 1)))
 
 
-@pytest.mark.parametrize("number", [2, 4])
-def test_autotune_full_size(number):
+def test_pair1_footprint_selects_thread_level_fusion():
+    """Pair 1's configuration is thread-level fusion; with the real register and LDS figures the
+    footprint rule selects it unprompted (matching grids, one barrier-free side, LDS and threads fit)."""
+    k1, k2 = RT_SIDES[1]
+    with bf.Operation(k1, k2) as op:
+        st = tuner.static_choice(op.k[0], op.k[1])
+        print(f"[tune] pair 1 static: {st}  regs {op.k[0].regs}/{op.k[1].regs} lds {op.k[0].lds_bytes}/{op.k[1].lds_bytes}", flush=True)
+        assert op.k[0].regs > 0 and op.k[0].lds_bytes > 0          # metadata comes from the code object
+        assert st["hfuse_ok"] and st["prefer"] == "hfuse"
+        h = tuner.find_variant(op.k[0], op.k[1], tuner.static_plan(op.k[0], op.k[1], kinds=CONFIG_KINDS[1]))
+        assert h is not None and h.name == op.fused("hfuse").name
+
+
+@pytest.mark.parametrize("number", [2, 3, 4, 5])
+def test_autotune_full_size_agrees_with_the_footprint_rule_and_the_headline(number):
+    """Times the candidate plans on the pair's run-time-plan kernel.  The plan the footprint rule
+    selects (the headline kernel's dispatch) must be within 3 % of the best candidate that has
+    one workgroup per fused block (persistent-workgroup launches exist only on the run-time-plan
+    kernel, so they cannot be the compile-time headline)."""
     pair = PAIRS[number]
     k1, k2 = RT_SIDES[number]
+    hk1, hk2, hkind, hsuffix = HEADLINE[number]
     I1, F1, I2, F2 = pair.inputs()
     with bf.Operation(k1, k2) as op:
         O1, O2 = op.run_kernel(0, I1, F1), op.run_kernel(1, I2, F2)
         op.upload(0, I1, F1)
         op.upload(1, I2, F2)
-        static = tuner.static_choice(op.k[0], op.k[1])
-        rows = tuner.autotune(op, warmup=3, reps=20)
+        choice = tuner.static_plan(op.k[0], op.k[1], kinds=CONFIG_KINDS[number])
+        rows = tuner.autotune(op, warmup=20, reps=100)
         assert rows == sorted(rows, key=lambda r: r["us_mean"]) and rows[0]["us_mean"] > 0
-        print(f"[tune] pair {number} static: {static}")
+        print(f"[tune] pair {number} static: {choice}")
         for r in rows:
-            print(f"[tune] pair {number}: {r['label']:44s} {r['us_mean']:8.2f} us (min {r['us_min']:.2f}) workgroups {r['workgroups']}", flush=True)
+            print(f"[tune] pair {number}: {r['label']:44s} {r['us_mean']:8.2f} us (median {r['us_median']:.2f}, min {r['us_min']:.2f}) workgroups {r['workgroups']}", flush=True)
         # the winner, installed again, still reproduces the unfused kernels
         best = rows[0]
         dims = [patterns.LaunchDims(tuple(k.grid), tuple(k.block)) for k in op.k]
@@ -111,6 +129,19 @@ def test_autotune_full_size(number):
         op.zero_outputs()
         Q1, Q2 = op.run_fuse(h, I1, F1, I2, F2)
         assert np.array_equal(Q1.view(np.uint8), O1.view(np.uint8)) and np.array_equal(Q2.view(np.uint8), O2.view(np.uint8))
+        # the footprint rule's plan among the timed candidates
+        assert choice["kind"] == "bfuse"
+        want = patterns.plan_blocks(choice["pattern"], dims, choice["p0"], choice["p1"])
+        plain = [r for r in rows if not r["persistent"]]
+        mine = [r for r in plain if tuner.same_dispatch(want, patterns.plan_blocks(r["pattern"], dims, r["p0"], r["p1"]))]
+        assert mine, "the footprint rule's plan is not among the candidates"
+        best_plain = min(r["us_median"] for r in plain)
+        print(f"[tune] pair {number}: footprint rule -> {mine[0]['label']} {mine[0]['us_median']:.2f} us, best plain candidate {best_plain:.2f} us", flush=True)
+        assert min(r["us_median"] for r in mine) <= 1.03 * best_plain
         # the 1:1 zig-zag (the reference's live pattern) is not the best placement on this chip
         zz = [r for r in rows if r["label"] == "zigzag 1:1"][0]
         assert rows[0]["us_mean"] <= zz["us_mean"]
+    # and the compile-time kernel with that dispatch is the headline kernel
+    a, b = bf.kernel_info(hk1), bf.kernel_info(hk2)
+    v = tuner.find_variant(a, b, tuner.static_plan(a, b, kinds=CONFIG_KINDS[number]))
+    assert v is not None and v.name == f"{hk1}_{hk2}_fused_{hkind}{hsuffix}"
