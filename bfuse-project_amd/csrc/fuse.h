@@ -135,6 +135,24 @@ struct loop_barriers : std::false_type {};
 template <class Op>
 struct loop_barriers<Op, std::void_t<decltype(Op::LOOP_BARRIERS)>> : std::bool_constant<Op::LOOP_BARRIERS> {};
 
+// how often the operator's body yields when run under JoinSync (0: it has no yield points), and how
+// many workgroup barriers every wave of the operator is certain to execute
+template <class Op, class = void>
+struct yield_count : std::integral_constant<int, 0> {};
+template <class Op>
+struct yield_count<Op, std::void_t<decltype(Op::YIELDS)>> : std::integral_constant<int, Op::YIELDS> {};
+template <class Op, class = void>
+struct min_barriers : std::integral_constant<int, 0> {};
+template <class Op>
+struct min_barriers<Op, std::void_t<decltype(Op::MIN_BARRIERS)>> : std::integral_constant<int, Op::MIN_BARRIERS> {};
+
+// Side X keeps the hardware barrier in its main loop and side Y, which has no barriers, joins the
+// first yield_count<Y> of them (JoinSync): possible when Y has yield points and X synchronises at
+// least that often.
+template <class X, class Y>
+constexpr bool joins_barriers = loop_barriers<X>::value && !Y::HAS_BARRIERS && yield_count<Y>::value > 0 &&
+                                yield_count<Y>::value <= min_barriers<X>::value;
+
 template <class A, class B>
 struct HfusePair {
     static constexpr LaunchDims dims[2] = {{A::GRID, A::BLOCK}, {B::GRID, B::BLOCK}};
@@ -165,11 +183,18 @@ __device__ __forceinline__ void hfuse_body(const void* I1, const void* F1, void*
     // side that synchronises only in its epilogue (the split-K GEMMs, the convolutions) and would
     // serialise the two sides if the barrier sat in the K loop: such a side (LOOP_BARRIERS), and
     // both sides whenever both synchronise, get barriers of their own (the LDS arrival counters).
+    // A side with a barrier in its K loop would pay one LDS-counter barrier per step; if its partner
+    // can yield (see JoinSync) it keeps the hardware barrier and the partner's waves take part in the
+    // first few of them.
     if (kernel_id == 0) {
-        if constexpr (!B::HAS_BARRIERS && !loop_barriers<A>::value) A::run((int)blockIdx.x, local, ss.a, I1, F1, O1, BlockSync{});
+        if constexpr (joins_barriers<A, B>) A::run((int)blockIdx.x, local, ss.a, I1, F1, O1, BlockSync{});
+        else if constexpr (joins_barriers<B, A>) A::run((int)blockIdx.x, local, ss.a, I1, F1, O1, JoinSync{});
+        else if constexpr (!B::HAS_BARRIERS && !loop_barriers<A>::value) A::run((int)blockIdx.x, local, ss.a, I1, F1, O1, BlockSync{});
         else A::run((int)blockIdx.x, local, ss.a, I1, F1, O1, GroupSync{&ss.arrive[0], (unsigned)(round_up(A::THREADS, kWaveSize) / kWaveSize), 0u});
     } else if (kernel_id == 1) {
-        if constexpr (!A::HAS_BARRIERS && !loop_barriers<B>::value) B::run((int)blockIdx.x, local, ss.b, I2, F2, O2, BlockSync{});
+        if constexpr (joins_barriers<B, A>) B::run((int)blockIdx.x, local, ss.b, I2, F2, O2, BlockSync{});
+        else if constexpr (joins_barriers<A, B>) B::run((int)blockIdx.x, local, ss.b, I2, F2, O2, JoinSync{});
+        else if constexpr (!A::HAS_BARRIERS && !loop_barriers<B>::value) B::run((int)blockIdx.x, local, ss.b, I2, F2, O2, BlockSync{});
         else B::run((int)blockIdx.x, local, ss.b, I2, F2, O2, GroupSync{&ss.arrive[1], (unsigned)(round_up(B::THREADS, kWaveSize) / kWaveSize), 0u});
     }
 }

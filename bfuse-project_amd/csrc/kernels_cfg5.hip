@@ -9,9 +9,10 @@ using namespace bfuse;
 
 BFUSE_MODULE_PROLOGUE()
 
-// 128 x 224 tiles: 4 x 64 = 256 workgroups; eight compute waves (4 x 2) of 32 x 112 plus four
-// producer waves that issue the direct-to-LDS loads; ring of three 64-k stages
-using GemmGate = GemmBf16NTDma<512, 14336, 4096, 128, 224, 3, 4, 4, 2, 4>;
+// 128 x 224 tiles: 4 x 64 = 256 workgroups; eight compute waves (4 x 2) of 32 x 112 plus two
+// producer waves that issue the direct-to-LDS loads (two, three and four producers run the same:
+// 47.6-47.8 us); ring of three 64-k stages
+using GemmGate = GemmBf16NTDma<512, 14336, 4096, 128, 224, 3, 4, 4, 2, 2>;
 using NormRope1 = RmsNormRope<512, 32, 128, 1>;             // 512 one-wave workgroups
 
 BFUSE_KERNEL(gemm_bf16_512x4096x14336, GemmGate, ({{512, 4096, 1, 1}, 2}), ({{14336, 4096, 1, 1}, 2}), ({{512, 14336, 1, 1}, 2}))
@@ -19,12 +20,19 @@ BFUSE_KERNEL(rmsnorm_rope_bf16_512x4096, NormRope1, ({{512, 4096, 1, 1}, 2}), ({
 
 BFUSE_BFUSE_KERNEL(gemm_bf16_512x4096x14336, GemmGate, rmsnorm_rope_bf16_512x4096, NormRope1, _c256, bfuse::kChunked, 256, 1)
 
+// Thread-level fusion: two RMSNorm+RoPE waves inside every GEMM workgroup (256 workgroups, one per
+// CU, twelve waves).  The GEMM keeps the hardware barrier of its K loop; the norm waves take part
+// in the first seven of them, one per section of their row (JoinSync), and leave.
+using NormRope2 = RmsNormRope<512, 32, 128, 2>;             // 256 two-wave workgroups
+BFUSE_KERNEL(rmsnorm_rope_bf16_512x4096_w2, NormRope2, ({{512, 4096, 1, 1}, 2}), ({{(int)NormRope2::F_BYTES, 1, 1, 1}, 1}), ({{512, 4096, 1, 1}, 2}))
+BFUSE_HFUSE_KERNEL(gemm_bf16_512x4096x14336, GemmGate, rmsnorm_rope_bf16_512x4096_w2, NormRope2)
+
 // alternative GEMM side: the same eight compute waves issue their own loads (no producer waves)
 using GemmGate8 = GemmBf16NTDma<512, 14336, 4096, 128, 224, 3, 4, 4, 2>;
 BFUSE_KERNEL(gemm_bf16_512x4096x14336_w8, GemmGate8, ({{512, 4096, 1, 1}, 2}), ({{14336, 4096, 1, 1}, 2}), ({{512, 14336, 1, 1}, 2}))
 BFUSE_BFUSE_KERNEL(gemm_bf16_512x4096x14336_w8, GemmGate8, rmsnorm_rope_bf16_512x4096, NormRope1, _c256, bfuse::kChunked, 256, 1)
 // the reference's live pattern (1:1 zig-zag), for the record, and the run-time-plan kernel (dispatch
-// plan as data, persistent workgroups).  Both on the eight-wave GEMM: with twelve waves the kernel is
+// plan as data, persistent workgroups).  Both on the eight-wave GEMM: with ten waves the kernel is
 // capped at 168 VGPRs and these two forms do not fit without spilling
 BFUSE_BFUSE_KERNEL(gemm_bf16_512x4096x14336_w8, GemmGate8, rmsnorm_rope_bf16_512x4096, NormRope1, , bfuse::kZigzag, 1, 1)
 BFUSE_BFUSE_RT_KERNEL(gemm_bf16_512x4096x14336_w8, GemmGate8, rmsnorm_rope_bf16_512x4096, NormRope1)

@@ -61,6 +61,7 @@ using GemmB2 = GemmBf16NTDma<128, 1792, 192, 128, 224, 2>;            // two sta
 using GemmB3 = GemmBf16NTDma<256, 1792, 320, 128, 224, 3>;            // two M-tiles, ring of three, five K-steps
 using GemmB5 = GemmBf16NTDma<256, 1792, 320, 128, 224, 3, 4, 4, 2>;   // the same with eight waves (uneven load groups per wave)
 using GemmB8 = GemmBf16NTDma<256, 1792, 384, 128, 224, 3, 4, 4, 2, 4>;   // eight compute + four producer waves
+using GemmB9 = GemmBf16NTDma<256, 1792, 448, 128, 224, 3, 4, 4, 2, 2>;   // eight compute + two producer waves, seven K-steps
 using NormRopeS = RmsNormRope<6, 8, 128, 2>;
 
 BFUSE_KERNEL(gemm_f32_64x32x48, GemmS1, ({{64, 32, 1, 1}, 4}), ({{32, 48, 1, 1}, 4}), ({{64, 48, 1, 1}, 4}))
@@ -80,6 +81,7 @@ BFUSE_KERNEL(gemm_bf16_128x192x1792, GemmB2, ({{128, 192, 1, 1}, 2}), ({{1792, 1
 BFUSE_KERNEL(gemm_bf16_256x320x1792, GemmB3, ({{256, 320, 1, 1}, 2}), ({{1792, 320, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
 BFUSE_KERNEL(gemm_bf16_256x320x1792_w8, GemmB5, ({{256, 320, 1, 1}, 2}), ({{1792, 320, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
 BFUSE_KERNEL(gemm_bf16_256x384x1792_p, GemmB8, ({{256, 384, 1, 1}, 2}), ({{1792, 384, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
+BFUSE_KERNEL(gemm_bf16_256x448x1792_p2, GemmB9, ({{256, 448, 1, 1}, 2}), ({{1792, 448, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
 BFUSE_KERNEL(rmsnorm_rope_bf16_6x1024, NormRopeS, ({{6, 1024, 1, 1}, 2}), ({{(int)NormRopeS::F_BYTES, 1, 1, 1}, 1}), ({{6, 1024, 1, 1}, 2}))
 
 // calibration kernel for the memory counters: 64 MiB read, 64 MiB written
@@ -97,8 +99,13 @@ BFUSE_BFUSE_KERNEL(conv3x3_f32_32x12x12_32, ConvS2, gemm_gelu_f32_96x128x192, Ge
 BFUSE_BFUSE_KERNEL(layernorm_8x256, LayerNormS, softmax_causal_2x256x256, SoftmaxS, , bfuse::kZigzag, 1, 1)
 BFUSE_BFUSE_KERNEL(gemm_bf16_256x320x1792, GemmB3, rmsnorm_rope_bf16_6x1024, NormRopeS, _c8, bfuse::kChunked, 8, 1)
 BFUSE_HFUSE_KERNEL(maxpool3x3s2_f32_4x16x16, PoolS, layernorm_8x256, LayerNormS)
-// a side with a barrier in its K loop under horizontal fusion: its fence-free barriers become the LDS-counter one
-BFUSE_HFUSE_KERNEL(gemm_bf16_256x320x1792_w8, GemmB5, rmsnorm_rope_bf16_6x1024, NormRopeS)
+// a side with a barrier in its K loop under horizontal fusion, both sides synchronising: its fence-free
+// barriers become the LDS-counter one
+BFUSE_HFUSE_KERNEL(gemm_bf16_256x320x1792_w8, GemmB5, gemm_f32_128x160x192_d, GemmS5)
+// the same GEMM with producer waves keeps the hardware barrier in its K loop and the norm waves join
+// its first four barriers (16 GEMM tiles, 3 norm workgroups: most workgroups have no norm waves at all)
+BFUSE_HFUSE_KERNEL(gemm_bf16_256x384x1792_p, GemmB8, rmsnorm_rope_bf16_6x1024, NormRopeS)
+BFUSE_HFUSE_KERNEL(gemm_bf16_256x448x1792_p2, GemmB9, rmsnorm_rope_bf16_6x1024, NormRopeS)
 // run-time plans / persistent workgroups: equal and unequal workgroup widths, barrier-bearing sides
 BFUSE_BFUSE_RT_KERNEL(conv3x3_f32_32x12x12_32, ConvS2, gemm_gelu_f32_96x128x192, GemmS2)
 BFUSE_BFUSE_RT_KERNEL(layernorm_8x256, LayerNormS, softmax_causal_2x256x256, SoftmaxS)

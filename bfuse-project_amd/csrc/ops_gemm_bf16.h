@@ -83,6 +83,7 @@ struct GemmBf16NTDma {
     static constexpr Dims3 BLOCK{THREADS, 1, 1};
     static constexpr bool HAS_BARRIERS = true;
     static constexpr bool LOOP_BARRIERS = true;   // one workgroup barrier per K-stage, not only in the epilogue
+    static constexpr int MIN_BARRIERS = K_ / 64 + 2;   // what every wave executes: one per K-step, two in the epilogue
     static constexpr int EPI_BYTES = BM * CPITCH * 2;
     struct Smem {
         __attribute__((aligned(1024))) unsigned char t[((NSTG * STAGE_BYTES > EPI_BYTES) ? NSTG * STAGE_BYTES : EPI_BYTES)];

@@ -229,7 +229,13 @@ struct RmsNormRope {
     static constexpr bool HAS_BARRIERS = false;
     static constexpr int OCT = HALF / 8;                 // octets per half head
     static constexpr int SLOTS = HEADS * OCT / 64;       // (head, octet) slots per lane
+    // Sections of the body when it runs under JoinSync (its partner's loop barriers), a yield after
+    // each but the last: every load the row needs is requested | WAIT_STEPS - 1 empty sections that
+    // let the partner's steps pass while the data arrives | the reduction | one slot each.
+    static constexpr int WAIT_STEPS = 3;
+    static constexpr int YIELDS = WAIT_STEPS + SLOTS;
     static_assert(S % WAVES == 0 && HALF % 8 == 0 && (HEADS * OCT) % 64 == 0, "whole slots per lane");
+    static_assert(64 % OCT == 0, "a lane's octet offset does not depend on the slot");
     static constexpr size_t COS_OFFSET = (size_t)D * 2;                 // bytes into F
     static constexpr size_t SIN_OFFSET = COS_OFFSET + (size_t)S * HD * 4;
     static constexpr size_t F_BYTES = SIN_OFFSET + (size_t)S * HD * 4;
@@ -246,13 +252,34 @@ struct RmsNormRope {
         u += 0x7fffu + ((u >> 16) & 1u);
         return (unsigned short)(u >> 16);
     }
+    // The arithmetic of one element pair (j, j + HALF) -- the one place it is written, whichever way
+    // the inputs arrived:  t = w (x r);  out_lo = t_lo cos_lo - t_hi sin_lo;  out_hi = t_hi cos_hi + t_lo sin_hi
+    __device__ static __forceinline__ void rotate_pair(float w_lo, float w_hi, float x_lo, float x_hi, float r, float c_lo, float s_lo,
+                                                       float c_hi, float s_hi, unsigned short& o_lo, unsigned short& o_hi)
+    {
+        const float tl = w_lo * (x_lo * r), th = w_hi * (x_hi * r);
+        o_lo = to_bf16(tl * c_lo + (-th) * s_lo);
+        o_hi = to_bf16(th * c_hi + tl * s_hi);
+    }
+    __device__ static __forceinline__ int slot_base(int slot) { return (slot / OCT) * HD + (slot % OCT) * 8; }
+    __device__ static __forceinline__ void load_octets(u16x8& lo, u16x8& hi, int slot, const unsigned short* __restrict__ p)
+    {
+        lo = *reinterpret_cast<const u16x8*>(p + slot_base(slot));
+        hi = *reinterpret_cast<const u16x8*>(p + slot_base(slot) + HALF);
+    }
 
     template <class Sync>
     __device__ static __forceinline__ void run(int vblock, int tid, Smem&, const void* I, const void* F,
-                                               void* O, Sync)
+                                               void* O, Sync sync)
     {
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;   // wave-uniform: addresses built on it stay in scalar registers
         const int pos = vblock * WAVES + wave;
+        if constexpr (Sync::kYields) {
+            // sections must stay sections: memory operations may not cross the yields
+            I = opaque_pointer(I);
+            F = opaque_pointer(F);
+            O = opaque_pointer(O);
+        }
         const unsigned short* __restrict__ x = static_cast<const unsigned short*>(I) + (size_t)pos * D;
         const unsigned short* __restrict__ w = static_cast<const unsigned short*>(F);
         const float* __restrict__ cosv = reinterpret_cast<const float*>(static_cast<const char*>(F) + COS_OFFSET) + (size_t)pos * HD;
@@ -263,12 +290,32 @@ struct RmsNormRope {
         // where it is used: half the registers of an fp32 copy
         u16x8 xl[SLOTS], xh[SLOTS];
         float ss = 0.f;
+        // held operands of the sectioned form: weights of every slot and the cos / sin values of the
+        // lane's octet, which are the same for every slot
+        u16x8 wlo[SLOTS], whi[SLOTS];
+        f32x4 cl[2], ch[2], sl[2], sh[2];
+        if constexpr (Sync::kYields) {
+            // Nothing the row needs depends on the reduction, so everything is requested first and is
+            // on its way while the partner's steps pass: a section that had to wait for memory would
+            // hold up the partner's barrier for as long.
+            const int j = (lane % OCT) * 8;
+#pragma unroll
+            for (int s = 0; s < SLOTS; ++s) load_octets(xl[s], xh[s], s * 64 + lane, x);
+#pragma unroll
+            for (int s = 0; s < SLOTS; ++s) load_octets(wlo[s], whi[s], s * 64 + lane, w);
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                cl[q] = *reinterpret_cast<const f32x4*>(cosv + j + 4 * q);
+                ch[q] = *reinterpret_cast<const f32x4*>(cosv + j + HALF + 4 * q);
+                sl[q] = *reinterpret_cast<const f32x4*>(sinv + j + 4 * q);
+                sh[q] = *reinterpret_cast<const f32x4*>(sinv + j + HALF + 4 * q);
+            }
+#pragma unroll
+            for (int i = 0; i < WAIT_STEPS; ++i) sync.yield();   // the loads stay in flight across them
+        }
 #pragma unroll
         for (int s = 0; s < SLOTS; ++s) {
-            const int slot = s * 64 + lane;
-            const int base = (slot / OCT) * HD + (slot % OCT) * 8;
-            xl[s] = *reinterpret_cast<const u16x8*>(x + base);
-            xh[s] = *reinterpret_cast<const u16x8*>(x + base + HALF);
+            if constexpr (!Sync::kYields) load_octets(xl[s], xh[s], s * 64 + lane, x);
             float lo[8], hi[8];
             unpack(xl[s], lo);
             unpack(xh[s], hi);
@@ -276,9 +323,37 @@ struct RmsNormRope {
             for (int e = 0; e < 8; ++e) ss += lo[e] * lo[e] + hi[e] * hi[e];
         }
         const float r = 1.0f / sqrtf(wave_sum(ss) / (float)D + 1e-5f);
+
+        if constexpr (Sync::kYields) {
 #pragma unroll
-        for (int s = 0; s < SLOTS; ++s) {
-            {
+            for (int s = 0; s < SLOTS; ++s) {
+                float rs = r;
+                sync.yield(rs);   // short sections: the partner waits at its barrier while one runs
+                // the row's octets are widened again here rather than kept widened since the reduction
+                opaque_value(xl[s]);
+                opaque_value(xh[s]);
+                const int slot = s * 64 + lane;
+                float wl[8], wh[8], lo[8], hi[8];
+                unpack(wlo[s], wl);
+                unpack(whi[s], wh);
+                unpack(xl[s], lo);
+                unpack(xh[s], hi);
+                u16x8 ol, oh;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    unsigned short a, b;
+                    rotate_pair(wl[e], wh[e], lo[e], hi[e], rs, cl[e / 4][e % 4], sl[e / 4][e % 4], ch[e / 4][e % 4], sh[e / 4][e % 4], a, b);
+                    ol[e] = a;
+                    oh[e] = b;
+                }
+                *reinterpret_cast<u16x8*>(y + slot_base(slot)) = ol;
+                *reinterpret_cast<u16x8*>(y + slot_base(slot) + HALF) = oh;
+            }
+        } else {
+            // on its own the body leaves the order of the operand loads to the compiler (it requests
+            // all of them before the reduction)
+#pragma unroll
+            for (int s = 0; s < SLOTS; ++s) {
                 const int slot = s * 64 + lane;
                 const int j = (slot % OCT) * 8;
                 const int base = (slot / OCT) * HD + j;
@@ -290,9 +365,10 @@ struct RmsNormRope {
                 u16x8 ol, oh;
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
-                    const float tl = wl[e] * (lo[e] * r), th = wh[e] * (hi[e] * r);
-                    ol[e] = to_bf16(tl * cosv[j + e] + (-th) * sinv[j + e]);
-                    oh[e] = to_bf16(th * cosv[j + HALF + e] + tl * sinv[j + HALF + e]);
+                    unsigned short a, b;
+                    rotate_pair(wl[e], wh[e], lo[e], hi[e], r, cosv[j + e], sinv[j + e], cosv[j + HALF + e], sinv[j + HALF + e], a, b);
+                    ol[e] = a;
+                    oh[e] = b;
                 }
                 *reinterpret_cast<u16x8*>(y + base) = ol;
                 *reinterpret_cast<u16x8*>(y + base + HALF) = oh;

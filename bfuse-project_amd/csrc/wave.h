@@ -69,6 +69,9 @@ static __device__ unsigned int g_sync_timeouts;
 // one operator; waves outside the operator's thread range have already exited, and the
 // hardware barrier only counts waves that are still alive).
 struct BlockSync {
+    static constexpr bool kYields = false;
+    __device__ __forceinline__ void yield() const {}   // see JoinSync
+    __device__ __forceinline__ void yield(float&) const {}
     __device__ __forceinline__ void operator()() const { __syncthreads(); }
     // Barrier WITHOUT a memory fence: only this wave's LDS accesses are drained.  For
     // pipelines that keep global->LDS loads in flight across the barrier and account for
@@ -103,6 +106,9 @@ static __device__ unsigned int g_sync_spin_limit = 1u << 22;
 // g_sync_spin_limit polls, records it in g_sync_timeouts and carries on, so the grid always
 // drains; the host reads the counter at its next synchronisation and reports BFUSE_ERR_SYNC.
 struct GroupSync {
+    static constexpr bool kYields = false;
+    __device__ __forceinline__ void yield() const {}   // see JoinSync
+    __device__ __forceinline__ void yield(float&) const {}
     unsigned int* counter;  // in LDS, zeroed before the sides diverge
     unsigned int waves;
     unsigned int epoch;
@@ -145,5 +151,67 @@ struct GroupSync {
         asm volatile("" ::: "memory");
     }
 };
+
+// Policy of a barrier-FREE side whose partner in a horizontally fused workgroup keeps the hardware
+// barrier inside its main loop.  s_barrier counts every live wave of the workgroup, so the partner's
+// first barrier would wait until this side's waves have exited -- the two sides would run one after
+// the other.  Instead this side takes part: its body is cut into sections at yield() calls, each
+// yield() is one s_barrier, matched with the partner's 1st, 2nd, ... loop barrier.  While this side
+// is alive the partner advances one loop step per section; after its last section it exits and the
+// hardware stops counting its waves.  A body may yield at most as often as every wave of the partner
+// is certain to synchronise (Op::YIELDS <= Partner::MIN_BARRIERS, checked at compile time), and it
+// keeps its loads in flight across the yield: it issues them before and waits for them after, so a
+// section costs the partner's step nothing but the arrival.
+// The compiler-level fences keep memory operations and the schedule on their side of the barrier.
+struct JoinSync {
+    static constexpr bool kYields = true;
+    __device__ __forceinline__ void yield() const
+    {
+        float none = 0.f;
+        yield(none);
+    }
+    // `carried` comes out as a value the compiler knows nothing about (unchanged).  The barrier is
+    // written as asm with `carried` as its operand so that it sits in the data flow: what `carried`
+    // was computed from is finished before the barrier, and arithmetic that uses it afterwards
+    // cannot be moved to before it.  (The memory clobber orders memory operations only, and only
+    // through pointers the compiler cannot trace -- see opaque_pointer; pure arithmetic it would
+    // otherwise compute early and keep in registers across the sections before.)
+    __device__ __forceinline__ void yield(float& carried) const
+    {
+        __builtin_amdgcn_sched_barrier(0);
+#if defined(__HIP_DEVICE_COMPILE__)
+        asm volatile("s_barrier" : "+v"(carried) : : "memory");
+#endif
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    // a side run under this policy has no barriers of its own (HAS_BARRIERS = false)
+    __device__ __forceinline__ void operator()() const {}
+};
+
+// The value, unchanged, as one the compiler knows nothing about: what was derived from it before
+// (say its widened copy) is not kept for later uses, it is derived again.
+template <class V>
+__device__ __forceinline__ void opaque_value(V& v)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("" : "+v"(v));
+#endif
+}
+
+// A kernel-argument pointer (wave-uniform, `__restrict__`) as the compiler sees an unknown pointer
+// into device memory.  The memory clobbers in JoinSync::yield() order nothing against memory that
+// is only reachable through a noalias argument (an asm without pointer operands cannot touch it, so
+// loads and stores through it may cross); a body that must keep its sections apart takes its
+// pointers through here.
+template <class T>
+__device__ __forceinline__ T* opaque_pointer(T* p)
+{
+    unsigned long long bits = (unsigned long long)p;
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("" : "+s"(bits));
+#endif
+    // an integer turned into a pointer to global memory: accesses stay global_load / global_store
+    return (T*)(__attribute__((address_space(1))) T*)bits;
+}
 
 }  // namespace bfuse

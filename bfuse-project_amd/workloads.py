@@ -126,10 +126,11 @@ PAIRS: Dict[int, Pair] = {
              ("softmax_causal_12x512x512_r3", "gemm_gelu_f32_512x768x3072", "hfuse", "")], _pair4_inputs,
             bytes1=2 * 12 * 512 * 512 * 4, bytes2=(512 * 768 + 768 * 3072 + 512 * 3072) * 4,
             flops=2 * 512 * 768 * 3072, bound="mfma", peak=157.3, dtype="f32", tol=1e-5),
-    5: Pair(5, "GEMM bf16 [512x4096].[14336x4096]^T (fp32 acc) || RMSNorm+RoPE [512x4096] bf16, bfuse",
-            "gemm_bf16_512x4096x14336", "rmsnorm_rope_bf16_512x4096", "bfuse",
-            [("bfuse", "_c256")],
-            [("gemm_bf16_512x4096x14336_w8", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
+    5: Pair(5, "GEMM bf16 [512x4096].[14336x4096]^T (fp32 acc) || RMSNorm+RoPE [512x4096] bf16, norm waves inside the GEMM workgroups",
+            "gemm_bf16_512x4096x14336", "rmsnorm_rope_bf16_512x4096_w2", "hfuse",
+            [("hfuse", "")],
+            [("gemm_bf16_512x4096x14336", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
+             ("gemm_bf16_512x4096x14336_w8", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
              ("gemm_bf16_512x4096x14336_w8", "rmsnorm_rope_bf16_512x4096", "bfuse", ""),
              ("gemm_bf16_512x4096x14336", "rmsnorm_rope_bf16_512x4096_w4", "bfuse", "_c256")], _pair5_inputs,
             bytes1=(512 * 4096 + 4096 * 14336 + 512 * 14336) * 2, bytes2=2 * 512 * 4096 * 2 + 4096 * 2,
@@ -152,12 +153,21 @@ HEADLINE = {
     2: ("gemm_f32_512x768x2304", "layernorm_512x768", "bfuse", "_r"),
     3: ("conv3x3_f32_64x56x56_64", "maxpool3x3s2_f32_64x112x112", "bfuse", "_c256"),
     4: ("softmax_causal_12x512x512", "gemm_gelu_f32_512x768x3072", "bfuse", "_c256"),
-    5: ("gemm_bf16_512x4096x14336", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256"),
+    5: ("gemm_bf16_512x4096x14336", "rmsnorm_rope_bf16_512x4096_w2", "hfuse", ""),
 }
 
-# fusion kinds the configuration of each pair allows: pair 1 is "horizontally fused", pairs 2-5 are
-# "block-fused"; the chooser picks within them
-CONFIG_KINDS = {1: ("hfuse",), 2: ("bfuse",), 3: ("bfuse",), 4: ("bfuse",), 5: ("bfuse",)}
+# fused forms that the configurations name but that are not the fastest on this chip, timed beside the
+# headline kernel: (label, k1, k2, kind, suffix)
+BESIDE = {
+    3: [("zigzag_1to1", "conv3x3_f32_64x56x56_64", "maxpool3x3s2_f32_64x112x112", "bfuse", "")],
+    5: [("block_fused_chunk256", "gemm_bf16_512x4096x14336", "rmsnorm_rope_bf16_512x4096", "bfuse", "_c256")],
+}
+
+# fusion kinds the chooser picks from for each pair.  The configurations call pair 1 "horizontally
+# fused" and pairs 2-5 "block-fused"; pair 5 is opened to both because block fusion cannot pay there
+# (every workgroup of a block-fused kernel is charged the GEMM's 135 KB of LDS, so no norm workgroup
+# ever shares a CU with a GEMM workgroup), and the block-fused kernel is timed beside it.
+CONFIG_KINDS = {1: ("hfuse",), 2: ("bfuse",), 3: ("bfuse",), 4: ("bfuse",), 5: ("hfuse", "bfuse")}
 
 # the pair whose block-fused kernel takes its dispatch plan at run time (`..._fused_bfuse_rt`), for the tuner
 RT_SIDES = {
@@ -178,6 +188,7 @@ MEASURED_TRAFFIC = {
     "conv3x3_f32_64x56x56_64_maxpool3x3s2_f32_64x112x112_fused_bfuse_c256": 12_320_000,
     "softmax_causal_12x512x512_gemm_gelu_f32_512x768x3072_fused_bfuse_c256": 47_740_000,
     "gemm_bf16_512x4096x14336_rmsnorm_rope_bf16_512x4096_fused_bfuse_c256": 174_820_000,
+    "gemm_bf16_512x4096x14336_rmsnorm_rope_bf16_512x4096_w2_fused_hfuse": None,
 }
 
 # the profile summary each figure above was taken from

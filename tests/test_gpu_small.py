@@ -67,6 +67,8 @@ def _cases():
                                       lambda I, F: orf.gemm_bf16(I.reshape(256, 320), F.reshape(1792, 320), b_is_nk=True), 1e-2, True),
         "gemm_bf16_256x384x1792_p": (lambda s: (f32_to_bf16(fill_normal(s, 256 * 384, 0, 1)), f32_to_bf16(fill_normal(s + 1, 1792 * 384, 0, 0.1))),
                                      lambda I, F: orf.gemm_bf16(I.reshape(256, 384), F.reshape(1792, 384), b_is_nk=True), 1e-2, True),
+        "gemm_bf16_256x448x1792_p2": (lambda s: (f32_to_bf16(fill_normal(s, 256 * 448, 0, 1)), f32_to_bf16(fill_normal(s + 1, 1792 * 448, 0, 0.1))),
+                                      lambda I, F: orf.gemm_bf16(I.reshape(256, 448), F.reshape(1792, 448), b_is_nk=True), 1e-2, True),
         "rmsnorm_rope_bf16_6x1024": (lambda s: (f32_to_bf16(fill_normal(s, 6 * 1024, 0, 1.5)), _norm_rope_operand(6, 1024, 128, s + 1)),
                                      lambda I, F: orf.rmsnorm_rope_bf16(I.reshape(6, 1024), *wl.unpack_norm_rope_operand(F, 6, 1024, 128), heads=8, eps=1e-5), 1e-2, True),
     }
@@ -83,7 +85,9 @@ FUSIONS = [
     ("maxpool3x3s2_f32_4x16x16", "layernorm_8x256", "hfuse", ""),
     ("gemm_f32_128x160x192_d", "bias_relu_4096", "hfuse", ""),
     ("gemm_gelu_f32_64x192x288_d", "layernorm_8x256", "bfuse", "_c4"),
-    ("gemm_bf16_256x320x1792_w8", "rmsnorm_rope_bf16_6x1024", "hfuse", ""),   # a barrier in the K loop under hfuse: LDS arrival counter
+    ("gemm_bf16_256x320x1792_w8", "gemm_f32_128x160x192_d", "hfuse", ""),     # a barrier in the K loop, both sides synchronise: LDS arrival counters
+    ("gemm_bf16_256x384x1792_p", "rmsnorm_rope_bf16_6x1024", "hfuse", ""),    # the norm waves join the GEMM's hardware loop barriers
+    ("gemm_bf16_256x448x1792_p2", "rmsnorm_rope_bf16_6x1024", "hfuse", ""),   # the same with two producer waves (twelve waves in all)
     ("gemm_f32_128x160x192_d", "gemm_gelu_f32_64x192x288_d", "hfuse", ""),    # both sides synchronise: LDS arrival counters
     ("conv3x3_f32_32x12x12_32", "bias_relu_4096", "hfuse", ""),
     ("conv3x3_f32_64x8x16_16", "layernorm_8x256", "bfuse", "_c4"),
