@@ -40,3 +40,7 @@ BFUSE_BFUSE_RT_KERNEL(gemm_bf16_512x4096x14336_w8, GemmGate8, rmsnorm_rope_bf16_
 using NormRope4 = RmsNormRope<512, 32, 128, 4>;
 BFUSE_KERNEL(rmsnorm_rope_bf16_512x4096_w4, NormRope4, ({{512, 4096, 1, 1}, 2}), ({{(int)NormRope4::F_BYTES, 1, 1, 1}, 1}), ({{512, 4096, 1, 1}, 2}))
 BFUSE_BFUSE_KERNEL(gemm_bf16_512x4096x14336, GemmGate, rmsnorm_rope_bf16_512x4096_w4, NormRope4, _c256, bfuse::kChunked, 256, 1)
+// the headline GEMM's tiling on a K of 256: every tile position of the full 512 x 14336 output with
+// dense inputs, small enough for the CPU reference to evaluate the whole matrix
+using GemmGateK256 = GemmBf16NTDma<512, 14336, 256, 128, 224, 3, 4, 4, 2, 2>;
+BFUSE_KERNEL(gemm_bf16_512x256x14336, GemmGateK256, ({{512, 256, 1, 1}, 2}), ({{14336, 256, 1, 1}, 2}), ({{512, 14336, 1, 1}, 2}))

@@ -47,3 +47,26 @@ def rel_error(got, want):
     want = np.asarray(want, np.float32)
     rms = float(np.sqrt(np.mean(np.square(want.astype(np.float64)))))
     return orf.max_rel(got, want, rms)
+
+
+def rel_stats(got, want, tol):
+    """The acceptance rule next to the rule the configuration states ("relative").
+
+    Accepted here: |got - want| <= tol * max(|want|, rms(want)).  Pure relative error has no meaning
+    for outputs near zero (sums of ~K products of both signs cancel to values far below the size of
+    the terms, and the rounding of the TERMS does not shrink with the sum), hence the RMS floor.
+    Returned: the worst error under the accepted rule, the worst PURE relative error over the
+    elements that are not tiny (|want| >= 1e-3 rms), and how many elements pass only thanks to the
+    floor (pure relative error above tol)."""
+    g = np.asarray(got, np.float64).ravel()
+    w = np.asarray(want, np.float64).ravel()
+    rms = float(np.sqrt(np.mean(w * w)))
+    d = np.abs(g - w)
+    floor = np.maximum(np.abs(w), rms)
+    sizable = np.abs(w) >= 1e-3 * rms
+    pure = np.where(np.abs(w) > 0, d / np.maximum(np.abs(w), 1e-300), np.where(d > 0, np.inf, 0.0))
+    return {"n": int(g.size), "rms": rms, "worst_floor_rel": float((d / floor).max()),
+            "worst_pure_rel_sizable": float(pure[sizable].max()) if sizable.any() else 0.0,
+            "n_sizable": int(sizable.sum()),
+            "n_pass_only_by_floor": int(((pure > tol) & (d <= tol * floor)).sum()),
+            "n_fail": int((d > tol * floor).sum())}
