@@ -279,4 +279,42 @@ BFUSE_HD constexpr Dims3 delinearize(int linear, const Dims3& extent)
     return Dims3{linear % extent.x, linear / extent.x % extent.y, linear / (extent.x * extent.y)};
 }
 
+// GEMM tile of a workgroup id, dealt over the eight XCDs.
+//
+// The hardware sends consecutive workgroup ids to consecutive XCDs, and every XCD has an L2 of its
+// own: an operand slab that tiles on k different XCDs share is fetched k times (from HBM or the
+// last-level cache).  Here id % 8 is taken as the XCD and the GX x GY tile grid is cut into AX x AY
+// rectangles, one per XCD; id / 8 walks the rectangle.  An XCD then fetches GY / AY row slabs of A
+// (BM rows each) and GX / AX column slabs of B (BN columns each); AX x AY = 8 is chosen to make
+// that sum smallest.  When the grid cannot be cut that way the plain x-fastest order is kept.
+template <int GX, int GY, int BM, int BN>
+struct XcdTiles {
+    static constexpr int cost(int ax, int ay) { return (GY / ay) * BM + (GX / ax) * BN; }
+    static constexpr bool fits(int ax, int ay) { return GX % ax == 0 && GY % ay == 0; }
+    static constexpr int pick_ax()
+    {
+        int best = 0, best_cost = 0;
+        for (int ax = 1; ax <= 8; ax *= 2) {
+            const int ay = 8 / ax;
+            if (fits(ax, ay) && (best == 0 || cost(ax, ay) < best_cost)) {
+                best = ax;
+                best_cost = cost(ax, ay);
+            }
+        }
+        return best;
+    }
+    static constexpr int AX = pick_ax();                 // 0: the grid cannot be cut into eight equal rectangles
+    static constexpr int AY = AX ? 8 / AX : 0;
+    BFUSE_HD static constexpr Dims3 tile(int id)
+    {
+        if constexpr (AX == 0) {
+            return Dims3{id % GX, id / GX, 0};
+        } else {
+            constexpr int RX = GX / AX;
+            const int xcd = id & 7, slot = id >> 3;
+            return Dims3{(xcd % AX) * RX + slot % RX, (xcd / AX) * (GY / AY) + slot / RX, 0};
+        }
+    }
+};
+
 }  // namespace bfuse

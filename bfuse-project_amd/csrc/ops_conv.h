@@ -72,7 +72,7 @@ struct Conv3x3F32Lds {
     static_assert(HW % TP == 0 && NGROUP % KS == 0 && W % 4 == 0, "pixel / reduction tiling");
     static_assert((2 * WP + 2) * 16 + 3 * PLANE < 65536, "tap offsets are 16-bit immediates");
 
-    static constexpr Dims3 GRID{NPT, CO / BM, 1};
+    static constexpr Dims3 GRID{NPT * (CO / BM), 1, 1};
     static constexpr Dims3 BLOCK{64 * KS, 1, 1};
     static constexpr int THREADS = 64 * KS;
     static constexpr bool HAS_BARRIERS = KS > 1;
@@ -81,6 +81,28 @@ struct Conv3x3F32Lds {
     struct Smem {
         __attribute__((aligned(16))) unsigned char t[KS * TILE_BYTES > PART_BYTES ? KS * TILE_BYTES : PART_BYTES];
     };
+
+    // Workgroup id -> (pixel tile, output-channel tile).  Consecutive ids go to consecutive XCDs, each
+    // with an L2 of its own, so id % 8 is taken as the XCD and id / 8 walks (pixel tile, channel tile)
+    // within it: the CO / BM workgroups that share a pixel tile -- and with it an image patch -- run on
+    // one XCD, and an XCD owns CONSECUTIVE pixel tiles, whose patches overlap in image rows.  Each L2
+    // then fetches its eighth of the image (plus halo rows) once; with ids simply running over the
+    // pixel tiles of one channel tile after the other, every L2 fetches most of the image.
+    static constexpr int NCT = CO / BM;
+    __device__ static __forceinline__ void tile_of(int vblock, int& pt, int& ct)
+    {
+        constexpr int PER_XCD = NPT / 8;                 // whole pixel tiles every XCD owns
+        constexpr int FULL = 8 * PER_XCD * NCT;          // ids covered by them
+        if (vblock < FULL) {
+            const int xcd = vblock & 7, slot = vblock >> 3;
+            pt = xcd * PER_XCD + slot / NCT;
+            ct = slot % NCT;
+        } else {                                         // the NPT % 8 pixel tiles left over
+            const int rem = vblock - FULL;
+            pt = 8 * PER_XCD + rem / NCT;
+            ct = rem % NCT;
+        }
+    }
 
     // accumulator layout: lane (j = pixel, rg) owns output channels 4*rg+v of the block
     __device__ static __forceinline__ void store_block(float* __restrict__ Y, int co0, int p0, int tm, int pb,
@@ -99,8 +121,9 @@ struct Conv3x3F32Lds {
         const float* __restrict__ X = static_cast<const float*>(I);
         const float* __restrict__ Wt = static_cast<const float*>(F);
         float* __restrict__ Y = static_cast<float*>(O);
-        const Dims3 vb = delinearize(vblock, GRID);
-        const int p0 = vb.x * TP, co0 = vb.y * BM;
+        int pt, ct;
+        tile_of(vblock, pt, ct);
+        const int p0 = pt * TP, co0 = ct * BM;
         const int y_lo = p0 / W;                       // first image row of the tile; staged row 0 is y_lo - 1
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;   // wave-uniform: addresses built on it stay in scalar registers
         const int li = lane & 15, kq = lane >> 4;

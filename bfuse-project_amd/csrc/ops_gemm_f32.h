@@ -195,7 +195,7 @@ struct GemmF32 {
         const float* __restrict__ A = static_cast<const float*>(I);
         const float* __restrict__ B = static_cast<const float*>(F);
         float* __restrict__ C = static_cast<float*>(O);
-        const Dims3 vb = delinearize(vblock, GRID);
+        const Dims3 vb = XcdTiles<N / BN, M / BM, BM, BN>::tile(vblock);   // tiles dealt so that each XCD's L2 fetches as little as possible
         const int m0 = vb.y * BM, n0 = vb.x * BN;
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;   // wave-uniform: addresses built on it stay in scalar registers
         const int kbeg = wave * KW;
