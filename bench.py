@@ -134,7 +134,7 @@ def pick_fusion(number, spec):
 def measure(number, K, W, spec):
     import bfuse_project_amd as bf
     from bfuse_project_amd import tuner
-    from bfuse_project_amd.workloads import PAIRS, MEASURED_TRAFFIC, TRAFFIC_SOURCE, CONFIG_KINDS, BESIDE
+    from bfuse_project_amd.workloads import PAIRS, MEASURED_TRAFFIC, TRAFFIC_SOURCE, CONFIG_KINDS, BESIDE, FLOORS
 
     pair = PAIRS[number]
     k1, k2, kind, suffix, note = pick_fusion(number, spec)
@@ -243,6 +243,8 @@ def measure(number, K, W, spec):
                      "algorithmic": {"flops": pair.flops, "bytes": pair.bytes1 + pair.bytes2}},
         **extra,
     }
+    if number in FLOORS:
+        res["floor"] = FLOORS[number]
     return res, dev, inputs
 
 
