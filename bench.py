@@ -63,17 +63,25 @@ def cpu_baseline(pair_number, I1, F1, I2, F2, passes=5):
         return b
 
     if pair_number == 5:
-        # the full bf16 GEMM takes minutes on the CPU: time a 1/64 strided sample of its outputs
-        # (64 rows x 1792 columns over the full K) and scale; the RMSNorm+RoPE side is timed in full
+        # The bf16 GEMM is 60 GFLOP in double on the CPU: ~1.5 s on a GPU box's host cores, minutes on a
+        # small host.  A 1/64 strided sample of its outputs (64 rows x 1792 columns over the full K) is
+        # timed first; if that projects to a few seconds the whole GEMM is timed, otherwise the sample is
+        # scaled.  The RMSNorm+RoPE side is timed in full either way.
         from bfuse_project_amd.workloads import unpack_norm_rope_operand
         A, Wt = I1.reshape(512, 4096), F1.reshape(14336, 4096)
         As, Ws = np.ascontiguousarray(A[3::8]), np.ascontiguousarray(Wt[5::8])
         w, cosv, sinv = unpack_norm_rope_operand(F2, 512, 4096, 128)
-        t_g = best(lambda: orf.gemm_bf16(As, Ws, b_is_nk=True))
+        t_s = best(lambda: orf.gemm_bf16(As, Ws, b_is_nk=True))
         t_n = best(lambda: orf.rmsnorm_rope_bf16(I2.reshape(512, 4096), w, cosv, sinv, heads=32, eps=1e-5))
-        total = t_g * 64 + t_n
-        sample = (f"GEMM timed on a 1/64 strided sample of the outputs (64x1792 over K=4096, {t_g * 1e3:.1f} ms) and "
-                  f"scaled x64; RMSNorm+RoPE in full ({t_n * 1e3:.2f} ms); best of {passes}")
+        if t_s * 64 <= 5.0:
+            t_g = best(lambda: orf.gemm_bf16(A, Wt, b_is_nk=True))
+            total = t_g + t_n
+            sample = (f"the whole pair: GEMM 512x4096x14336 in full ({t_g * 1e3:.0f} ms; its 1/64 output sample alone {t_s * 1e3:.1f} ms), "
+                      f"RMSNorm+RoPE in full ({t_n * 1e3:.2f} ms); OpenMP, double accumulation, best of {passes}")
+        else:
+            total = t_s * 64 + t_n
+            sample = (f"GEMM timed on a 1/64 strided sample of the outputs (64x1792 over K=4096, {t_s * 1e3:.1f} ms) and "
+                      f"scaled x64; RMSNorm+RoPE in full ({t_n * 1e3:.2f} ms); best of {passes}")
     else:
         total = best(lambda: oracle_cases.expected(pair_number, I1, F1, I2, F2))
         sample = f"best of {passes} full passes of pair {pair_number} (both operators, OpenMP, double accumulation)"

@@ -234,3 +234,31 @@ def test_full_size_norm_sides_with_non_trivial_parameters():
         Q1, Q2 = op.run_fuse(op.fused("hfuse"), A, Wt, xb, F)
     assert np.array_equal(Q1.view(np.uint8), O1.view(np.uint8))
     assert np.array_equal(Q2.view(np.uint8), outs["rmsnorm_rope_bf16_512x4096_w2"].view(np.uint8))
+
+
+def test_pair5_gemm_whole_matrix_at_full_k_when_the_host_is_fast_enough():
+    """The whole 512 x 14336 output of pair 5's GEMM at the full K = 4096 against the CPU oracle.
+    The oracle needs 60 GFLOP in double for it: about 1.5 s on the GPU box's 16 host threads, minutes
+    on a small host, so the sample (1/64 of the outputs) is timed first and the whole matrix is
+    checked when that projects to under 40 s; otherwise the test says so and is skipped."""
+    import time
+    from oracle import oracle as orf
+    from bfuse_project_amd.operation import bf16_to_f32
+    pair = PAIRS[5]
+    A, W, _, _ = pair.inputs()
+    A2, W2 = A.reshape(512, 4096), W.reshape(14336, 4096)
+    t0 = time.perf_counter()
+    orf.gemm_bf16(np.ascontiguousarray(A2[3::8]), np.ascontiguousarray(W2[5::8]), b_is_nk=True)
+    projected = (time.perf_counter() - t0) * 64
+    _say(f"[pair 5] whole matrix at full K: the CPU oracle is projected to take {projected:.1f} s on {orf.num_threads()} threads")
+    if projected > 40:
+        pytest.skip(f"host too slow for the full 60 GFLOP oracle ({projected:.0f} s projected); the 1/64 sample and the K-reduced whole matrix cover it")
+    want = bf16_to_f32(orf.gemm_bf16(A2, W2, b_is_nk=True))
+    with bf.Operation(pair.k1, pair.k2) as op:
+        got = bf16_to_f32(op.run_kernel(0, A, W))
+    st = oracle_cases.rel_stats(got, want, pair.tol)
+    same = float(np.mean(got.ravel() == want.ravel()))
+    _say(f"[parity] pair 5 whole matrix, full K: worst |d|/max(|ref|,rms) {st['worst_floor_rel']:.3e}; worst pure relative over "
+         f"|ref| >= 1e-3 rms {st['worst_pure_rel_sizable']:.3e}; {st['n_pass_only_by_floor']} pass only by the floor; {st['n_fail']} fail; "
+         f"{100 * same:.3f} % bit-identical to the oracle")
+    assert st["n_fail"] == 0 and same > 0.95
