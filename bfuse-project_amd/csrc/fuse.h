@@ -13,8 +13,10 @@
 //            with a few workgroups per CU it is the persistent-block form of
 //            legacy/tests/thread_pooling_test/temp.cu:576-612
 //   hfuse  : horizontal fusion -- one workgroup hosts both operators on disjoint wave
-//            ranges; LDS is the sum of both sides; an intra-side barrier is the LDS-counter
-//            GroupSync instead of CUDA's bar.sync id,count (Matchers.cc:288-320, 655-727)
+//            ranges; LDS is the sum of both sides; where CUDA has bar.sync id,count
+//            (Matchers.cc:288-320, 655-727) a side keeps the hardware barrier when that is
+//            harmless, gets the LDS-counter GroupSync, or keeps the hardware barrier while the
+//            barrier-free partner joins it (JoinSync) -- chosen per pair at compile time
 //
 // Every instantiation calls the same Op::run body with a virtual (block, thread) id -- the
 // counterpart of the reference rewriting blockIdx/threadIdx to locals (Matchers.cc:255-286)

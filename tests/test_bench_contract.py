@@ -1,0 +1,48 @@
+"""The benchmark's command-line contract: one GPU only, one JSON line with the agreed keys."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_more_than_one_gpu_is_refused_with_a_message():
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=60)
+    assert r.returncode != 0 and "ONE GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_a_pinned_fusion_needs_a_pair():
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--fusion", "bfuse:_c8"], capture_output=True, text=True, timeout=60)
+    assert r.returncode != 0 and "--pair" in r.stderr
+
+
+@pytest.mark.gpu
+def test_one_json_line_covering_all_five_pairs():
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--steps", "20", "--warmup", "5"],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [l for l in r.stdout.splitlines() if l.strip()]
+    assert len(lines) == 1
+    d = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling", "vs_baseline",
+                "dtype", "data", "config", "roofline", "cpu_baseline", "pairs"):
+        assert key in d, key
+    assert d["n_gpus"] == 1 and d["steps"] == 20 and d["warmup"] == 5 and d["higher_is_better"] is False and d["vs_baseline"] is None
+    assert d["dtype"] == "bf16" and d["config"]["workload"].startswith("pair 5")
+    assert sorted(d["pairs"]) == ["1", "2", "3", "4", "5"]
+    assert d["value"] == d["pairs"]["5"]["fused_us"] and d["roofline"] == d["pairs"]["5"]["roofline"]
+    rf = d["roofline"]
+    assert rf["bound"] == "mfma" and rf["peak"] == 2500.0 and rf["unit"] == "TFLOP/s"
+    assert abs(rf["frac"] - rf["achieved"] / rf["peak"]) < 1e-3
+    assert abs(rf["achieved"] - rf["algorithmic"]["flops"] / d["value"] * 1e-6) < 0.5
+    assert rf["traffic"] and rf["traffic_source"].startswith("profiles/") and os.path.exists(os.path.join(ROOT, rf["traffic_source"]))
+    cb = d["cpu_baseline"]
+    assert cb["kind"] == "port" and cb["cores"] >= 1 and cb["value"] > 0 and cb["sample"]
+    for n, p in d["pairs"].items():
+        assert p["bit_exact_vs_unfused"] is True, n
+        assert p["chooser"]["is_measured_kernel"] is True, n
+        assert 0 < p["fused_us"] < p["serial_sum_us"], n
+    assert "zigzag_1to1" in d["pairs"]["3"] and "block_fused_chunk256" in d["pairs"]["5"] and "floor" in d["pairs"]["1"]
