@@ -14,8 +14,10 @@ compiler produced (`hipcc -save-temps`) and checks it:
   * a wait `lgkmcnt(n)` with n > 0 retires all but the n youngest LDS operations, which is only
     sound while nothing but LDS operations is in flight (they return in order; scalar loads do
     not): a scalar-memory load in flight together with a tracked read at such a wait is an error;
-  * a tracked read still in flight at `s_endpgm`, or at a backward branch (the rolled K loops wait
-    for everything they issued before they branch), is an error.
+  * a tracked read still in flight at `s_endpgm` is an error, and so is a backward branch taken with
+    other reads in flight (other registers, or another order) than the loop was entered with: a
+    software-pipelined K loop carries the first reads of its next step round the branch, in the
+    registers that held them on entry.
 
 The scan is linear over each kernel's text (forward branches are passed straight through), which
 is how the hand-written sequences are laid out; operations the compiler itself has in flight are
@@ -56,7 +58,7 @@ def check(path):
     func = None
     in_asm = False
     queue = []          # LDS / scalar-memory operations in flight, oldest first: (tracked regs or None, is_smem, line no)
-    labels_seen = set()
+    labels_seen = {}        # label -> destinations of the hand-issued reads in flight when the scan passed it
     n_tracked = 0
     for ln, raw in enumerate(open(path, errors="replace"), 1):
         line = raw.split(";;#", 1)[0] if ";;#" in raw and not raw.strip().startswith(";;#") else raw
@@ -71,9 +73,9 @@ def check(path):
         if m:
             name = m.group(1)
             if not name.startswith(".L"):
-                func, queue, labels_seen = name, [], set()
+                func, queue, labels_seen = name, [], {}
             else:
-                labels_seen.add(name)
+                labels_seen[name] = [q[0] for q in queue if q[0]]
                 # A basic-block boundary: what the compiler itself has in flight here depends on the
                 # path taken, which a linear scan does not know; its own waits take care of those.
                 # Forgetting them is the conservative side for the hand-issued reads (fewer younger
@@ -122,8 +124,12 @@ def check(path):
             continue
         if mn.startswith("s_cbranch") or mn == "s_branch":
             target = ops.strip()
-            if target in labels_seen and tracked_in_flight:     # backward branch
-                findings.append(f"{path}:{ln}: {func}: backward branch with the asm LDS read from line {tracked_in_flight[0][2]} in flight")
+            # backward branch: the loop head is entered again with exactly the reads in flight that
+            # the code after it was checked with (same registers, same order), or with none
+            if target in labels_seen and [q[0] for q in tracked_in_flight] != labels_seen[target]:
+                at = tracked_in_flight[0][2] if tracked_in_flight else ln
+                findings.append(f"{path}:{ln}: {func}: backward branch to {target} with other hand-issued LDS reads in flight "
+                                f"(first from line {at}) than when the loop was entered")
             continue
         if counts_in_lgkm(mn):
             if in_asm and mn.startswith("ds_read"):

@@ -11,8 +11,8 @@ BFUSE_MODULE_PROLOGUE()
 
 // 128 x 224 tiles: 4 x 64 = 256 workgroups; eight compute waves (4 x 2) of 32 x 112 plus two
 // producer waves that issue the direct-to-LDS loads (two, three and four producers run the same:
-// 47.6-47.8 us); ring of three 64-k stages
-using GemmGate = GemmBf16NTDma<512, 14336, 4096, 128, 224, 3, 4, 4, 2, 2>;
+// 47.6-47.8 us); ring of three 64-k stages; the barrier of the next K-step before MFMA group 11 of 14
+using GemmGate = GemmBf16NTDma<512, 14336, 4096, 128, 224, 3, 4, 4, 2, 2, 11>;
 using NormRope1 = RmsNormRope<512, 32, 128, 1>;             // 512 one-wave workgroups
 
 BFUSE_KERNEL(gemm_bf16_512x4096x14336, GemmGate, ({{512, 4096, 1, 1}, 2}), ({{14336, 4096, 1, 1}, 2}), ({{512, 14336, 1, 1}, 2}))
@@ -42,5 +42,5 @@ BFUSE_KERNEL(rmsnorm_rope_bf16_512x4096_w4, NormRope4, ({{512, 4096, 1, 1}, 2}),
 BFUSE_BFUSE_KERNEL(gemm_bf16_512x4096x14336, GemmGate, rmsnorm_rope_bf16_512x4096_w4, NormRope4, _c256, bfuse::kChunked, 256, 1)
 // the headline GEMM's tiling on a K of 256: every tile position of the full 512 x 14336 output with
 // dense inputs, small enough for the CPU reference to evaluate the whole matrix
-using GemmGateK256 = GemmBf16NTDma<512, 14336, 256, 128, 224, 3, 4, 4, 2, 2>;
+using GemmGateK256 = GemmBf16NTDma<512, 14336, 256, 128, 224, 3, 4, 4, 2, 2, 11>;
 BFUSE_KERNEL(gemm_bf16_512x256x14336, GemmGateK256, ({{512, 256, 1, 1}, 2}), ({{14336, 256, 1, 1}, 2}), ({{512, 14336, 1, 1}, 2}))

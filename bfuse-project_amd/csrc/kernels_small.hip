@@ -60,8 +60,8 @@ using GemmB1 = GemmBf16NTDma<128, 1792, 64, 128, 224, 2>;             // one K-s
 using GemmB2 = GemmBf16NTDma<128, 1792, 192, 128, 224, 2>;            // two stages, three K-steps
 using GemmB3 = GemmBf16NTDma<256, 1792, 320, 128, 224, 3>;            // two M-tiles, ring of three, five K-steps
 using GemmB5 = GemmBf16NTDma<256, 1792, 320, 128, 224, 3, 4, 4, 2>;   // the same with eight waves (uneven load groups per wave)
-using GemmB8 = GemmBf16NTDma<256, 1792, 384, 128, 224, 3, 4, 4, 2, 4>;   // eight compute + four producer waves
-using GemmB9 = GemmBf16NTDma<256, 1792, 448, 128, 224, 3, 4, 4, 2, 2>;   // eight compute + two producer waves, seven K-steps
+using GemmB8 = GemmBf16NTDma<256, 1792, 384, 128, 224, 3, 4, 4, 2, 4, 11>;   // eight compute + four producer waves, early barrier, six K-steps (all after the rolled loop)
+using GemmB9 = GemmBf16NTDma<256, 1792, 448, 128, 224, 3, 4, 4, 2, 2, 10>;   // eight compute + two producer waves, early barrier, seven K-steps (one round of the rolled loop, then the last step)
 using NormRopeS = RmsNormRope<6, 8, 128, 2>;
 
 BFUSE_KERNEL(gemm_f32_64x32x48, GemmS1, ({{64, 32, 1, 1}, 4}), ({{32, 48, 1, 1}, 4}), ({{64, 48, 1, 1}, 4}))

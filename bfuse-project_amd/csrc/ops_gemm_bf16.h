@@ -53,7 +53,15 @@ __device__ __forceinline__ float bf16_bits_to_f32(unsigned int h) { return __bui
 // another wave of the SIMD cost the MFMA wave nothing.  With PW_ extra waves the direct-to-LDS
 // loads are issued by them and the WGM_ x WGN_ compute waves issue only LDS reads and MFMAs.  All
 // waves take part in every barrier.
-template <int M_, int N_, int K_, int BM_, int BN_, int NSTG_ = 3, int PD_ = 4, int WGM_ = 2, int WGN_ = 2, int PW_ = 0>
+// EARLY_ > 0 (with producer waves): the barrier that certifies K-step kt+1 is taken inside step kt,
+// before MFMA group EARLY_ of its STEPS groups, and the first operand fragments of step kt+1 are
+// requested right after it, so that they arrive while the last groups of step kt multiply.  With the
+// barrier at the top of the step every wave of the workgroup waits for its first LDS reads at the
+// same moment and the matrix cores idle for that long once per step.  The fragments of two
+// consecutive steps live in two register sets, so the rolled loop holds 2 * NSTG_ steps.  Measured
+// on MI355X on the 512 x 4096 x 14336 instance, both forms in one run: 46.8 against 48.2 us, and
+// 47.8 against 49.4-49.8 us with the norm waves fused in.
+template <int M_, int N_, int K_, int BM_, int BN_, int NSTG_ = 3, int PD_ = 4, int WGM_ = 2, int WGN_ = 2, int PW_ = 0, int EARLY_ = 0>
 struct GemmBf16NTDma {
     static constexpr int M = M_, N = N_, K = K_, BM = BM_, BN = BN_, NSTG = NSTG_;
     static constexpr int BK = 64;
@@ -221,6 +229,94 @@ struct GemmBf16NTDma {
         }
     }
 
+    // ---- the same chain with the next step's barrier and first reads inside it (EARLY_) -----------
+    static constexpr int EARLY = EARLY_;
+    static_assert(EARLY_ == 0 || (PW_ > 0 && BK / 32 == 2 && EARLY_ >= STEPS - PD_ && EARLY_ > 1 && EARLY_ < STEPS),
+                  "the early barrier needs producer waves and comes after the step's last read has been issued");
+    struct Frags {
+        bf16x8 af[BK / 32][TM], bq[RING];
+    };
+    // every read of the step has been issued: wait for all of them; the fragments still to be used are named
+    __device__ static __forceinline__ void wait_rest(Frags& f)
+    {
+#if defined(__HIP_DEVICE_COMPILE__)
+        // (an operand named twice would make the compiler copy it -- a register with a read in flight)
+        static_assert(TM == 2 || TM == 4, "the wait names two or four A fragments");
+        constexpr int G = EARLY_ > 0 ? EARLY_ : STEPS - 1, REST = STEPS - G;
+        static_assert(REST >= 1 && REST <= 4, "the wait names at most four B fragments");
+        bf16x8(&a)[TM] = f.af[1];
+        bf16x8& a2 = a[TM == 4 ? 2 : 0];   // only named when TM == 4
+        bf16x8& a3 = a[TM == 4 ? 3 : 1];
+        bf16x8& b0 = f.bq[G % RING];
+        bf16x8& b1 = f.bq[(G + 1) % RING];
+        bf16x8& b2 = f.bq[(G + 2) % RING];
+        bf16x8& b3 = f.bq[(G + 3) % RING];
+#define BFUSE_WAIT_REST(...)                                                                                            \
+    do {                                                                                                                \
+        if constexpr (TM == 4) asm volatile("s_waitcnt lgkmcnt(0)" : __VA_ARGS__, "+v"(a[0]), "+v"(a[1]), "+v"(a2), "+v"(a3)); \
+        else asm volatile("s_waitcnt lgkmcnt(0)" : __VA_ARGS__, "+v"(a[0]), "+v"(a[1]));                               \
+    } while (0)
+        if constexpr (REST == 1) BFUSE_WAIT_REST("+v"(b0));
+        else if constexpr (REST == 2) BFUSE_WAIT_REST("+v"(b0), "+v"(b1));
+        else if constexpr (REST == 3) BFUSE_WAIT_REST("+v"(b0), "+v"(b1), "+v"(b2));
+        else BFUSE_WAIT_REST("+v"(b0), "+v"(b1), "+v"(b2), "+v"(b3));
+#undef BFUSE_WAIT_REST
+#endif
+    }
+    // LAST: this is the final K-step, there is no next step to meet for
+    template <int U, int ST, bool LAST, class Sync>
+    __device__ static __forceinline__ void early_chain(f32x4 (&acc)[TM][TN], Frags& cur, Frags& nxt, const Addr& ad, Sync& sync)
+    {
+        if constexpr (ST < STEPS) {
+            constexpr int ks = ST / TN, b = ST % TN;
+            if constexpr (ST < EARLY_) {
+                wait_lds<allowed(ST)>(cur.bq[ST % RING], cur.af[ks]);
+            } else if constexpr (ST == EARLY_) {
+                wait_rest(cur);
+                if constexpr (!LAST) {
+                    // K-step kt+1 is in LDS (the producers waited for it) and every wave has read all of
+                    // step kt: its slot may be refilled, and step kt+1's first fragments are requested now
+                    sync.bare();
+                    read_a_all<(U + 1) % NSTG, 0, 0>(nxt.af[0], ad);
+                    read_b_first<(U + 1) % NSTG, 0>(nxt.bq, ad);
+                }
+            }
+#pragma unroll
+            for (int a = 0; a < TM; ++a)
+                acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.af[ks][a], cur.bq[ST % RING], acc[a][b], 0, 0, 0);
+            if constexpr (ST + PD < STEPS) cur.bq[(ST + PD) % RING] = read_b<U, (ST + PD) / TN, (ST + PD) % TN>(ad);
+            if constexpr (b == 1 && ks + 1 < BK / 32) {
+                read_a_all<U, ks + 1, 0>(cur.af[ks + 1], ad);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            early_chain<U, ST + 1, LAST>(acc, cur, nxt, ad, sync);
+        }
+    }
+    // K-step S (compile-time position in a group of 2 * NSTG steps): ring slot S % NSTG, fragment set S % 2
+    template <int S, bool LAST, class Sync>
+    __device__ static __forceinline__ void early_step(f32x4 (&acc)[TM][TN], Frags (&fr)[2], const Addr& ad, Sync& sync)
+    {
+        early_chain<S % NSTG, 0, LAST>(acc, fr[S % 2], fr[(S + 1) % 2], ad, sync);
+    }
+    static constexpr int UNR = 2 * NSTG_;                                      // slots and fragment sets are back where they started
+    static constexpr int MAIN_STEPS = NKT > 1 ? ((NKT - 1) / UNR) * UNR : 0;   // in the rolled loop; the last step is never in it
+    template <int J, class Sync>
+    __device__ static __forceinline__ void early_main(f32x4 (&acc)[TM][TN], Frags (&fr)[2], const Addr& ad, Sync& sync)
+    {
+        if constexpr (J < UNR) {
+            early_step<J, false>(acc, fr, ad, sync);
+            early_main<J + 1>(acc, fr, ad, sync);
+        }
+    }
+    template <int S, class Sync>
+    __device__ static __forceinline__ void early_tail(f32x4 (&acc)[TM][TN], Frags (&fr)[2], const Addr& ad, Sync& sync)
+    {
+        if constexpr (S < NKT) {
+            early_step<S % UNR, S == NKT - 1>(acc, fr, ad, sync);
+            early_tail<S + 1>(acc, fr, ad, sync);
+        }
+    }
+
     // one K-step out of LDS stage U
     // the loading half of a K-step: wait for own loads of step kt, meet, refill the stage step kt-1 used
     template <int U, class Sync>
@@ -325,12 +421,23 @@ struct GemmBf16NTDma {
         // the loop stays rolled whatever K is: operand registers with reads in flight must never be
         // spilled (the compiler takes an asm output for written when the asm is issued), and a
         // fully unrolled short loop is where the register allocator runs out
+        if constexpr (EARLY_ > 0) {
+            Frags fr[2];
+            sync.raw();   // K-step 0 is in LDS
+            read_a_all<0, 0, 0>(fr[0].af[0], ad);
+            read_b_first<0, 0>(fr[0].bq, ad);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll 1
-        for (int kt0 = 0; kt0 < NKT; kt0 += NSTG) {
-            k_step<0, PW == 0>(kt0, acc, ad, src, lds, full, sync);
-            if constexpr (NSTG > 1) k_step<1, PW == 0>(kt0 + 1, acc, ad, src, lds, full, sync);
-            if constexpr (NSTG > 2) k_step<2, PW == 0>(kt0 + 2, acc, ad, src, lds, full, sync);
-            if constexpr (NSTG > 3) k_step<3, PW == 0>(kt0 + 3, acc, ad, src, lds, full, sync);
+            for (int kt0 = 0; kt0 < MAIN_STEPS; kt0 += UNR) early_main<0>(acc, fr, ad, sync);
+            early_tail<MAIN_STEPS>(acc, fr, ad, sync);
+        } else {
+#pragma unroll 1
+            for (int kt0 = 0; kt0 < NKT; kt0 += NSTG) {
+                k_step<0, PW == 0>(kt0, acc, ad, src, lds, full, sync);
+                if constexpr (NSTG > 1) k_step<1, PW == 0>(kt0 + 1, acc, ad, src, lds, full, sync);
+                if constexpr (NSTG > 2) k_step<2, PW == 0>(kt0 + 2, acc, ad, src, lds, full, sync);
+                if constexpr (NSTG > 3) k_step<3, PW == 0>(kt0 + 3, acc, ad, src, lds, full, sync);
+            }
         }
         sync();  // all waves are done reading the last stage before the tile buffer overwrites it
 

@@ -64,6 +64,19 @@ def test_reads_never_waited_for_and_reads_across_a_backward_branch_are_flagged(t
     assert len(findings) == 1 and "backward branch" in findings[0]
 
 
+def test_a_loop_may_carry_reads_round_its_branch_in_the_registers_it_was_entered_with(tmp_path):
+    use_a = WAIT.format(n=0) + "\tv_mfma_f32_16x16x32_bf16 a[4:7], v[20:23], v[30:33], a[4:7]\n"
+    # software pipelining: the first read of the next step is in flight at the loop head, each time
+    findings, _ = _run(tmp_path, READ_A + ".LBB0_1:\n" + use_a + READ_A + "\ts_cbranch_scc1 .LBB0_1\n" + use_a)
+    assert findings == []
+    # the branch is taken with the read in other registers than the loop head expects
+    findings, _ = _run(tmp_path, READ_A + ".LBB0_1:\n" + use_a + READ_B + "\ts_cbranch_scc1 .LBB0_1\n" + use_a)
+    assert len(findings) == 1 and "backward branch" in findings[0]
+    # ... or with nothing in flight where the loop head was entered with a read
+    findings, _ = _run(tmp_path, READ_A + ".LBB0_1:\n" + use_a + "\ts_cbranch_scc1 .LBB0_1\n")
+    assert len(findings) == 1 and "backward branch" in findings[0]
+
+
 def test_the_compilers_own_reads_are_not_tracked_but_take_a_counter_slot(tmp_path):
     # a compiler-issued ds_read after the asm read is the youngest: lgkmcnt(1) retires the asm read
     body = READ_A + "\tds_read_b32 v50, v51\n" + "\ts_waitcnt lgkmcnt(1)\n" + "\tv_mov_b32_e32 v40, v20\n" + "\ts_waitcnt lgkmcnt(0)\n"
