@@ -31,6 +31,15 @@ __device__ __forceinline__ unsigned int f32_to_bf16_bits(float f)
     u += 0x7fffu + ((u >> 16) & 1u);
     return u >> 16;
 }
+// two fp32 -> two bf16 in one word (lo in the low half), round to nearest even: v_cvt_pk_bf16_f32
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ unsigned int pack_bf16(float lo, float hi)
+{
+    const f32x2 v = {lo, hi};
+    return __builtin_bit_cast(unsigned int, __builtin_convertvector(v, bf16x2));
+}
 __device__ __forceinline__ float bf16_bits_to_f32(unsigned int h) { return __builtin_bit_cast(float, h << 16); }
 
 // The K-pipeline is built around direct global->LDS loads
@@ -219,7 +228,7 @@ struct GemmBf16NTDma {
             wait_lds<allowed(ST)>(bq[ST % RING], af[ks]);
 #pragma unroll
             for (int a = 0; a < TM; ++a)
-                acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[ks][a], bq[ST % RING], acc[a][b], 0, 0, 0);
+                acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bq[ST % RING], af[ks][a], acc[a][b], 0, 0, 0);
             if constexpr (ST + PD < STEPS) bq[(ST + PD) % RING] = read_b<U, (ST + PD) / TN, (ST + PD) % TN>(ad);
             if constexpr (b == 1 && ks + 1 < BK / 32) {
                 read_a_all<U, ks + 1, 0>(af[ks + 1], ad);
@@ -283,7 +292,7 @@ struct GemmBf16NTDma {
             }
 #pragma unroll
             for (int a = 0; a < TM; ++a)
-                acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.af[ks][a], cur.bq[ST % RING], acc[a][b], 0, 0, 0);
+                acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.bq[ST % RING], cur.af[ks][a], acc[a][b], 0, 0, 0);
             if constexpr (ST + PD < STEPS) cur.bq[(ST + PD) % RING] = read_b<U, (ST + PD) / TN, (ST + PD) % TN>(ad);
             if constexpr (b == 1 && ks + 1 < BK / 32) {
                 read_a_all<U, ks + 1, 0>(cur.af[ks + 1], ad);
@@ -446,11 +455,15 @@ struct GemmBf16NTDma {
 #pragma unroll
             for (int a = 0; a < TM; ++a)
 #pragma unroll
-                for (int b = 0; b < TN; ++b)
-#pragma unroll
-                    for (int v = 0; v < 4; ++v)
-                        ct[(wm * WM + a * 16 + 4 * kq + v) * CPITCH + wn * WN + b * 16 + li] =
-                            (unsigned short)f32_to_bf16_bits(acc[a][b][v]);
+                for (int b = 0; b < TN; ++b) {
+                    // the W fragment is the MFMA's first operand: a lane holds four consecutive n of
+                    // one output row (m = li), eight bytes of the tile once rounded
+                    const f32x4 r = acc[a][b];
+                    u32x2 packed;
+                    packed[0] = pack_bf16(r[0], r[1]);
+                    packed[1] = pack_bf16(r[2], r[3]);
+                    *reinterpret_cast<u32x2*>(ct + (wm * WM + a * 16 + li) * CPITCH + wn * WN + b * 16 + 4 * kq) = packed;
+                }
         }
         sync();
         if (compute) {
