@@ -9,4 +9,4 @@ from .patterns import (  # noqa: F401
     LaunchDims, plan_threads, plan_blocks, PATTERNS,
 )
 from .config import KernelInfo, FusionInfo, load_kernels_yaml, load_fusions_yaml, dump_kernels_yaml, FusionContext  # noqa: F401
-from .operation import Operation, kernel_info, list_kernels  # noqa: F401
+from .operation import Operation, GroupOperation, kernel_info, list_kernels  # noqa: F401

@@ -45,7 +45,13 @@ class KernelInfoC(C.Structure):
                 ("grid", C.c_uint * 3), ("block", C.c_uint * 3), ("has_barriers", C.c_int),
                 ("regs", C.c_int), ("lds_bytes", C.c_int), ("shape", (C.c_int * 4) * 3),
                 ("elem_bytes", C.c_int * 3), ("side", (C.c_char * 64) * 2),
-                ("pattern", C.c_int), ("p0", C.c_int), ("p1", C.c_int)]
+                ("pattern", C.c_int), ("p0", C.c_int), ("p1", C.c_int),
+                ("n_sides", C.c_int), ("side_more", (C.c_char * 64) * (MAXK - 2))]
+
+
+class LaunchDescC(C.Structure):
+    _fields_ = [("func", C.c_void_p), ("grid", C.c_uint * 3), ("block", C.c_uint * 3),
+                ("n_sides", C.c_int), ("sides", C.c_int * MAXK)]
 
 
 # every symbol include/bfuse_rt.h declares
@@ -58,6 +64,7 @@ EXPORTS = [
     "run_kernel1", "run_kernel2", "run_parallel", "run_fuse",
     "bfuse_upload", "bfuse_zero_output", "bfuse_download", "bfuse_synchronize", "bfuse_launch",
     "bfuse_time", "bfuse_time_batched", "bfuse_module_load", "bfuse_module_unload", "bfuse_module_launch",
+    "bfuse_initialize_side", "bfuse_finalize_side", "bfuse_launch_list", "bfuse_time_list",
     "bfuse_fill_uniform", "bfuse_fill_normal", "bfuse_f32_to_bf16", "bfuse_bf16_to_f32", "bfuse_check_matrix",
 ]
 
@@ -109,6 +116,10 @@ def lib():
         fp = C.POINTER(C.c_float)
         l.bfuse_time.argtypes = [C.c_int, vp, up, up, vp, up, up, C.c_int, C.c_int, fp, fp, fp]
         l.bfuse_time_batched.argtypes = [C.c_int, vp, up, up, vp, up, up, C.c_int, C.c_int, fp]
+        l.bfuse_initialize_side.argtypes = [C.c_int, ip, ip, ip]
+        l.bfuse_finalize_side.argtypes = [C.c_int]
+        l.bfuse_launch_list.argtypes = [C.c_int, C.POINTER(LaunchDescC)]
+        l.bfuse_time_list.argtypes = [C.c_int, C.POINTER(LaunchDescC), C.c_int, C.c_int, fp, fp]
         l.bfuse_module_load.argtypes = [C.c_char_p, ip]
         l.bfuse_module_launch.argtypes = [C.c_int, C.c_char_p, up, up, C.c_int, C.c_int, fp]
         _LIB = l

@@ -26,12 +26,22 @@
 // Kernel ABI, as in the reference (macro_h.py:182-198): extern "C", three pointers per
 // operator (input, second operand, output), six for a fused pair (operator 1's three, then
 // operator 2's), 1-D launch, no dynamic shared memory.
+//
+// The reference's emitter fuses a LIST of kernels (horizontal-fuser/src/Algorithms.cc:23-35,
+// 540-566: the maps take any number of grids; Matchers.cc:523-602 concatenates the parameter
+// lists).  The pair templates below are the tuned forms the five headline pairs use; the
+// *_group templates further down are the same three fusions over up to kMaxKernels operators,
+// with 3 x n pointers in operator order.
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstring>
+#include <initializer_list>
 #include <string>
+#include <tuple>
 #include <type_traits>
+#include <utility>
 #include <vector>
 
 #include "dispatch.h"
@@ -201,6 +211,154 @@ __device__ __forceinline__ void hfuse_body(const void* I1, const void* F1, void*
     }
 }
 
+
+// ---- fusions of more than two operators ----------------------------------------------------
+struct SidePtrs {
+    const void* i;
+    const void* f;
+    void* o;
+};
+
+// LDS of the operators as a union (block fusion: one operator per workgroup) or one after the
+// other (horizontal fusion: all of them in every workgroup), Tools.cc:219-251
+template <class... Ops>
+union SmemUnion;
+template <class A>
+union SmemUnion<A> {
+    typename A::Smem head;
+};
+template <class A, class... R>
+union SmemUnion<A, R...> {
+    typename A::Smem head;
+    SmemUnion<R...> tail;
+};
+template <class... Ops>
+struct SmemSum;
+template <class A>
+struct SmemSum<A> {
+    typename A::Smem head;
+};
+template <class A, class... R>
+struct SmemSum<A, R...> {
+    typename A::Smem head;
+    SmemSum<R...> tail;
+};
+template <int K, class U>
+__device__ __forceinline__ auto& smem_at(U& u)
+{
+    if constexpr (K == 0) return u.head;
+    else return smem_at<K - 1>(u.tail);
+}
+
+template <class... Ops>
+struct GroupDims {
+    static constexpr int N = sizeof...(Ops);
+    static_assert(N >= 2 && N <= kMaxKernels, "a fusion takes two to kMaxKernels operators");
+    static_assert(((Ops::THREADS % kWaveSize == 0) && ...), "block sizes must be whole waves");
+    static constexpr LaunchDims dims[N] = {{Ops::GRID, Ops::BLOCK}...};
+    static constexpr int WIDEST = std::max({Ops::THREADS...});
+    static constexpr int SUM_THREADS = (round_up(Ops::THREADS, kWaveSize) + ...);
+    static constexpr int SUM_GRID = (Ops::GRID.size() + ...);
+    static constexpr int MAX_GRID = std::max({Ops::GRID.size()...});
+    static constexpr int BARRIER_SIDES = (int(Ops::HAS_BARRIERS) + ...);
+};
+
+template <int PATTERN, int P0, int P1, class... Ops>
+struct BfuseGroup : GroupDims<Ops...> {
+    using D = GroupDims<Ops...>;
+    static constexpr BlockPlan plan() { return make_block_plan(PATTERN, D::N, D::dims, P0, P1); }
+    static constexpr int THREADS = D::WIDEST;
+    static constexpr int GRID = D::SUM_GRID;
+};
+
+template <int PATTERN, int P0, int P1, class... Ops, int... K>
+__device__ __forceinline__ void bfuse_group_body(const SidePtrs (&p)[sizeof...(Ops)], std::integer_sequence<int, K...>)
+{
+    __shared__ SmemUnion<Ops...> su;
+    constexpr BlockPlan plan = BfuseGroup<PATTERN, P0, P1, Ops...>::plan();
+    int virt = 0;
+    const int kernel_id = map_block(plan, (int)blockIdx.x, &virt);
+    const int tid = (int)threadIdx.x;
+    // exactly one operator's body runs in a workgroup; waves past its block size leave
+    ((kernel_id == K && tid < Ops::THREADS ? (Ops::run(virt, tid, smem_at<K>(su), p[K].i, p[K].f, p[K].o, BlockSync{}), 0) : 0), ...);
+}
+
+template <class... Ops>
+struct BfuseRtGroup : GroupDims<Ops...> {
+    static constexpr int THREADS = GroupDims<Ops...>::WIDEST;
+    static constexpr int GRID = GroupDims<Ops...>::SUM_GRID;
+};
+
+template <int K, int T, class Op>
+__device__ __forceinline__ void rt_run_side(int virt, int tid, typename Op::Smem& sm, const SidePtrs& p, unsigned int* arrive)
+{
+    // see bfuse_rt_body: an operator narrower than the workgroup synchronises over its own waves
+    if constexpr (Op::THREADS == T) Op::run(virt, tid, sm, p.i, p.f, p.o, BlockSync{});
+    else Op::run(virt, tid, sm, p.i, p.f, p.o, GroupSync{arrive, (unsigned)(Op::THREADS / kWaveSize), 0u});
+}
+
+template <class... Ops, int... K>
+__device__ __forceinline__ void bfuse_rt_group_body(const BlockPlan& plan, const SidePtrs (&p)[sizeof...(Ops)],
+                                                    std::integer_sequence<int, K...>)
+{
+    constexpr int N = sizeof...(Ops);
+    struct Shrd {
+        SmemUnion<Ops...> u;
+        unsigned int arrive[3][N];   // three sets in rotation, as in bfuse_rt_body
+    };
+    __shared__ Shrd sh;
+    constexpr int T = BfuseRtGroup<Ops...>::THREADS;
+    const int tid = (int)threadIdx.x;
+    const int total = plan.fused_grid;
+    if (tid < 3 * N) (&sh.arrive[0][0])[tid] = 0u;
+    int set = 0;
+    for (int id = (int)blockIdx.x; id < total; id += (int)gridDim.x) {
+        const int next = set == 2 ? 0 : set + 1;
+        if (tid < N) sh.arrive[next][tid] = 0u;
+        __syncthreads();
+        int virt = 0;
+        const int kernel_id = map_block(plan, id, &virt);
+        ((kernel_id == K && tid < Ops::THREADS ? (rt_run_side<K, T, Ops>(virt, tid, smem_at<K>(sh.u), p[K], &sh.arrive[set][K]), 0) : 0), ...);
+        set = next;
+    }
+}
+
+template <class... Ops>
+struct HfuseGroup : GroupDims<Ops...> {
+    using D = GroupDims<Ops...>;
+    static constexpr ThreadPlan plan() { return plan_threads(D::N, D::dims, kWaveSize); }
+    static constexpr int THREADS = D::SUM_THREADS;
+    static constexpr int GRID = D::MAX_GRID;
+};
+
+template <int BARRIER_SIDES, class Op>
+__device__ __forceinline__ void hfuse_run_side(int local, typename Op::Smem& sm, const SidePtrs& p, unsigned int* arrive)
+{
+    // The only side that synchronises keeps the hardware barrier unless the barrier sits in its main
+    // loop (its first barrier waits until the other sides' waves have left, see hfuse_body); every
+    // other synchronising side meets on its own LDS arrival counter.
+    constexpr bool alone = BARRIER_SIDES - int(Op::HAS_BARRIERS) == 0;
+    if constexpr (alone && !loop_barriers<Op>::value) Op::run((int)blockIdx.x, local, sm, p.i, p.f, p.o, BlockSync{});
+    else Op::run((int)blockIdx.x, local, sm, p.i, p.f, p.o, GroupSync{arrive, (unsigned)(round_up(Op::THREADS, kWaveSize) / kWaveSize), 0u});
+}
+
+template <class... Ops, int... K>
+__device__ __forceinline__ void hfuse_group_body(const SidePtrs (&p)[sizeof...(Ops)], std::integer_sequence<int, K...>)
+{
+    constexpr int N = sizeof...(Ops);
+    struct ShrdSum {
+        SmemSum<Ops...> s;
+        unsigned int arrive[N];
+    };
+    __shared__ ShrdSum ss;
+    constexpr ThreadPlan plan = HfuseGroup<Ops...>::plan();
+    if (threadIdx.x < N) ss.arrive[threadIdx.x] = 0u;
+    __syncthreads();
+    int local = 0;
+    const int kernel_id = map_thread(plan, (int)blockIdx.x, (int)threadIdx.x, &local);
+    ((kernel_id == K ? (hfuse_run_side<GroupDims<Ops...>::BARRIER_SIDES, Ops>(local, smem_at<K>(ss.s), p[K], &ss.arrive[K]), 0) : 0), ...);
+}
+
 // ---- registry ---------------------------------------------------------------------------
 enum KernelKind : int { kSingle = 0, kBfuse = 1, kHfuse = 2, kBfuseRt = 3 };
 
@@ -216,7 +374,8 @@ struct KernelEntry {
     unsigned grid[3], block[3];
     bool has_barriers;
     TensorDesc io[3];       // single: I, F, O
-    std::string side[2];    // fused: names of the two standalone kernels
+    int n_sides;            // fused: how many standalone kernels it runs (2 .. kMaxKernels)
+    std::string side[kMaxKernels];   // fused: their names, in pointer order
     int pattern, p0, p1;    // bfuse: dispatch pattern and its parameters
     unsigned (*read_sync_timeouts)();  // device counter of GroupSync give-ups in this module (read and reset)
     int (*set_spin_limit)(unsigned);   // polls a side barrier of this module makes before it gives up (0 = ok)
@@ -253,7 +412,7 @@ KernelEntry make_single_entry(const char* name, const void* func, TensorDesc i, 
 }
 
 template <class Pair>
-KernelEntry make_fused_entry(const char* name, const void* func, int kind, const char* k1, const char* k2,
+KernelEntry make_group_entry(const char* name, const void* func, int kind, std::initializer_list<const char*> sides,
                              bool barriers, int pattern, int p0, int p1, const ModuleHooks& hooks)
 {
     KernelEntry e{};
@@ -263,11 +422,19 @@ KernelEntry make_fused_entry(const char* name, const void* func, int kind, const
     e.grid[0] = Pair::GRID; e.grid[1] = 1; e.grid[2] = 1;
     e.block[0] = Pair::THREADS; e.block[1] = 1; e.block[2] = 1;
     e.has_barriers = barriers;
-    e.side[0] = k1; e.side[1] = k2;
+    e.n_sides = 0;
+    for (const char* k : sides) e.side[e.n_sides++] = k;
     e.pattern = pattern; e.p0 = p0; e.p1 = p1;
     e.read_sync_timeouts = hooks.read_sync_timeouts;
     e.set_spin_limit = hooks.set_spin_limit;
     return e;
+}
+
+template <class Pair>
+KernelEntry make_fused_entry(const char* name, const void* func, int kind, const char* k1, const char* k2,
+                             bool barriers, int pattern, int p0, int p1, const ModuleHooks& hooks)
+{
+    return make_group_entry<Pair>(name, func, kind, {k1, k2}, barriers, pattern, p0, p1, hooks);
 }
 
 }  // namespace bfuse
@@ -343,5 +510,84 @@ KernelEntry make_fused_entry(const char* name, const void* func, int kind, const
             #K1 "_" #K2 "_fused_bfuse_rt", (const void*)&K1##_##K2##_fused_bfuse_rt, bfuse::kBfuseRt, #K1, #K2, \
             true, -1, 0, 0, bfuse_module_hooks);                                       \
         e.set_plan = &set_plan_##K1##_##K2##_rt;                                                     \
+        return e;                                                                                   \
+    }());
+
+// ---- three and four operators: 3 x n pointers in operator order, names joined as the reference's
+//      emitter joins them (Contexts.cc:56-92) ---------------------------------------------------
+#define BFUSE_PTRS3(N) const void* __restrict__ I##N, const void* __restrict__ F##N, void* __restrict__ O##N
+#define BFUSE_SIDE(N) {I##N, F##N, O##N}
+
+#define BFUSE_BFUSE3_KERNEL(K1, OP1, K2, OP2, K3, OP3, SUFFIX, PATTERN, P0, P1)                      \
+    using grp_##K1##_##K2##_##K3##_bfuse##SUFFIX = bfuse::BfuseGroup<PATTERN, P0, P1, OP1, OP2, OP3>; \
+    extern "C" __global__ __launch_bounds__(grp_##K1##_##K2##_##K3##_bfuse##SUFFIX::THREADS, bfuse::kMinWavesPerEu) \
+    void K1##_##K2##_##K3##_fused_bfuse##SUFFIX(BFUSE_PTRS3(1), BFUSE_PTRS3(2), BFUSE_PTRS3(3))      \
+    {                                                                                               \
+        const bfuse::SidePtrs p[3] = {BFUSE_SIDE(1), BFUSE_SIDE(2), BFUSE_SIDE(3)};                 \
+        bfuse::bfuse_group_body<PATTERN, P0, P1, OP1, OP2, OP3>(p, std::make_integer_sequence<int, 3>{}); \
+    }                                                                                               \
+    static bfuse::Registrar reg_##K1##_##K2##_##K3##_bfuse##SUFFIX(                                  \
+        bfuse::make_group_entry<grp_##K1##_##K2##_##K3##_bfuse##SUFFIX>(                             \
+            #K1 "_" #K2 "_" #K3 "_fused_bfuse" #SUFFIX, (const void*)&K1##_##K2##_##K3##_fused_bfuse##SUFFIX, \
+            bfuse::kBfuse, {#K1, #K2, #K3}, OP1::HAS_BARRIERS || OP2::HAS_BARRIERS || OP3::HAS_BARRIERS, \
+            PATTERN, P0, P1, bfuse_module_hooks));
+
+#define BFUSE_BFUSE4_KERNEL(K1, OP1, K2, OP2, K3, OP3, K4, OP4, SUFFIX, PATTERN, P0, P1)             \
+    using grp_##K1##_##K2##_##K3##_##K4##_bfuse##SUFFIX = bfuse::BfuseGroup<PATTERN, P0, P1, OP1, OP2, OP3, OP4>; \
+    extern "C" __global__ __launch_bounds__(grp_##K1##_##K2##_##K3##_##K4##_bfuse##SUFFIX::THREADS, bfuse::kMinWavesPerEu) \
+    void K1##_##K2##_##K3##_##K4##_fused_bfuse##SUFFIX(BFUSE_PTRS3(1), BFUSE_PTRS3(2), BFUSE_PTRS3(3), BFUSE_PTRS3(4)) \
+    {                                                                                               \
+        const bfuse::SidePtrs p[4] = {BFUSE_SIDE(1), BFUSE_SIDE(2), BFUSE_SIDE(3), BFUSE_SIDE(4)};  \
+        bfuse::bfuse_group_body<PATTERN, P0, P1, OP1, OP2, OP3, OP4>(p, std::make_integer_sequence<int, 4>{}); \
+    }                                                                                               \
+    static bfuse::Registrar reg_##K1##_##K2##_##K3##_##K4##_bfuse##SUFFIX(                           \
+        bfuse::make_group_entry<grp_##K1##_##K2##_##K3##_##K4##_bfuse##SUFFIX>(                      \
+            #K1 "_" #K2 "_" #K3 "_" #K4 "_fused_bfuse" #SUFFIX,                                      \
+            (const void*)&K1##_##K2##_##K3##_##K4##_fused_bfuse##SUFFIX, bfuse::kBfuse, {#K1, #K2, #K3, #K4}, \
+            OP1::HAS_BARRIERS || OP2::HAS_BARRIERS || OP3::HAS_BARRIERS || OP4::HAS_BARRIERS, PATTERN, P0, P1, \
+            bfuse_module_hooks));
+
+#define BFUSE_HFUSE3_KERNEL(K1, OP1, K2, OP2, K3, OP3)                                               \
+    using grp_##K1##_##K2##_##K3##_hfuse = bfuse::HfuseGroup<OP1, OP2, OP3>;                         \
+    extern "C" __global__ __launch_bounds__(grp_##K1##_##K2##_##K3##_hfuse::THREADS, bfuse::kMinWavesPerEu) \
+    void K1##_##K2##_##K3##_fused_hfuse(BFUSE_PTRS3(1), BFUSE_PTRS3(2), BFUSE_PTRS3(3))              \
+    {                                                                                               \
+        const bfuse::SidePtrs p[3] = {BFUSE_SIDE(1), BFUSE_SIDE(2), BFUSE_SIDE(3)};                 \
+        bfuse::hfuse_group_body<OP1, OP2, OP3>(p, std::make_integer_sequence<int, 3>{});            \
+    }                                                                                               \
+    static bfuse::Registrar reg_##K1##_##K2##_##K3##_hfuse(bfuse::make_group_entry<grp_##K1##_##K2##_##K3##_hfuse>( \
+        #K1 "_" #K2 "_" #K3 "_fused_hfuse", (const void*)&K1##_##K2##_##K3##_fused_hfuse, bfuse::kHfuse,  \
+        {#K1, #K2, #K3}, OP1::HAS_BARRIERS || OP2::HAS_BARRIERS || OP3::HAS_BARRIERS, -1, 0, 0, bfuse_module_hooks));
+
+#define BFUSE_HFUSE4_KERNEL(K1, OP1, K2, OP2, K3, OP3, K4, OP4)                                      \
+    using grp_##K1##_##K2##_##K3##_##K4##_hfuse = bfuse::HfuseGroup<OP1, OP2, OP3, OP4>;             \
+    extern "C" __global__ __launch_bounds__(grp_##K1##_##K2##_##K3##_##K4##_hfuse::THREADS, bfuse::kMinWavesPerEu) \
+    void K1##_##K2##_##K3##_##K4##_fused_hfuse(BFUSE_PTRS3(1), BFUSE_PTRS3(2), BFUSE_PTRS3(3), BFUSE_PTRS3(4)) \
+    {                                                                                               \
+        const bfuse::SidePtrs p[4] = {BFUSE_SIDE(1), BFUSE_SIDE(2), BFUSE_SIDE(3), BFUSE_SIDE(4)};  \
+        bfuse::hfuse_group_body<OP1, OP2, OP3, OP4>(p, std::make_integer_sequence<int, 4>{});       \
+    }                                                                                               \
+    static bfuse::Registrar reg_##K1##_##K2##_##K3##_##K4##_hfuse(                                   \
+        bfuse::make_group_entry<grp_##K1##_##K2##_##K3##_##K4##_hfuse>(                              \
+            #K1 "_" #K2 "_" #K3 "_" #K4 "_fused_hfuse", (const void*)&K1##_##K2##_##K3##_##K4##_fused_hfuse, \
+            bfuse::kHfuse, {#K1, #K2, #K3, #K4},                                                     \
+            OP1::HAS_BARRIERS || OP2::HAS_BARRIERS || OP3::HAS_BARRIERS || OP4::HAS_BARRIERS, -1, 0, 0, \
+            bfuse_module_hooks));
+
+// run-time plan over three operators: the plan is the kernel's last argument, as for pairs
+#define BFUSE_BFUSE_RT3_KERNEL(K1, OP1, K2, OP2, K3, OP3)                                            \
+    using grp_##K1##_##K2##_##K3##_bfuse_rt = bfuse::BfuseRtGroup<OP1, OP2, OP3>;                    \
+    extern "C" __global__ __launch_bounds__(grp_##K1##_##K2##_##K3##_bfuse_rt::THREADS, bfuse::kMinWavesPerEu) \
+    void K1##_##K2##_##K3##_fused_bfuse_rt(BFUSE_PTRS3(1), BFUSE_PTRS3(2), BFUSE_PTRS3(3), const bfuse::BlockPlan plan) \
+    {                                                                                               \
+        const bfuse::SidePtrs p[3] = {BFUSE_SIDE(1), BFUSE_SIDE(2), BFUSE_SIDE(3)};                 \
+        bfuse::bfuse_rt_group_body<OP1, OP2, OP3>(plan, p, std::make_integer_sequence<int, 3>{});   \
+    }                                                                                               \
+    static int set_plan_##K1##_##K2##_##K3##_rt(const bfuse::BlockPlan*) { return 0; }               \
+    static bfuse::Registrar reg_##K1##_##K2##_##K3##_bfuse_rt([] {                                   \
+        bfuse::KernelEntry e = bfuse::make_group_entry<grp_##K1##_##K2##_##K3##_bfuse_rt>(           \
+            #K1 "_" #K2 "_" #K3 "_fused_bfuse_rt", (const void*)&K1##_##K2##_##K3##_fused_bfuse_rt, bfuse::kBfuseRt, \
+            {#K1, #K2, #K3}, true, -1, 0, 0, bfuse_module_hooks);                                    \
+        e.set_plan = &set_plan_##K1##_##K2##_##K3##_rt;                                              \
         return e;                                                                                   \
     }());

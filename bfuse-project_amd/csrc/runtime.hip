@@ -63,7 +63,7 @@ struct Side {
 struct State {
     bool inited = false;
     int device = -1;
-    Side side[2];
+    Side side[kMaxKernels];   // the harness functions use the first two; launch lists may use all
 } g;
 
 // 0 for a shape with a dimension below 1 (callers refuse empty tensors)
@@ -176,7 +176,7 @@ int check_launch(const void* func, const unsigned* grid, const unsigned* block, 
     if (!func || !grid || !block) return fail(BFUSE_ERR_ARG, "null launch argument");
     const KernelEntry* e = entry_of(func);
     if (!e) return fail(BFUSE_ERR_ARG, "func is not a kernel of this library");
-    const int ptrs = e->kind == kSingle ? 3 : 6;
+    const int ptrs = e->kind == kSingle ? 3 : 3 * e->n_sides;
     if (ptrs != want_ptrs) return fail(BFUSE_ERR_ARG, "%s takes %d pointers, not %d", e->name.c_str(), ptrs, want_ptrs);
     if (e->kind == kBfuseRt) {
         // persistent workgroups stride over the plan's fused grid: any grid from 1 to that size covers it
@@ -212,16 +212,17 @@ int check_side_fits(const void* func, int idx)
     return BFUSE_OK;
 }
 
-int check_fused_fits(const void* func)
+// `sides` (0-based, one per operator of the fused kernel) or nullptr for sides 0, 1, ...
+int check_fused_fits(const void* func, const int* sides = nullptr)
 {
     const KernelEntry* e = entry_of(func);
     if (!e || e->kind == kSingle) return fail(BFUSE_ERR_ARG, "not a fused kernel");
-    for (int k = 0; k < 2; ++k) {
+    for (int k = 0; k < e->n_sides; ++k) {
         const KernelEntry* sk = nullptr;
         for (const auto& c : registry())
             if (c.kind == kSingle && c.name == e->side[k]) sk = &c;
         if (!sk) return fail(BFUSE_ERR_ARG, "fused kernel %s names unknown side %s", e->name.c_str(), e->side[k].c_str());
-        int rc = check_side_fits(sk->func, k);
+        int rc = check_side_fits(sk->func, sides ? sides[k] : k);
         if (rc) return rc;
     }
     return BFUSE_OK;
@@ -239,14 +240,16 @@ int launch3(const void* func, const unsigned* grid, const unsigned* block, int i
     return BFUSE_OK;
 }
 
-int launch6(const void* func, const unsigned* grid, const unsigned* block, hipStream_t stream,
-            hipEvent_t ev0 = nullptr, hipEvent_t ev1 = nullptr)
+// A fused kernel over n sides (0-based indices, operator order): 3 x n pointers.
+int launch_fused(const void* func, const unsigned* grid, const unsigned* block, int n, const int* sides, hipStream_t stream,
+                 hipEvent_t ev0 = nullptr, hipEvent_t ev1 = nullptr)
 {
-    Side &a = g.side[0], &b = g.side[1];
-    void* args[7] = {&a.buf[0], &a.buf[1], &a.buf[2], &b.buf[0], &b.buf[1], &b.buf[2], nullptr};
-    // a run-time-plan kernel takes its installed plan by value as a seventh argument
+    void* args[3 * kMaxKernels + 1] = {};
+    for (int k = 0; k < n; ++k)
+        for (int i = 0; i < 3; ++i) args[3 * k + i] = &g.side[sides[k]].buf[i];
+    // a run-time-plan kernel takes its installed plan by value as its last argument
     auto it = installed_plans().find(func);
-    if (it != installed_plans().end()) args[6] = &it->second;
+    if (it != installed_plans().end()) args[3 * n] = &it->second;
     bool known = false;
     for (const void* f : g_pending_fused) known = known || f == func;
     if (!known) g_pending_fused.push_back(func);
@@ -255,6 +258,13 @@ int launch6(const void* func, const unsigned* grid, const unsigned* block, hipSt
     else
         HIP_TRY(hipLaunchKernel(func, d3(grid), d3(block), args, 0, stream));
     return BFUSE_OK;
+}
+
+int launch6(const void* func, const unsigned* grid, const unsigned* block, hipStream_t stream,
+            hipEvent_t ev0 = nullptr, hipEvent_t ev1 = nullptr)
+{
+    const int sides[2] = {0, 1};
+    return launch_fused(func, grid, block, 2, sides, stream, ev0, ev1);
 }
 
 // kernels of a loaded code object report give-ups of their side barriers in this device variable
@@ -435,7 +445,7 @@ int bfuse_init(int device)
 
 int bfuse_shutdown(void)
 {
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < kMaxKernels; ++i)
         if (g.side[i].live) {
             int rc = fini_side(i);
             if (rc) return rc;
@@ -580,26 +590,31 @@ int bfuse_set_plan(const void* func, const bfuse_block_plan* plan)
     BlockPlan p;
     memcpy(&p, plan, sizeof(p));
     // The kernel trusts the plan for every index it forms, so it is checked here in full: it must
-    // send the fused block ids one-to-one onto the blocks of the two sides.
-    int side_grid[2] = {0, 0};
-    for (int k = 0; k < 2; ++k)
+    // send the fused block ids one-to-one onto the blocks of the kernel's sides.
+    const int ns = e->n_sides;
+    int side_grid[kMaxKernels] = {};
+    int sum_grid = 0;
+    for (int k = 0; k < ns; ++k) {
         for (const auto& c : registry())
             if (c.kind == kSingle && c.name == e->side[k]) side_grid[k] = (int)c.grid[0];
-    if (p.n_kernels != 2 || p.n_seg < 1 || p.n_seg > kMaxSegments) return fail(BFUSE_ERR_ARG, "plan: bad kernel or segment count");
-    if (p.fused_grid != side_grid[0] + side_grid[1])
-        return fail(BFUSE_ERR_ARG, "plan covers %d blocks, %s has %d + %d", p.fused_grid, e->name.c_str(), side_grid[0], side_grid[1]);
+        sum_grid += side_grid[k];
+    }
+    if (p.n_kernels != ns || p.n_seg < 1 || p.n_seg > kMaxSegments) return fail(BFUSE_ERR_ARG, "plan: bad kernel or segment count");
+    if (p.fused_grid != sum_grid)
+        return fail(BFUSE_ERR_ARG, "plan covers %d blocks, the %d sides of %s have %d", p.fused_grid, ns, e->name.c_str(), sum_grid);
     for (int i = 0; i < p.n_seg; ++i) {
         const Segment& sg = p.seg[i];
         if (sg.period < 1 || sg.n_slot < 1 || sg.n_slot > kMaxKernels || sg.lo < 0 || sg.hi < sg.lo) return fail(BFUSE_ERR_ARG, "plan: malformed segment %d", i);
         for (int j = 0; j < sg.n_slot; ++j)
-            if (sg.slot[j].kern < 0 || sg.slot[j].kern > 1 || sg.slot[j].width < 1 || sg.slot[j].off < 0 || sg.slot[j].base < 0)
+            if (sg.slot[j].kern < 0 || sg.slot[j].kern >= ns || sg.slot[j].width < 1 || sg.slot[j].off < 0 || sg.slot[j].base < 0)
                 return fail(BFUSE_ERR_ARG, "plan: malformed slot %d of segment %d", j, i);
     }
-    std::vector<unsigned char> seen[2] = {std::vector<unsigned char>((size_t)side_grid[0], 0), std::vector<unsigned char>((size_t)side_grid[1], 0)};
+    std::vector<unsigned char> seen[kMaxKernels];
+    for (int k = 0; k < ns; ++k) seen[k].assign((size_t)side_grid[k], 0);
     for (int bid = 0; bid < p.fused_grid; ++bid) {
         int v = -1;
         const int k = map_block(p, bid, &v);
-        if (k < 0 || k > 1 || v < 0 || v >= side_grid[k] || seen[k][(size_t)v])
+        if (k < 0 || k >= ns || v < 0 || v >= side_grid[k] || seen[k][(size_t)v])
             return fail(BFUSE_ERR_ARG, "plan: fused block %d maps to kernel %d block %d (out of range or visited twice)", bid, k, v);
         seen[k][(size_t)v] = 1;
     }
@@ -653,6 +668,8 @@ static void fill_info(const KernelEntry& e, bfuse_kernel_info* o)
     }
     snprintf(o->side[0], sizeof(o->side[0]), "%s", e.side[0].c_str());
     snprintf(o->side[1], sizeof(o->side[1]), "%s", e.side[1].c_str());
+    o->n_sides = e.kind == kSingle ? 1 : e.n_sides;
+    for (int k = 2; k < kMaxKernels; ++k) snprintf(o->side_more[k - 2], sizeof(o->side_more[k - 2]), "%s", e.side[k].c_str());
     o->pattern = e.pattern;
     o->p0 = e.p0;
     o->p1 = e.p1;
@@ -681,7 +698,7 @@ int bfuse_kernel_find(const char* name, bfuse_kernel_info* out)
 // ---- harness ----------------------------------------------------------------------------
 int bfuse_set_elem_bytes(int side, int ib, int fb, int ob)
 {
-    if (side < 1 || side > 2) return fail(BFUSE_ERR_ARG, "side must be 1 or 2");
+    if (side < 1 || side > kMaxKernels) return fail(BFUSE_ERR_ARG, "side must be 1 .. %d", kMaxKernels);
     if (g.side[side - 1].live) return fail(BFUSE_ERR_STATE, "set element sizes before initialize_kernel%d", side);
     const int v[3] = {ib, fb, ob};
     for (int i = 0; i < 3; ++i) {
@@ -695,6 +712,16 @@ int initialize_kernel1(const int* I, const int* F, const int* O) { return init_s
 int initialize_kernel2(const int* I, const int* F, const int* O) { return init_side(1, I, F, O); }
 int finalize_kernel1(void) { return fini_side(0); }
 int finalize_kernel2(void) { return fini_side(1); }
+int bfuse_initialize_side(int side, const int* I, const int* F, const int* O)
+{
+    if (side < 1 || side > kMaxKernels) return fail(BFUSE_ERR_ARG, "side must be 1 .. %d", kMaxKernels);
+    return init_side(side - 1, I, F, O);
+}
+int bfuse_finalize_side(int side)
+{
+    if (side < 1 || side > kMaxKernels) return fail(BFUSE_ERR_ARG, "side must be 1 .. %d", kMaxKernels);
+    return fini_side(side - 1);
+}
 
 static int run_single(int idx, const void* I, const void* F, void* O, const int* Is, const int* Fs, const int* Os,
                       const void* func, const unsigned* grid, const unsigned* block)
@@ -777,7 +804,7 @@ int run_fuse(const void* I1, const void* F1, void* O1, const void* I2, const voi
 // ---- device-resident operation and timing -------------------------------------------------
 int bfuse_upload(int side, const void* I, const void* F)
 {
-    if (side < 1 || side > 2) return fail(BFUSE_ERR_ARG, "side must be 1 or 2");
+    if (side < 1 || side > kMaxKernels) return fail(BFUSE_ERR_ARG, "side must be 1 .. %d", kMaxKernels);
     Side& s = g.side[side - 1];
     if (!s.live) return fail(BFUSE_ERR_STATE, "kernel%d is not initialized", side);
     if (!I || !F) return fail(BFUSE_ERR_ARG, "null host buffer");
@@ -788,7 +815,7 @@ int bfuse_upload(int side, const void* I, const void* F)
 
 int bfuse_zero_output(int side)
 {
-    if (side < 1 || side > 2) return fail(BFUSE_ERR_ARG, "side must be 1 or 2");
+    if (side < 1 || side > kMaxKernels) return fail(BFUSE_ERR_ARG, "side must be 1 .. %d", kMaxKernels);
     Side& s = g.side[side - 1];
     if (!s.live) return fail(BFUSE_ERR_STATE, "kernel%d is not initialized", side);
     HIP_TRY(hipMemset(s.buf[2], 0, s.bytes[2]));
@@ -797,7 +824,7 @@ int bfuse_zero_output(int side)
 
 int bfuse_download(int side, void* O)
 {
-    if (side < 1 || side > 2) return fail(BFUSE_ERR_ARG, "side must be 1 or 2");
+    if (side < 1 || side > kMaxKernels) return fail(BFUSE_ERR_ARG, "side must be 1 .. %d", kMaxKernels);
     Side& s = g.side[side - 1];
     if (!s.live) return fail(BFUSE_ERR_STATE, "kernel%d is not initialized", side);
     if (!O) return fail(BFUSE_ERR_ARG, "null host buffer");
@@ -888,6 +915,93 @@ int bfuse_time_batched(int mode, const void* fa, const unsigned* ga, const unsig
     return BFUSE_OK;
 }
 
+// ---- launch lists: any registered kernel over any sides -------------------------------------
+static int validate_list(int n, const bfuse_launch_desc* l)
+{
+    if (!g.inited) return fail(BFUSE_ERR_STATE, "bfuse_init has not been called");
+    if (n < 1 || n > 16 || !l) return fail(BFUSE_ERR_ARG, "a launch list holds 1 .. 16 launches");
+    for (int j = 0; j < n; ++j) {
+        const bfuse_launch_desc& d = l[j];
+        const KernelEntry* e = entry_of(d.func);
+        if (!e) return fail(BFUSE_ERR_ARG, "launch %d: func is not a kernel of this library", j);
+        const int want = e->kind == kSingle ? 1 : e->n_sides;
+        if (d.n_sides != want) return fail(BFUSE_ERR_ARG, "launch %d: %s runs over %d sides, not %d", j, e->name.c_str(), want, d.n_sides);
+        int rc;
+        if ((rc = check_launch(d.func, d.grid, d.block, 3 * want))) return rc;
+        int sides0[kMaxKernels];
+        for (int k = 0; k < want; ++k) {
+            if (d.sides[k] < 1 || d.sides[k] > kMaxKernels) return fail(BFUSE_ERR_ARG, "launch %d: side must be 1 .. %d", j, kMaxKernels);
+            for (int m = 0; m < k; ++m)
+                if (d.sides[m] == d.sides[k]) return fail(BFUSE_ERR_ARG, "launch %d: side %d named twice", j, d.sides[k]);
+            sides0[k] = d.sides[k] - 1;
+        }
+        if ((rc = e->kind == kSingle ? check_side_fits(d.func, sides0[0]) : check_fused_fits(d.func, sides0))) return rc;
+    }
+    return BFUSE_OK;
+}
+
+static int enqueue_list(int n, const bfuse_launch_desc* l, hipEvent_t* ev /* 2 per launch or nullptr */)
+{
+    for (int j = 0; j < n; ++j) {
+        const bfuse_launch_desc& d = l[j];
+        int sides0[kMaxKernels];
+        for (int k = 0; k < d.n_sides; ++k) sides0[k] = d.sides[k] - 1;
+        const KernelEntry* e = entry_of(d.func);
+        hipEvent_t e0 = ev ? ev[2 * j] : nullptr, e1 = ev ? ev[2 * j + 1] : nullptr;
+        int rc = e->kind == kSingle ? launch3(d.func, d.grid, d.block, sides0[0], nullptr, e0, e1)
+                                    : launch_fused(d.func, d.grid, d.block, d.n_sides, sides0, nullptr, e0, e1);
+        if (rc) return rc;
+    }
+    return BFUSE_OK;
+}
+
+int bfuse_launch_list(int n, const bfuse_launch_desc* launches)
+{
+    int rc = validate_list(n, launches);
+    if (rc) return rc;
+    return enqueue_list(n, launches, nullptr);
+}
+
+int bfuse_time_list(int n, const bfuse_launch_desc* launches, int warmup, int reps, float* us_each, float* us_queued)
+{
+    int rc = validate_list(n, launches);
+    if (rc) return rc;
+    if (warmup < 0 || reps < 1 || reps > 100000 || (!us_each && !us_queued)) return fail(BFUSE_ERR_ARG, "bad repetition count or no output");
+    for (int i = 0; i < warmup; ++i)
+        if ((rc = enqueue_list(n, launches, nullptr))) return rc;
+    HIP_TRY(hipDeviceSynchronize());
+    if (us_each) {
+        EventList evl((size_t)reps * 2 * n);
+        for (auto& e : evl.v) HIP_TRY(hipEventCreate(&e));
+        for (int r = 0; r < reps; ++r)
+            if ((rc = enqueue_list(n, launches, &evl.v[(size_t)r * 2 * n]))) return rc;
+        if ((rc = sync_and_check())) return rc;
+        for (int j = 0; j < n; ++j) {
+            double sum = 0.0;
+            for (int r = 0; r < reps; ++r) {
+                float ms = 0.f;
+                HIP_TRY(hipEventElapsedTime(&ms, evl.v[((size_t)r * n + j) * 2], evl.v[((size_t)r * n + j) * 2 + 1]));
+                sum += ms;
+            }
+            us_each[j] = (float)(sum * 1000.0 / reps);
+        }
+    }
+    if (us_queued) {
+        EventList evl(2);
+        HIP_TRY(hipEventCreate(&evl.v[0]));
+        HIP_TRY(hipEventCreate(&evl.v[1]));
+        HIP_TRY(hipEventRecord(evl.v[0], nullptr));
+        for (int r = 0; r < reps; ++r)
+            if ((rc = enqueue_list(n, launches, nullptr))) return rc;
+        HIP_TRY(hipEventRecord(evl.v[1], nullptr));
+        if ((rc = sync_and_check())) return rc;
+        float ms = 0.f;
+        HIP_TRY(hipEventElapsedTime(&ms, evl.v[0], evl.v[1]));
+        *us_queued = ms * 1000.f / (float)reps;
+    }
+    return BFUSE_OK;
+}
+
 // ---- kernels from a code object -------------------------------------------------------------
 
 int bfuse_module_load(const char* path, int* module_id)
@@ -928,8 +1042,8 @@ int bfuse_module_launch(int id, const char* name, const unsigned* grid, const un
     auto& ms = modules();
     if (id < 0 || id >= (int)ms.size() || !ms[id]) return fail(BFUSE_ERR_ARG, "unknown module %d", id);
     if (!name || !grid || !block) return fail(BFUSE_ERR_ARG, "null argument");
-    if (n_ptrs != 3 && n_ptrs != 6) return fail(BFUSE_ERR_ARG, "n_ptrs must be 3 or 6");
-    if (n_ptrs == 3 && side != 1 && side != 2) return fail(BFUSE_ERR_ARG, "side must be 1 or 2");
+    if (n_ptrs < 3 || n_ptrs > 3 * kMaxKernels || n_ptrs % 3) return fail(BFUSE_ERR_ARG, "n_ptrs must be 3, 6, ... %d", 3 * kMaxKernels);
+    if (n_ptrs == 3 && (side < 1 || side > kMaxKernels)) return fail(BFUSE_ERR_ARG, "side must be 1 .. %d", kMaxKernels);
     for (int i = 0; i < 3; ++i)
         if (grid[i] == 0 || block[i] == 0) return fail(BFUSE_ERR_ARG, "empty launch shape");
     if ((size_t)block[0] * block[1] * block[2] > 1024) return fail(BFUSE_ERR_ARG, "more than 1024 threads per workgroup");
@@ -939,19 +1053,18 @@ int bfuse_module_launch(int id, const char* name, const unsigned* grid, const un
         (void)hipGetLastError();
         return fail(BFUSE_ERR_ARG, "kernel '%s' is not in module %d: %s", name, id, hipGetErrorString(st));
     }
-    void* ptrs[6];
+    void* ptrs[3 * kMaxKernels];
     if (n_ptrs == 3) {
         Side& s = g.side[side - 1];
         if (!s.live) return fail(BFUSE_ERR_STATE, "kernel%d is not initialized", side);
         for (int i = 0; i < 3; ++i) ptrs[i] = s.buf[i];
     } else {
-        if (!g.side[0].live || !g.side[1].live) return fail(BFUSE_ERR_STATE, "both sides must be initialized");
-        for (int i = 0; i < 3; ++i) {
-            ptrs[i] = g.side[0].buf[i];
-            ptrs[3 + i] = g.side[1].buf[i];
+        for (int k = 0; k < n_ptrs / 3; ++k) {
+            if (!g.side[k].live) return fail(BFUSE_ERR_STATE, "sides 1 .. %d must be initialized", n_ptrs / 3);
+            for (int i = 0; i < 3; ++i) ptrs[3 * k + i] = g.side[k].buf[i];
         }
     }
-    void* args[6];
+    void* args[3 * kMaxKernels];
     for (int i = 0; i < n_ptrs; ++i) args[i] = &ptrs[i];
     EventList evl(2);
     hipEvent_t &e0 = evl.v[0], &e1 = evl.v[1];

@@ -29,12 +29,15 @@ class KernelHandle:
     pattern: int
     p0: int
     p1: int
+    n_sides: int = 2          # kernels a fused kernel runs (1 for a standalone kernel)
 
 
 def _handle(ci: "_lib.KernelInfoC") -> KernelHandle:
     return KernelHandle(ci.name.decode(), ci.func, ci.kind, tuple(ci.grid), tuple(ci.block), bool(ci.has_barriers),
                         ci.regs, ci.lds_bytes, tuple(tuple(s) for s in ci.shape), tuple(ci.elem_bytes),
-                        (ci.side[0].value.decode(), ci.side[1].value.decode()), ci.pattern, ci.p0, ci.p1)
+                        tuple([ci.side[0].value.decode(), ci.side[1].value.decode()] +
+                              [ci.side_more[i].value.decode() for i in range(max(0, ci.n_sides - 2))]),
+                        ci.pattern, ci.p0, ci.p1, ci.n_sides)
 
 
 def kernel_info(name: str) -> KernelHandle:
@@ -202,6 +205,96 @@ class Operation:
         us = C.c_float()
         _lib.check(self.l.bfuse_time_batched(MODES[mode], *self._mode_args(mode, fused), warmup, reps, C.byref(us)))
         return us.value
+
+
+class GroupOperation:
+    """Two to four sides for fusions of more than two kernels (the reference's fuser takes a list of
+    kernels, horizontal-fuser/src/Algorithms.cc:23-35; its harness is two-sided).  Side i holds the
+    buffers of standalone kernel names[i]; launches are lists of (kernel, sides)."""
+
+    def __init__(self, names: Sequence[str], device: int = 0):
+        self.l = _lib.lib()
+        _lib.check(self.l.bfuse_init(device))
+        if not 2 <= len(names) <= _lib.MAXK:
+            raise ValueError(f"a group has 2 .. {_lib.MAXK} kernels")
+        self.k = [kernel_info(n) for n in names]
+        self.live_sides = []
+        try:
+            for side, k in enumerate(self.k, 1):
+                if k.kind != 0:
+                    raise ValueError(f"{k.name} is a fused kernel; sides must be standalone kernels")
+                _lib.check(self.l.bfuse_set_elem_bytes(side, *k.elem_bytes))
+                _lib.check(self.l.bfuse_initialize_side(side, *[_i4(s) for s in k.shapes]))
+                self.live_sides.append(side)
+        except Exception:
+            self.close()
+            raise
+
+    def close(self):
+        while self.live_sides:
+            _lib.check(self.l.bfuse_finalize_side(self.live_sides.pop()))
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def fused(self, kind: str, suffix: str = "") -> KernelHandle:
+        return kernel_info("_".join(k.name for k in self.k) + f"_fused_{kind}{suffix}")
+
+    def set_plan(self, fused: KernelHandle, plan, workgroups: Optional[int] = None) -> KernelHandle:
+        _lib.check(self.l.bfuse_set_plan(fused.func, C.byref(plan.c)))
+        n = plan.fused_grid if workgroups is None else min(int(workgroups), plan.fused_grid)
+        return replace(fused, grid=(n, 1, 1))
+
+    def upload(self, side: int, I, F):
+        k = self.k[side]
+        a = [np.ascontiguousarray(x, dtype=_DT[k.elem_bytes[i]]) for i, x in enumerate((I, F))]
+        for i in range(2):
+            if a[i].size != int(np.prod(k.shapes[i])):
+                raise ValueError(f"{k.name}: tensor {i} has {a[i].size} elements, kernel expects {int(np.prod(k.shapes[i]))}")
+        _lib.check(self.l.bfuse_upload(side + 1, a[0].ctypes.data, a[1].ctypes.data))
+
+    def zero_outputs(self):
+        for side in self.live_sides:
+            _lib.check(self.l.bfuse_zero_output(side))
+
+    def download(self, side: int) -> np.ndarray:
+        k = self.k[side]
+        O = np.empty(tuple(k.shapes[2]), _DT[k.elem_bytes[2]])
+        _lib.check(self.l.bfuse_download(side + 1, O.ctypes.data))
+        return O
+
+    def _descs(self, launches):
+        """launches: [(KernelHandle, (side, ...)), ...] with 0-based sides; a standalone kernel takes one."""
+        arr = (_lib.LaunchDescC * len(launches))()
+        for d, (k, sides) in zip(arr, launches):
+            d.func = k.func
+            d.grid[:] = k.grid
+            d.block[:] = k.block
+            d.n_sides = len(sides)
+            for i, sd in enumerate(sides):
+                d.sides[i] = sd + 1
+        return arr
+
+    def unfused(self):
+        return [(k, (i,)) for i, k in enumerate(self.k)]
+
+    def launch(self, launches):
+        arr = self._descs(launches)
+        _lib.check(self.l.bfuse_launch_list(len(arr), arr))
+
+    def synchronize(self):
+        _lib.check(self.l.bfuse_synchronize())
+
+    def time(self, launches, warmup: int = 3, reps: int = 30):
+        """(mean GPU-side microseconds of each launch, wall-clock microseconds per round when queued)."""
+        arr = self._descs(launches)
+        each = np.zeros(len(arr), np.float32)
+        queued = C.c_float()
+        _lib.check(self.l.bfuse_time_list(len(arr), arr, warmup, reps, each.ctypes.data_as(C.POINTER(C.c_float)), C.byref(queued)))
+        return each, queued.value
 
 
 class GenericOperation:

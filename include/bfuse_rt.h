@@ -128,7 +128,7 @@ int bfuse_set_sync_spin_limit(const void* func, unsigned polls);
  * (test-utils/test-suite-files/macro_h.py:79-198) and of kernels.yaml / {b,h}fuse_kernels.yaml
  * (horizontal-fuser/include/fuse/Utils.h:70-112).
  * ---------------------------------------------------------------------------------------- */
-enum { BFUSE_KIND_SINGLE = 0, BFUSE_KIND_BFUSE = 1, BFUSE_KIND_HFUSE = 2 };
+enum { BFUSE_KIND_SINGLE = 0, BFUSE_KIND_BFUSE = 1, BFUSE_KIND_HFUSE = 2, BFUSE_KIND_BFUSE_RT = 3 /* block fusion, plan set at run time */ };
 
 typedef struct {
     char name[128];          /* KernelName; fused: <K1>_<K2>_fused_{bfuse,hfuse} (Contexts.cc:56-92) */
@@ -140,8 +140,10 @@ typedef struct {
     int lds_bytes;           /* static LDS of the kernel (-1 without a GPU) */
     int shape[3][4];         /* single kernels: I, F, O shapes, padded with 1s */
     int elem_bytes[3];
-    char side[2][64];        /* fused kernels: the two standalone kernels */
+    char side[2][64];        /* fused kernels: the first two standalone kernels */
     int pattern, p0, p1;     /* bfuse kernels: dispatch pattern */
+    int n_sides;             /* 1 for a standalone kernel; fused: how many kernels it runs (3 pointers each, in order) */
+    char side_more[BFUSE_MAX_KERNELS - 2][64];   /* fused kernels of more than two: the third, fourth standalone kernel */
 } bfuse_kernel_info;
 
 int bfuse_kernel_count(void);
@@ -192,7 +194,7 @@ int run_fuse(const void* I1, const void* F1, void* O1, const void* I2, const voi
  * (scripts/profile_test_suite.py:10-11,106-109; scripts/analyze_test_suite.py:103-161);
  * these entry points keep the operands in HBM and return those durations directly.
  * ---------------------------------------------------------------------------------------- */
-int bfuse_upload(int side, const void* I, const void* F);   /* side 1 or 2 */
+int bfuse_upload(int side, const void* I, const void* F);   /* side 1 .. BFUSE_MAX_KERNELS */
 int bfuse_zero_output(int side);
 int bfuse_download(int side, void* O);
 int bfuse_synchronize(void);
@@ -226,6 +228,32 @@ int bfuse_time_batched(int mode, const void* func_a, const unsigned* grid_a, con
                        int reps, float* us_per_launch);
 
 /* ------------------------------------------------------------------------------------------
+ * More than two kernels.  The reference's harness is two-sided (operation_h.py:9-27) while its
+ * fuser takes a list of kernels of any length (horizontal-fuser/src/Algorithms.cc:23-35,540-566;
+ * the fused kernel's parameters are the kernels' parameter lists one after the other,
+ * Matchers.cc:523-602).  Sides 3 .. BFUSE_MAX_KERNELS are set up with the generic form of
+ * initialize_kernelN / finalize_kernelN, and a launch list runs any registered kernels over any
+ * sides: a standalone kernel over one side, a fused kernel over as many sides as it has kernels
+ * (bfuse_kernel_info.n_sides), in the order of its pointers.
+ * ---------------------------------------------------------------------------------------- */
+int bfuse_initialize_side(int side, const int* I_shape, const int* F_shape, const int* O_shape);
+int bfuse_finalize_side(int side);
+
+typedef struct {
+    const void* func;                 /* registry handle */
+    unsigned grid[3], block[3];       /* must be the kernel's own launch shape (bfuse_kernel_info) */
+    int n_sides;                      /* must equal the kernel's n_sides */
+    int sides[BFUSE_MAX_KERNELS];     /* 1-based, distinct: which resident buffers each of its kernels runs over */
+} bfuse_launch_desc;
+
+/* The launches in order on the default stream, asynchronously (no copies, no host sync). */
+int bfuse_launch_list(int n, const bfuse_launch_desc* launches);
+/* `warmup` untimed rounds, then two measurements of `reps` rounds each (either output may be NULL):
+ * us_each[j] = mean GPU-side duration of launch j (its own start and end timestamps);
+ * *us_queued = wall clock per round with all rounds enqueued back to back. */
+int bfuse_time_list(int n, const bfuse_launch_desc* launches, int warmup, int reps, float* us_each, float* us_queued);
+
+/* ------------------------------------------------------------------------------------------
  * Kernels from a code object: what the horizontal-fuser front end emits (one fused HIP kernel
  * per fusion, compiled with `hipcc --genco`), or any kernel with the reference's three- /
  * six-pointer ABI (macro_h.py:182-198).  Launched over the same resident buffers as the
@@ -234,7 +262,7 @@ int bfuse_time_batched(int mode, const void* func_a, const unsigned* grid_a, con
  * ---------------------------------------------------------------------------------------- */
 int bfuse_module_load(const char* code_object_path, int* module_id);
 int bfuse_module_unload(int module_id);
-/* n_ptrs = 3: launch `kernel_name` over side `side` (1 or 2); n_ptrs = 6: over both sides.
+/* n_ptrs = 3: launch `kernel_name` over side `side`; n_ptrs = 6, 9, 12: over sides 1 .. n_ptrs / 3.
  * Asynchronous on the default stream; if us_out is not NULL the call synchronises and returns
  * the kernel's GPU-side duration in microseconds. */
 int bfuse_module_launch(int module_id, const char* kernel_name, const unsigned* gridDim, const unsigned* blockDim,
