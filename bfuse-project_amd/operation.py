@@ -298,25 +298,33 @@ class GroupOperation:
 
 
 class GenericOperation:
-    """Two sides with caller-given shapes, for kernels that come from a code object (the
-    front end's output) rather than from the library's registry."""
+    """Two to four sides with caller-given (I, F, O) shapes, for kernels that come from a code object
+    (the front end's output) rather than from the library's registry."""
 
-    def __init__(self, shapes1, shapes2, device: int = 0):
+    def __init__(self, *shapes, device: int = 0):
         self.l = _lib.lib()
         _lib.check(self.l.bfuse_init(device))
-        for side in (1, 2):
-            _lib.check(self.l.bfuse_set_elem_bytes(side, 4, 4, 4))
-        self.shapes = [[_i4(s) for s in shapes1], [_i4(s) for s in shapes2]]
-        self.nelem = [[int(np.prod(s)) for s in shapes1], [int(np.prod(s)) for s in shapes2]]
-        _lib.check(self.l.initialize_kernel1(*self.shapes[0]))
-        _lib.check(self.l.initialize_kernel2(*self.shapes[1]))
+        if not 2 <= len(shapes) <= _lib.MAXK:
+            raise ValueError(f"2 .. {_lib.MAXK} sides")
+        self.shapes = [[_i4(s) for s in sh] for sh in shapes]
+        self.nelem = [[int(np.prod(s)) for s in sh] for sh in shapes]
         self.modules = []
+        self.live_sides = []
+        try:
+            for side in range(1, len(shapes) + 1):
+                _lib.check(self.l.bfuse_set_elem_bytes(side, 4, 4, 4))
+                _lib.check(self.l.bfuse_initialize_side(side, *self.shapes[side - 1]))
+                self.live_sides.append(side)
+        except Exception:
+            self.close()
+            raise
 
     def close(self):
         for m in self.modules:
             self.l.bfuse_module_unload(m)
-        _lib.check(self.l.finalize_kernel1())
-        _lib.check(self.l.finalize_kernel2())
+        self.modules = []
+        while self.live_sides:
+            _lib.check(self.l.bfuse_finalize_side(self.live_sides.pop()))
 
     def __enter__(self):
         return self
@@ -336,8 +344,8 @@ class GenericOperation:
         _lib.check(self.l.bfuse_upload(side + 1, I.ctypes.data, F.ctypes.data))
 
     def zero_outputs(self):
-        _lib.check(self.l.bfuse_zero_output(1))
-        _lib.check(self.l.bfuse_zero_output(2))
+        for side in self.live_sides:
+            _lib.check(self.l.bfuse_zero_output(side))
 
     def download(self, side: int) -> np.ndarray:
         O = np.empty(self.nelem[side][2], np.float32)

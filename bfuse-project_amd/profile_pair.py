@@ -7,12 +7,14 @@
 With --copy-probe a 64 MiB -> 64 MiB copy kernel is launched first (in a separate operation), so
 that the same counter can be read for a kernel whose traffic is known.
 Order of launches per repetition: kernel1, kernel2 (back to back on one stream), fused.
+With --group NAME the kernels of a fusion of more than two (workloads.GROUPS) are launched instead:
+its standalone kernels back to back, then the fused kernel.
 """
 import argparse
 import numpy as np
 
 import bfuse_project_amd as bf
-from bfuse_project_amd.workloads import HEADLINE, PAIRS
+from bfuse_project_amd.workloads import GROUPS, HEADLINE, PAIRS
 
 
 def main():
@@ -21,6 +23,7 @@ def main():
     ap.add_argument("--reps", type=int, default=20)
     ap.add_argument("--fusion", default="", help="kind[:suffix][@k1,k2]; default: the pair's headline fusion")
     ap.add_argument("--copy-probe", action="store_true")
+    ap.add_argument("--group", default="", help="a fusion of more than two kernels (workloads.GROUPS) instead of a pair")
     args = ap.parse_args()
     if args.copy_probe:
         with bf.Operation("copy_f32_16777216", "bias_relu_4096") as op:
@@ -28,6 +31,18 @@ def main():
             for _ in range(args.reps):
                 op.launch("kernel1")
             op.synchronize()
+    if args.group:
+        names, kind, suffixes, inputs = GROUPS[args.group]
+        with bf.GroupOperation(names) as op:
+            for i, (I, F) in enumerate(inputs()):
+                op.upload(i, I, F)
+            fused = op.fused(kind, suffixes[0])
+            for _ in range(args.reps):
+                op.launch(op.unfused())
+                op.launch([(fused, tuple(range(len(names))))])
+            op.synchronize()
+        print(f"launched {args.reps} x [{', '.join(names)}, {fused.name}]")
+        return
     pair = PAIRS[args.pair]
     k1, k2, kind, suffix = HEADLINE[args.pair]
     if args.fusion:

@@ -138,6 +138,21 @@ PAIRS: Dict[int, Pair] = {
 }
 
 
+def _qkv_ln_softmax_inputs():
+    I1, F1, I2, F2 = _pair2_inputs()
+    I3, F3, _, _ = _pair4_inputs()
+    return [(I1, F1), (I2, F2), (I3, F3)]
+
+
+# Fusions of more than two kernels (the reference's fuser takes a list of any length,
+# horizontal-fuser/src/Algorithms.cc:23-35): name -> (standalone kernels, kind, suffixes built, inputs).
+# One full-size group: the fp32 QKV projection, the LayerNorm and the causal softmax of pairs 2 and 4.
+GROUPS = {
+    "qkv_ln_softmax": (("gemm_f32_512x768x2304", "layernorm_512x768", "softmax_causal_12x512x512"), "bfuse",
+                       ("_c256", "_r"), _qkv_ln_softmax_inputs),
+}
+
+
 def fusions(pair: Pair):
     """Every built fusion of a pair, grouped by the two standalone kernels it fuses:
     {(k1, k2): [(kind, suffix), ...]}."""

@@ -49,33 +49,42 @@ PAIRS = [("mm_tiled", "row_scale"), ("mm_tiled", "ew_max")]
 
 @pytest.mark.parametrize("k1,k2", PAIRS)
 def test_emitted_kernels_match_unfused(k1, k2):
+    _emitted_match_unfused((k1, k2), VARIANTS)
+
+
+def test_emitted_kernels_of_three_match_unfused():
+    _emitted_match_unfused(("mm_tiled", "row_scale", "ew_max"), [("zigzag3", "bfuse"), ("chunk8_3", "bfuse"), ("hfuse3", "hfuse")])
+
+
+def _emitted_match_unfused(names, variants):
     kmap = config.load_kernels_yaml(os.path.join(os.path.dirname(BUILD), "kernels.yaml"))
+    n = len(names)
     ins = []
-    for side, k in enumerate((k1, k2)):
+    for side, k in enumerate(names):
         n_i, n_f = int(np.prod(SHAPES[k][0])), int(np.prod(SHAPES[k][1]))
         ins.append((fill_uniform(11 + side, n_i, -1.0, 1.0), fill_uniform(23 + side, n_f, -1.0, 1.0)))
-    with GenericOperation(SHAPES[k1], SHAPES[k2]) as op:
-        for side in (0, 1):
+    with GenericOperation(*[SHAPES[k] for k in names]) as op:
+        for side in range(n):
             op.upload(side, *ins[side])
         unf = op.load(need(os.path.join(BUILD, "zigzag", "kernels.hsaco")))
         op.zero_outputs()
-        for side, k in enumerate((k1, k2)):
+        for side, k in enumerate(names):
             op.launch(unf, k, kmap[k].GridDim, kmap[k].BlockDim, 3, side)
-        base = [op.download(0), op.download(1)]
-        for side, k in enumerate((k1, k2)):
+        base = [op.download(side) for side in range(n)]
+        for side, k in enumerate(names):
             ref = numpy_ref(k, *ins[side])
             if k == "mm_tiled":
                 np.testing.assert_allclose(base[side], ref, rtol=0, atol=1e-5 * np.sqrt(np.mean(ref ** 2)) * 8)
             else:
                 assert np.array_equal(base[side], ref), k
-        for folder, kind in VARIANTS:
+        for folder, kind in variants:
             fused = config.load_kernels_yaml(need(os.path.join(BUILD, folder, f"{kind}_kernels.yaml")))
-            name = f"{k1}_{k2}_fused_{kind}"
-            mod = op.load(need(os.path.join(BUILD, folder, f"{k1}_{k2}_{kind}.hsaco")))
+            name = "_".join(names) + f"_fused_{kind}"
+            mod = op.load(need(os.path.join(BUILD, folder, "_".join(names) + f"_{kind}.hsaco")))
             op.zero_outputs()
-            us = op.launch(mod, name, fused[name].GridDim, fused[name].BlockDim, 6)
+            us = op.launch(mod, name, fused[name].GridDim, fused[name].BlockDim, 3 * n)
             assert us > 0
-            for side in (0, 1):
+            for side in range(n):
                 got = op.download(side)
                 assert np.array_equal(got.view(np.uint32), base[side].view(np.uint32)), (folder, name, side)
 

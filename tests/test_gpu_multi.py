@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 
 import bfuse_project_amd as bf
-from bfuse_project_amd.workloads import PAIRS
+from bfuse_project_amd.workloads import GROUPS
 from tests import oracle_cases
 from tests.test_gpu_small import _cases, _check
 from tests.test_group_host import GROUPS
@@ -112,9 +112,8 @@ def test_launch_lists_check_their_arguments():
 
 
 def test_full_size_three_kernels_bit_exact_close_to_cpu_and_timed():
-    names = ("gemm_f32_512x768x2304", "layernorm_512x768", "softmax_causal_12x512x512")
-    I1, F1, I2, F2 = PAIRS[2].inputs()
-    I3, F3, _, _ = PAIRS[4].inputs()
+    names, _, _, inputs = GROUPS["qkv_ln_softmax"]
+    (I1, F1), (I2, F2), (I3, F3) = inputs()
     E1, E2 = oracle_cases.expected(2, I1, F1, I2, F2)
     from oracle import oracle as orf
     E3 = orf.softmax_causal(np.asarray(I3).reshape(12, 512, 512))
