@@ -31,6 +31,8 @@ Per pair:
                     `traffic` is HBM bytes per launch from the rocprofv3 --pmc summary named in
                     `traffic_source` (not measured by this run)
 Top level only:
+  groups            fusions of more than two kernels (one: the fp32 QKV GEMM, LayerNorm and causal softmax
+                    as one block-fused kernel) against their standalone kernels queued back to back
   cpu_baseline      the OpenMP CPU reference (oracle/) timed on this host's cores
   hbm_copy_GBps     what the library's 64 MiB -> 64 MiB copy kernel reaches in this run (a measured
                     ceiling beside the nominal 8000)
@@ -256,6 +258,30 @@ def measure(number, K, W, spec):
     return res, dev, inputs
 
 
+def measure_group(name, K, W):
+    """A fusion of more than two kernels (workloads.GROUPS): the fused kernel against its standalone
+    kernels queued back to back, outputs compared byte for byte in the same run."""
+    import bfuse_project_amd as bf
+    from bfuse_project_amd import workloads as wl
+    names, kind, suffixes, inputs = wl.GROUPS[name]
+    with bf.GroupOperation(names) as op:
+        for i, (I, F) in enumerate(inputs()):
+            op.upload(i, I, F)
+        op.zero_outputs()
+        op.launch(op.unfused())
+        want = [op.download(i) for i in range(len(names))]
+        fused = op.fused(kind, suffixes[0])
+        op.zero_outputs()
+        op.launch([(fused, tuple(range(len(names))))])
+        exact = all(np.array_equal(op.download(i).view(np.uint8), want[i].view(np.uint8)) for i in range(len(names)))
+        each_u, queued_u = op.time(op.unfused(), warmup=W, reps=K)
+        each_f, queued_f = op.time([(fused, tuple(range(len(names))))], warmup=W, reps=K)
+    return {"kernels": list(names), "fused_kernel": fused.name, "fused_us": round(float(each_f[0]), 3),
+            "kernel_us": [round(float(x), 3) for x in each_u], "batched_fused_us": round(queued_f, 3),
+            "batched_back_to_back_us": round(queued_u, 3), "batched_fused_over_back_to_back": round(queued_f / queued_u, 4),
+            "bit_exact_vs_unfused": bool(exact)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -303,6 +329,10 @@ def main():
         "hbm_copy_GBps": round(hbm_copy_rate(), 1),
         "pairs": pairs,
     }
+    if not args.pair:
+        from bfuse_project_amd.workloads import GROUPS
+        out["groups"] = {g: measure_group(g, K, W) for g in GROUPS}
+        out["bit_exact_vs_unfused"] = out["bit_exact_vs_unfused"] and all(g["bit_exact_vs_unfused"] for g in out["groups"].values())
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(top, *top_inputs)
     print(json.dumps(out))

@@ -41,11 +41,15 @@ BFUSE_HFUSE3_KERNEL(conv3x3_f32_32x12x12_32, ConvS2, gemm_gelu_f32_96x128x192, G
 BFUSE_HFUSE4_KERNEL(conv3x3_f32_32x12x12_32, ConvS2, gemm_f32_128x160x192_d, GemmS5, layernorm_8x256, LayerNormS, bias_relu_4096, BiasReluS)
 
 // Full size: QKV projection 512x768x2304 (256 tiles, MFMA-bound), LayerNorm 512x768 and causal
-// softmax 12x512x512 (memory-bound), the three standalone kernels of pairs 2 and 4.
-using GemmQkv = GemmF32Dma<512, 2304, 768, 32, 144, 4>;
+// softmax 12x512x512 (memory-bound), the kernels of pairs 2 and 4.  The GEMM runs here with a ring
+// of two stages: every workgroup of a block-fused kernel is charged the largest side's LDS, and
+// with 48 KB instead of 72 three workgroups fit a CU instead of two -- the GEMM alone is as fast
+// (16.0 us either way), the fused kernel 19.0 instead of 20.6 us.
+using GemmQkvS2 = GemmF32Dma<512, 2304, 768, 32, 144, 4, kEpiNone, 2>;
 using LnBert = LayerNorm<512, 768, 1, 1>;
 using Softmax4 = SoftmaxCausal<12, 512, 4, 1>;
+BFUSE_KERNEL(gemm_f32_512x768x2304_s2, GemmQkvS2, ({{512, 768, 1, 1}, 4}), ({{768, 2304, 1, 1}, 4}), ({{512, 2304, 1, 1}, 4}))
 // GEMM tiles first (one per CU), then the two memory-bound grids in their shadow
-BFUSE_BFUSE3_KERNEL(gemm_f32_512x768x2304, GemmQkv, layernorm_512x768, LnBert, softmax_causal_12x512x512, Softmax4, _r, bfuse::kRanges, 0, 0)
-BFUSE_BFUSE3_KERNEL(gemm_f32_512x768x2304, GemmQkv, layernorm_512x768, LnBert, softmax_causal_12x512x512, Softmax4, _c256, bfuse::kChunked, 256, 1)
-BFUSE_BFUSE_RT3_KERNEL(gemm_f32_512x768x2304, GemmQkv, layernorm_512x768, LnBert, softmax_causal_12x512x512, Softmax4)
+BFUSE_BFUSE3_KERNEL(gemm_f32_512x768x2304_s2, GemmQkvS2, layernorm_512x768, LnBert, softmax_causal_12x512x512, Softmax4, _c256, bfuse::kChunked, 256, 1)
+BFUSE_BFUSE3_KERNEL(gemm_f32_512x768x2304_s2, GemmQkvS2, layernorm_512x768, LnBert, softmax_causal_12x512x512, Softmax4, _r, bfuse::kRanges, 0, 0)
+BFUSE_BFUSE_RT3_KERNEL(gemm_f32_512x768x2304_s2, GemmQkvS2, layernorm_512x768, LnBert, softmax_causal_12x512x512, Softmax4)

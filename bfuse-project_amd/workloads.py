@@ -148,7 +148,7 @@ def _qkv_ln_softmax_inputs():
 # horizontal-fuser/src/Algorithms.cc:23-35): name -> (standalone kernels, kind, suffixes built, inputs).
 # One full-size group: the fp32 QKV projection, the LayerNorm and the causal softmax of pairs 2 and 4.
 GROUPS = {
-    "qkv_ln_softmax": (("gemm_f32_512x768x2304", "layernorm_512x768", "softmax_causal_12x512x512"), "bfuse",
+    "qkv_ln_softmax": (("gemm_f32_512x768x2304_s2", "layernorm_512x768", "softmax_causal_12x512x512"), "bfuse",
                        ("_c256", "_r"), _qkv_ln_softmax_inputs),
 }
 

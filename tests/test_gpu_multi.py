@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 
 import bfuse_project_amd as bf
-from bfuse_project_amd.workloads import GROUPS
+from bfuse_project_amd.workloads import GROUPS as WORKLOAD_GROUPS
 from tests import oracle_cases
 from tests.test_gpu_small import _cases, _check
 from tests.test_group_host import GROUPS
@@ -112,7 +112,7 @@ def test_launch_lists_check_their_arguments():
 
 
 def test_full_size_three_kernels_bit_exact_close_to_cpu_and_timed():
-    names, _, _, inputs = GROUPS["qkv_ln_softmax"]
+    names, _, _, inputs = WORKLOAD_GROUPS["qkv_ln_softmax"]
     (I1, F1), (I2, F2), (I3, F3) = inputs()
     E1, E2 = oracle_cases.expected(2, I1, F1, I2, F2)
     from oracle import oracle as orf

@@ -17,8 +17,8 @@ GROUPS = [
     (("gemm_f32_128x160x192_d", "bias_relu_4096", "maxpool3x3s2_f32_4x16x16"), "hfuse", "", None),
     (("conv3x3_f32_32x12x12_32", "gemm_gelu_f32_96x128x192", "bias_relu_4096"), "hfuse", "", None),
     (("conv3x3_f32_32x12x12_32", "gemm_f32_128x160x192_d", "layernorm_8x256", "bias_relu_4096"), "hfuse", "", None),
-    (("gemm_f32_512x768x2304", "layernorm_512x768", "softmax_causal_12x512x512"), "bfuse", "_r", ("ranges", 0, 0)),
-    (("gemm_f32_512x768x2304", "layernorm_512x768", "softmax_causal_12x512x512"), "bfuse", "_c256", ("chunked", 256, 1)),
+    (("gemm_f32_512x768x2304_s2", "layernorm_512x768", "softmax_causal_12x512x512"), "bfuse", "_r", ("ranges", 0, 0)),
+    (("gemm_f32_512x768x2304_s2", "layernorm_512x768", "softmax_causal_12x512x512"), "bfuse", "_c256", ("chunked", 256, 1)),
 ]
 PATTERN_ID = {"zigzag": 0, "proportional": 1, "chunked": 2, "ranges": 3}
 
