@@ -31,15 +31,6 @@ __device__ __forceinline__ unsigned int f32_to_bf16_bits(float f)
     u += 0x7fffu + ((u >> 16) & 1u);
     return u >> 16;
 }
-// two fp32 -> two bf16 in one word (lo in the low half), round to nearest even: v_cvt_pk_bf16_f32
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ unsigned int pack_bf16(float lo, float hi)
-{
-    const f32x2 v = {lo, hi};
-    return __builtin_bit_cast(unsigned int, __builtin_convertvector(v, bf16x2));
-}
 __device__ __forceinline__ float bf16_bits_to_f32(unsigned int h) { return __builtin_bit_cast(float, h << 16); }
 
 // The K-pipeline is built around direct global->LDS loads

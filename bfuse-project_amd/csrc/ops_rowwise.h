@@ -14,6 +14,7 @@ namespace bfuse {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned short u16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 struct NoSmem {
     // empty: the operator uses no LDS
@@ -246,20 +247,22 @@ struct RmsNormRope {
 #pragma unroll
         for (int e = 0; e < 8; ++e) f[e] = __builtin_bit_cast(float, (unsigned int)h[e] << 16);
     }
-    __device__ static __forceinline__ unsigned short to_bf16(float f)
-    {
-        unsigned int u = __builtin_bit_cast(unsigned int, f);
-        u += 0x7fffu + ((u >> 16) & 1u);
-        return (unsigned short)(u >> 16);
-    }
     // The arithmetic of one element pair (j, j + HALF) -- the one place it is written, whichever way
     // the inputs arrived:  t = w (x r);  out_lo = t_lo cos_lo - t_hi sin_lo;  out_hi = t_hi cos_hi + t_lo sin_hi
     __device__ static __forceinline__ void rotate_pair(float w_lo, float w_hi, float x_lo, float x_hi, float r, float c_lo, float s_lo,
-                                                       float c_hi, float s_hi, unsigned short& o_lo, unsigned short& o_hi)
+                                                       float c_hi, float s_hi, float& o_lo, float& o_hi)
     {
         const float tl = w_lo * (x_lo * r), th = w_hi * (x_hi * r);
-        o_lo = to_bf16(tl * c_lo + (-th) * s_lo);
-        o_hi = to_bf16(th * c_hi + tl * s_hi);
+        o_lo = tl * c_lo + (-th) * s_lo;
+        o_hi = th * c_hi + tl * s_hi;
+    }
+    // eight fp32 -> eight bf16 (round to nearest even), two per conversion instruction
+    __device__ static __forceinline__ u16x8 round_octet(const float (&f)[8])
+    {
+        u32x4 p;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) p[e] = pack_bf16(f[2 * e], f[2 * e + 1]);
+        return __builtin_bit_cast(u16x8, p);
     }
     __device__ static __forceinline__ int slot_base(int slot) { return (slot / OCT) * HD + (slot % OCT) * 8; }
     __device__ static __forceinline__ void load_octets(u16x8& lo, u16x8& hi, int slot, const unsigned short* __restrict__ p)
@@ -338,16 +341,12 @@ struct RmsNormRope {
                 unpack(whi[s], wh);
                 unpack(xl[s], lo);
                 unpack(xh[s], hi);
-                u16x8 ol, oh;
+                float ol[8], oh[8];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    unsigned short a, b;
-                    rotate_pair(wl[e], wh[e], lo[e], hi[e], rs, cl[e / 4][e % 4], sl[e / 4][e % 4], ch[e / 4][e % 4], sh[e / 4][e % 4], a, b);
-                    ol[e] = a;
-                    oh[e] = b;
-                }
-                *reinterpret_cast<u16x8*>(y + slot_base(slot)) = ol;
-                *reinterpret_cast<u16x8*>(y + slot_base(slot) + HALF) = oh;
+                for (int e = 0; e < 8; ++e)
+                    rotate_pair(wl[e], wh[e], lo[e], hi[e], rs, cl[e / 4][e % 4], sl[e / 4][e % 4], ch[e / 4][e % 4], sh[e / 4][e % 4], ol[e], oh[e]);
+                *reinterpret_cast<u16x8*>(y + slot_base(slot)) = round_octet(ol);
+                *reinterpret_cast<u16x8*>(y + slot_base(slot) + HALF) = round_octet(oh);
             }
         } else {
             // on its own the body leaves the order of the operand loads to the compiler (it requests
@@ -362,16 +361,12 @@ struct RmsNormRope {
                 unpack(*reinterpret_cast<const u16x8*>(w + base + HALF), wh);
                 unpack(xl[s], lo);
                 unpack(xh[s], hi);
-                u16x8 ol, oh;
+                float ol[8], oh[8];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    unsigned short a, b;
-                    rotate_pair(wl[e], wh[e], lo[e], hi[e], r, cosv[j + e], sinv[j + e], cosv[j + HALF + e], sinv[j + HALF + e], a, b);
-                    ol[e] = a;
-                    oh[e] = b;
-                }
-                *reinterpret_cast<u16x8*>(y + base) = ol;
-                *reinterpret_cast<u16x8*>(y + base + HALF) = oh;
+                for (int e = 0; e < 8; ++e)
+                    rotate_pair(wl[e], wh[e], lo[e], hi[e], r, cosv[j + e], sinv[j + e], cosv[j + HALF + e], sinv[j + HALF + e], ol[e], oh[e]);
+                *reinterpret_cast<u16x8*>(y + base) = round_octet(ol);
+                *reinterpret_cast<u16x8*>(y + base + HALF) = round_octet(oh);
             }
         }
     }

@@ -61,6 +61,16 @@ __device__ __forceinline__ void dma_load_lds_b128(unsigned voff, const void* bas
 #endif
 }
 
+// two fp32 -> two bf16 in one word (lo in the low half), round to nearest even: v_cvt_pk_bf16_f32
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ unsigned int pack_bf16(float lo, float hi)
+{
+    const f32x2 v = {lo, hi};
+    return __builtin_bit_cast(unsigned int, __builtin_convertvector(v, bf16x2));
+}
+
 // ---- synchronisation policies ---------------------------------------------------------
 // Counts waits that gave up (see GroupSync); read back by the host after a fused launch.
 static __device__ unsigned int g_sync_timeouts;
