@@ -1,4 +1,4 @@
-"""Pattern / ratio chooser for a pair, measured at run time.
+"""Pattern / ratio chooser for a pair (or a group of up to four kernels), measured at run time.
 
 The reference hard-codes the live pattern and its M, N in Contexts.cc:64-79 and sweeps ratios
 by editing that file and rebuilding the tool and the suite for every point
@@ -136,3 +136,66 @@ def find_variant(k1: KernelHandle, k2: KernelHandle, choice: dict) -> Optional[K
         if same_dispatch(want, have):
             return k
     return None
+
+
+# ---- groups of more than two kernels (the fuser's Kernels list, Algorithms.cc:23-35) ---------------
+def group_candidates(grids: Sequence[int], cus: int = 256) -> List[Candidate]:
+    big = max(grids)
+    out = [Candidate("ranges", "ranges")]
+    for c in (cus // 4, cus // 2, cus, 2 * cus):
+        if c < big:
+            out.append(Candidate(f"chunk {c}", "chunked", c))
+    out.append(Candidate("zigzag 1:1", "zigzag", 1, 1))
+    out.append(Candidate("zigzag M=4", "zigzag", 4, 1))
+    out.append(Candidate("proportional", "proportional", 1))
+    for k in (1, 2, 4):
+        if k * cus < sum(grids):
+            out.append(Candidate(f"chunk {cus}, {k * cus} persistent workgroups", "chunked", cus, 1, k * cus))
+    return out
+
+
+def static_plan_group(kernels: Sequence[KernelHandle], cus: int = 256) -> dict:
+    """The footprint rule for more than two kernels: block fusion in chunks of one round over the CUs
+    (the largest LDS footprint is charged to every workgroup; `wg_per_cu` says how many then fit)."""
+    lds = max(max(k.lds_bytes, 0) for k in kernels)
+    regs = max(max(k.regs, 1) for k in kernels)
+    fit = []
+    for k in kernels:
+        waves = -(-(k.block[0] * k.block[1] * k.block[2]) // 64)
+        by_reg = (config.VGPRS_PER_SIMD // regs) * 4 // waves
+        by_wave = config.MAX_WAVES_PER_SIMD * 4 // waves
+        by_lds = config.LDS_PER_CU // lds if lds else 1 << 30
+        fit.append(max(1, min(by_reg, by_wave, by_lds)))
+    return {"kind": "bfuse", "pattern": "chunked", "p0": cus, "p1": 1, "static": {"wg_per_cu": tuple(fit), "chunk": cus}}
+
+
+def built_group_variants(names: Sequence[str]) -> List[KernelHandle]:
+    from .operation import list_kernels
+    return [k for k in list_kernels() if k.kind in (1, 2) and k.sides == tuple(names)]
+
+
+def find_group_variant(kernels: Sequence[KernelHandle], choice: dict) -> Optional[KernelHandle]:
+    """The built compile-time kernel of the group whose dispatch table equals the chosen plan's."""
+    dims = [patterns.LaunchDims(tuple(k.grid), tuple(k.block)) for k in kernels]
+    want = patterns.plan_blocks(choice["pattern"], dims, max(choice["p0"], 1), max(choice["p1"], 1))
+    for k in built_group_variants([k.name for k in kernels]):
+        if k.kind == 1 and same_dispatch(want, patterns.plan_blocks(_PATTERN_NAMES[k.pattern], dims, max(k.p0, 1), max(k.p1, 1))):
+            return k
+    return None
+
+
+def autotune_group(op, candidates: Optional[Sequence[Candidate]] = None, warmup: int = 20, reps: int = 100,
+                   cus: int = 256) -> List[dict]:
+    """autotune for a GroupOperation: times candidate plans on the group's run-time-plan kernel."""
+    rt = op.fused("bfuse", "_rt")
+    ldims = [patterns.LaunchDims(tuple(k.grid), tuple(k.block)) for k in op.k]
+    sides = tuple(range(len(op.k)))
+    rows = []
+    for c in (candidates if candidates is not None else group_candidates([k.grid[0] for k in op.k], cus)):
+        plan = patterns.plan_blocks(c.pattern, ldims, c.p0, c.p1)
+        h = op.set_plan(rt, plan, c.workgroups)
+        each, queued = op.time([(h, sides)], warmup=warmup, reps=reps)
+        rows.append({"label": c.label, "pattern": c.pattern, "p0": c.p0, "p1": c.p1, "workgroups": h.grid[0],
+                     "persistent": c.workgroups is not None, "us_mean": float(each[0]), "us_queued": float(queued)})
+    rows.sort(key=lambda r: r["us_mean"])
+    return rows

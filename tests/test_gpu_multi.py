@@ -10,6 +10,7 @@ import numpy as np
 import pytest
 
 import bfuse_project_amd as bf
+from bfuse_project_amd import patterns, tuner
 from bfuse_project_amd.workloads import GROUPS as WORKLOAD_GROUPS
 from tests import oracle_cases
 from tests.test_gpu_small import _cases, _check
@@ -145,3 +146,42 @@ def test_full_size_three_kernels_bit_exact_close_to_cpu_and_timed():
             assert _same(op.download(i), want[i]), ("rt", names[i])
         # three kernels hidden behind one: the fused kernel must beat the queued triple clearly
         assert queued_f < 0.95 * queued_u
+
+
+def test_autotune_of_the_full_size_group_agrees_with_the_footprint_rule():
+    """Candidate plans timed on the group's run-time-plan kernel: the rule's plan (one chunk per round
+    over the CUs) must be within 3 % of the best candidate with one workgroup per fused block, and
+    the compile-time kernel with that dispatch is the one the benchmark measures."""
+    names, kind, suffixes, inputs = WORKLOAD_GROUPS["qkv_ln_softmax"]
+    with bf.GroupOperation(names) as op:
+        for i, (I, F) in enumerate(inputs()):
+            op.upload(i, I, F)
+        op.launch(op.unfused())
+        want_out = [op.download(i) for i in range(len(names))]
+        choice = tuner.static_plan_group(op.k)
+        dims = [patterns.LaunchDims(tuple(k.grid), tuple(k.block)) for k in op.k]
+        want = patterns.plan_blocks(choice["pattern"], dims, choice["p0"], choice["p1"])
+
+        def timed():
+            rows = tuner.autotune_group(op, warmup=20, reps=100)
+            plain = [r for r in rows if not r["persistent"]]
+            mine = [r for r in plain if tuner.same_dispatch(want, patterns.plan_blocks(r["pattern"], dims, r["p0"], r["p1"]))]
+            return rows, mine, min(r["us_mean"] for r in plain)
+
+        rows, mine, best_plain = timed()
+        for r in rows:
+            _say(f"[tune-group] {r['label']:44s} {r['us_mean']:8.2f} us (queued {r['us_queued']:.2f}) workgroups {r['workgroups']}")
+        assert mine, "the footprint rule's plan is not among the candidates"
+        if min(r["us_mean"] for r in mine) > 1.03 * best_plain:
+            rows, mine, best_plain = timed()   # a 3 % comparison: one disturbed sample must not decide it
+        _say(f"[tune-group] footprint rule -> {mine[0]['label']} {mine[0]['us_mean']:.2f} us, best plain candidate {best_plain:.2f} us")
+        assert min(r["us_mean"] for r in mine) <= 1.03 * best_plain
+        # the winner, installed again, still reproduces the standalone kernels
+        best = rows[0]
+        h = op.set_plan(op.fused("bfuse", "_rt"), patterns.plan_blocks(best["pattern"], dims, best["p0"], best["p1"]), best["workgroups"])
+        op.zero_outputs()
+        op.launch([(h, tuple(range(len(names))))])
+        for i in range(len(names)):
+            assert _same(op.download(i), want_out[i]), (best["label"], names[i])
+        v = tuner.find_group_variant(op.k, choice)
+        assert v is not None and v.name == "_".join(names) + f"_fused_{kind}{suffixes[0]}"
