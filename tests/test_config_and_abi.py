@@ -55,6 +55,20 @@ def test_device_entry_points_fail_loudly_without_a_gpu():
     assert rc == -2 and "no CPU path" in out.stdout
 
 
+def test_launch_lists_and_generic_sides_refuse_work_before_init():
+    """No compute call without a device: the entry points for more than two kernels return an error
+    state (not a crash) when bfuse_init has not succeeded."""
+    import subprocess
+    import sys
+    code = ("import ctypes as C, sys; sys.path.insert(0, %r); from bfuse_project_amd import _lib; l = _lib.lib();"
+            "d = (_lib.LaunchDescC * 1)(); s = (C.c_int * 4)(1, 1, 1, 1); us = C.c_float();"
+            "print(l.bfuse_launch_list(1, d), l.bfuse_time_list(1, d, 1, 1, C.byref(us), C.byref(us)),"
+            " l.bfuse_initialize_side(3, s, s, s), l.bfuse_initialize_side(5, s, s, s), l.bfuse_finalize_side(0))" % ROOT)
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env={**os.environ, "HIP_VISIBLE_DEVICES": "-1"})
+    rcs = [int(x) for x in out.stdout.split()]
+    assert len(rcs) == 5 and all(rc < 0 for rc in rcs), (out.stdout, out.stderr[-500:])
+
+
 def test_reference_yaml_files_load(golden_dir):
     d = os.path.join(golden_dir, "config_sample")
     kernels = bf.load_kernels_yaml(os.path.join(d, "kernels.yaml"))          # written by PyYAML
