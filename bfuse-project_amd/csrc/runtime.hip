@@ -865,8 +865,14 @@ int bfuse_time(int mode, const void* fa, const unsigned* ga, const unsigned* ba,
     const int per = two ? 4 : 2;
     for (int r = 0; r < reps; ++r)
         for (int j = 0; j < per; ++j) HIP_TRY(hipEventCreate(&ev[(size_t)r * 4 + j]));
-    for (int r = 0; r < reps; ++r)
+    for (int r = 0; r < reps; ++r) {
         if ((rc = enqueue_mode(mode, fa, ga, ba, fb, gb, bb, &ev[(size_t)r * 4]))) return rc;
+        // Two streams run ahead of each other: without a meeting point per repetition the short
+        // kernel's stream would be hundreds of launches ahead and "first start -> last end" of
+        // repetition r would span all of them.  The reference synchronises after every run_parallel
+        // (operation_cu.py:199-228).
+        if (mode == BFUSE_MODE_PARALLEL) HIP_TRY(hipDeviceSynchronize());
+    }
     if ((rc = sync_and_check())) return rc;
     for (int r = 0; r < reps; ++r) {
         hipEvent_t* e = &ev[(size_t)r * 4];

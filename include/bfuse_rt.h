@@ -216,7 +216,9 @@ int bfuse_launch(int mode, const void* func_a, const unsigned* grid_a, const uns
 
 /* `warmup` untimed + `reps` timed launches of `mode`; GPU timestamps of each kernel's own
  * start and end.  us_total[r] = first kernel start -> last kernel end of repetition r;
- * us_a[r], us_b[r] = duration of each kernel (us_b only for modes 2 and 5; may be NULL). */
+ * us_a[r], us_b[r] = duration of each kernel (us_b only for modes 2 and 5; may be NULL).
+ * In mode 2 the device is synchronised after every repetition, as the reference's run_parallel
+ * does (operation_cu.py:199-228): two free-running streams would drift whole launches apart. */
 int bfuse_time(int mode, const void* func_a, const unsigned* grid_a, const unsigned* block_a,
                const void* func_b, const unsigned* grid_b, const unsigned* block_b, int warmup, int reps,
                float* us_total, float* us_a, float* us_b);
