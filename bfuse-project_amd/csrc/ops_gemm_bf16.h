@@ -24,15 +24,6 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
-// fp32 -> bf16 bits, round to nearest even (finite inputs)
-__device__ __forceinline__ unsigned int f32_to_bf16_bits(float f)
-{
-    unsigned int u = __builtin_bit_cast(unsigned int, f);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return u >> 16;
-}
-__device__ __forceinline__ float bf16_bits_to_f32(unsigned int h) { return __builtin_bit_cast(float, h << 16); }
-
 // The K-pipeline is built around direct global->LDS loads
 // (global_load_lds_dwordx4): no staging registers, NSTG LDS stages in a ring, NSTG-1
 // K-steps of loads in flight while one is multiplied.  A wave-level load writes 64 lanes x
