@@ -24,6 +24,42 @@ def test_every_declared_symbol_is_exported():
         assert hasattr(lib, name), f"libbfuse_rt.so does not export {name}"
 
 
+def test_the_header_is_plain_c_and_the_group_example_compiles(tmp_path):
+    """include/bfuse_rt.h must be usable from C (the reference's harness is C-callable) and the
+    three-kernel binding shown to maintainers must compile against it."""
+    import shutil
+    import subprocess
+    if not shutil.which("gcc"):
+        pytest.skip("no gcc")
+    hdr = os.path.join(ROOT, "include", "bfuse_rt.h")
+    subprocess.check_call(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only", "-x", "c", hdr])
+    src = tmp_path / "group.c"
+    src.write_text('''
+#include <stdio.h>
+#include "bfuse_rt.h"
+int run(const void* I[3], const void* F[3], void* O[3]) {
+    bfuse_kernel_info k[3], fused;
+    const char* names[3] = {"gemm_f32_512x768x2304_s2", "layernorm_512x768", "softmax_causal_12x512x512"};
+    int i;
+    for (i = 0; i < 3; ++i) {
+        if (bfuse_kernel_find(names[i], &k[i])) return 1;
+        bfuse_set_elem_bytes(i + 1, k[i].elem_bytes[0], k[i].elem_bytes[1], k[i].elem_bytes[2]);
+        if (bfuse_initialize_side(i + 1, k[i].shape[0], k[i].shape[1], k[i].shape[2])) return 2;
+        bfuse_upload(i + 1, I[i], F[i]);
+    }
+    if (bfuse_kernel_find("gemm_f32_512x768x2304_s2_layernorm_512x768_softmax_causal_12x512x512_fused_bfuse_c256", &fused)) return 3;
+    {
+        bfuse_launch_desc d = {fused.func, {fused.grid[0], 1, 1}, {fused.block[0], 1, 1}, fused.n_sides, {1, 2, 3, 0}};
+        float us_each, us_queued;
+        if (bfuse_launch_list(1, &d) || bfuse_time_list(1, &d, 20, 300, &us_each, &us_queued)) { fprintf(stderr, "%s\\n", bfuse_last_error()); return 4; }
+    }
+    for (i = 0; i < 3; ++i) { bfuse_download(i + 1, O[i]); bfuse_finalize_side(i + 1); }
+    return 0;
+}
+''')
+    subprocess.check_call(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), "-c", str(src), "-o", str(tmp_path / "group.o")])
+
+
 def test_registry_lists_pairs_and_fused_names_follow_the_reference():
     ks = {k.name: k for k in bf.list_kernels()}
     from bfuse_project_amd.workloads import PAIRS, fusions
