@@ -102,6 +102,8 @@ BFUSE_HFUSE_KERNEL(maxpool3x3s2_f32_4x16x16, PoolS, layernorm_8x256, LayerNormS)
 // a side with a barrier in its K loop under horizontal fusion, both sides synchronising: its fence-free
 // barriers become the LDS-counter one
 BFUSE_HFUSE_KERNEL(gemm_bf16_256x320x1792_w8, GemmB5, gemm_f32_128x160x192_d, GemmS5)
+// (the producer-wave GEMMs are not paired with a synchronising partner: their K loop under the LDS-counter
+// barrier needs more scalar registers than there are, and the build refuses kernels that spill)
 // the same GEMM with producer waves keeps the hardware barrier in its K loop and the norm waves join
 // its first four barriers (16 GEMM tiles, 3 norm workgroups: most workgroups have no norm waves at all)
 BFUSE_HFUSE_KERNEL(gemm_bf16_256x384x1792_p, GemmB8, rmsnorm_rope_bf16_6x1024, NormRopeS)

@@ -15,6 +15,8 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "dispatch.h"
 #include "wave.h"
 
@@ -412,7 +414,10 @@ struct GemmBf16NTDma {
         // the loop stays rolled whatever K is: operand registers with reads in flight must never be
         // spilled (the compiler takes an asm output for written when the asm is issued), and a
         // fully unrolled short loop is where the register allocator runs out
-        if constexpr (EARLY_ > 0) {
+        // the early barrier is built on the hardware barrier: the LDS-counter barrier a side gets when its
+        // partner synchronises too has LDS traffic of its own, and its inlined polls in every unrolled step
+        // cost more scalar registers than there are -- that side runs the loop with the barrier on top
+        if constexpr (EARLY_ > 0 && std::is_same<Sync, BlockSync>::value) {
             Frags fr[2];
             sync.raw();   // K-step 0 is in LDS
             read_a_all<0, 0, 0>(fr[0].af[0], ad);
