@@ -50,6 +50,10 @@ if ROOT not in sys.path:
 import numpy as np  # noqa: E402
 
 
+# launches per unfused baseline and per queued figure when --steps is smaller (see measure())
+BASELINE_MIN_REPS = 500
+
+
 def cpu_baseline(pair_number, I1, F1, I2, F2, passes=5):
     """Times the CPU oracle (the checker, not the product) on this host: best of `passes`."""
     from oracle import oracle as orf
@@ -172,10 +176,15 @@ def measure(number, K, W, spec):
         bit_exact = bool(np.array_equal(U1.view(np.uint8), Q1.view(np.uint8)) and
                          np.array_equal(U2.view(np.uint8), Q2.view(np.uint8)))
 
-        # GPU-side durations (dispatch timestamps), W warm-up + K timed launches each
+        # GPU-side durations (dispatch timestamps).  The fused kernel: W warm-up + exactly K timed
+        # launches per pass.  The unfused baselines are figures of their own and take R = max(K, 500)
+        # launches, so that a short run (K = 20 is one millisecond of work) still compares against
+        # baselines with usable statistics -- and the reported fused pass, which follows them, finds the
+        # chip at the clock a busy GPU runs at instead of the one it idles at.
+        R = max(K, BASELINE_MIN_REPS)
         t_f1 = op.time(kind, fused, warmup=W, reps=K)[0]
-        t_ser, t_a, t_b = op.time("serial", warmup=W, reps=K)
-        t_par = op.time("parallel", warmup=W, reps=K)[0]
+        t_par = op.time("parallel", warmup=W, reps=R)[0]     # meets the host after every repetition: run first
+        t_ser, t_a, t_b = op.time("serial", warmup=W, reps=R)
         t_f = op.time(kind, fused, warmup=W, reps=K)[0]     # the reported pass: after the baselines
         fused_us = float(t_f.mean())
 
@@ -189,10 +198,13 @@ def measure(number, K, W, spec):
         op.synchronize()
         wall_ms = (time.perf_counter() - t0) * 1e3 / K
 
-        b_f = op.time_batched(kind, fused, warmup=W, reps=K)
-        b_ser = op.time_batched("serial", warmup=W, reps=K)
-        b_k1 = op.time_batched("kernel1", warmup=W, reps=K)
-        b_k2 = op.time_batched("kernel2", warmup=W, reps=K)
+        # queued figures: fused and unfused alike, R untimed launches of the same thing and then R timed
+        # ones (a ratio of two like runs; whichever came first would otherwise meet the colder chip)
+        BW = max(W, R)
+        b_f = op.time_batched(kind, fused, warmup=BW, reps=R)
+        b_ser = op.time_batched("serial", warmup=BW, reps=R)
+        b_k1 = op.time_batched("kernel1", warmup=BW, reps=R)
+        b_k2 = op.time_batched("kernel2", warmup=BW, reps=R)
 
     # fused forms the configuration names that are not the measured kernel, timed beside it
     extra = {}
@@ -210,9 +222,9 @@ def measure(number, K, W, spec):
             op.launch(akind, alt)
             Z1, Z2 = op.download(0), op.download(1)
             alt_exact = bool(np.array_equal(V1.view(np.uint8), Z1.view(np.uint8)) and np.array_equal(V2.view(np.uint8), Z2.view(np.uint8)))
-            t_z = op.time(akind, alt, warmup=W, reps=K)[0]
-            b_z = op.time_batched(akind, alt, warmup=W, reps=K)
-            b_zs = op.time_batched("serial", warmup=W, reps=K)
+            t_z = op.time(akind, alt, warmup=W, reps=R)[0]
+            b_z = op.time_batched(akind, alt, warmup=BW, reps=R)
+            b_zs = op.time_batched("serial", warmup=BW, reps=R)
         extra[label] = {"kernel": alt.name, "fused_us": round(float(t_z.mean()), 3), "batched_fused_us": round(b_z, 3),
                         "batched_back_to_back_us": round(b_zs, 3), "batched_fused_over_back_to_back": round(b_z / b_zs, 4),
                         "bit_exact_vs_unfused": alt_exact}
@@ -246,6 +258,7 @@ def measure(number, K, W, spec):
         "batched_kernel2_us": round(b_k2, 3),
         "batched_fused_over_back_to_back": round(b_f / b_ser, 4),
         "ms_per_step": round(wall_ms, 6),
+        "baseline_reps": R,
         "roofline": {"bound": pair.bound, "achieved": round(achieved, 2), "peak": pair.peak, "unit": unit,
                      "frac": round(achieved / pair.peak, 4), "traffic": MEASURED_TRAFFIC.get(fused.name),
                      "traffic_source": TRAFFIC_SOURCE.get(fused.name),
@@ -274,8 +287,9 @@ def measure_group(name, K, W):
         op.zero_outputs()
         op.launch([(fused, tuple(range(len(names))))])
         exact = all(np.array_equal(op.download(i).view(np.uint8), want[i].view(np.uint8)) for i in range(len(names)))
-        each_u, queued_u = op.time(op.unfused(), warmup=W, reps=K)
-        each_f, queued_f = op.time([(fused, tuple(range(len(names))))], warmup=W, reps=K)
+        R = max(K, BASELINE_MIN_REPS)
+        each_u, queued_u = op.time(op.unfused(), warmup=max(W, R), reps=R)
+        each_f, queued_f = op.time([(fused, tuple(range(len(names))))], warmup=max(W, R), reps=R)
     return {"kernels": list(names), "fused_kernel": fused.name, "fused_us": round(float(each_f[0]), 3),
             "kernel_us": [round(float(x), 3) for x in each_u], "batched_fused_us": round(queued_f, 3),
             "batched_back_to_back_us": round(queued_u, 3), "batched_fused_over_back_to_back": round(queued_f / queued_u, 4),
