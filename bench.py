@@ -34,8 +34,10 @@ Top level only:
   groups            fusions of more than two kernels (one: the fp32 QKV GEMM, LayerNorm and causal softmax
                     as one block-fused kernel) against their standalone kernels queued back to back
   cpu_baseline      the OpenMP CPU reference (oracle/) timed on this host's cores
-  hbm_copy_GBps     what the library's 64 MiB -> 64 MiB copy kernel reaches in this run (a measured
-                    ceiling beside the nominal 8000)
+  measured_ceilings what this chip sustains in this run, beside the published peaks `roofline.peak` divides by:
+                    the library's 64 MiB -> 64 MiB copy kernel (GB/s; also `hbm_copy_GBps`) and its MFMA-only
+                    kernels, bf16 and fp32, with operands that toggle bits and no memory traffic (TFLOP/s);
+                    each pair's `roofline.measured_peak` / `frac_of_measured_peak` use the one of its bound
 """
 import argparse
 import json
@@ -104,6 +106,31 @@ def hbm_copy_rate(reps=50):
     return 2 * 16777216 * 4 / float(np.mean(t)) * 1e-3
 
 
+# the library's MFMA-only kernels (csrc/ops_ceiling.h): name and flops per launch, by arithmetic type
+MFMA_STREAMS = {"bf16": ("mfma_stream_bf16_2000", 256 * 8 * 14 * 2000 * 16384.0),
+                "f32": ("mfma_stream_f32_1000", 256 * 8 * 14 * 1000 * 2048.0)}
+
+
+def mfma_stream_rate(dtype, reps=100):
+    """TFLOP/s of a dense stream of independent MFMAs of this type with operands that toggle bits and no
+    memory traffic (two waves per SIMD on every CU): what the matrix cores sustain at the clock the chip
+    grants them in this run -- a measured ceiling beside the published peak."""
+    import bfuse_project_amd as bf
+    name, flops = MFMA_STREAMS[dtype]
+    with bf.Operation(name, "bias_relu_4096") as op:
+        op.upload(0, np.zeros(1, np.float32), np.zeros(1, np.float32))
+        # 100 launches of 0.4-0.6 ms: long enough for the power management to settle (the first few
+        # milliseconds of a burst run faster than what the chip then sustains)
+        t = op.time("kernel1", warmup=20, reps=reps)[0]
+    return flops / float(np.mean(t[reps // 2:])) * 1e-6
+
+
+def measured_ceilings():
+    return {"hbm_copy_GBps": round(hbm_copy_rate(), 1),
+            "mfma_bf16_TFLOPs": round(mfma_stream_rate("bf16"), 1),
+            "mfma_f32_TFLOPs": round(mfma_stream_rate("f32"), 1)}
+
+
 def pick_fusion(number, spec):
     """(k1, k2, kind, suffix, note) for a pair under --fusion `spec`."""
     import bfuse_project_amd as bf
@@ -145,7 +172,7 @@ def pick_fusion(number, spec):
     return k1, k2, hk, sfx, note
 
 
-def measure(number, K, W, spec):
+def measure(number, K, W, spec, ceilings):
     import bfuse_project_amd as bf
     from bfuse_project_amd import tuner
     from bfuse_project_amd.workloads import PAIRS, MEASURED_TRAFFIC, TRAFFIC_SOURCE, CONFIG_KINDS, BESIDE, FLOORS
@@ -234,8 +261,10 @@ def measure(number, K, W, spec):
     back_to_back = float(t_ser.mean())
     if pair.bound == "mfma":
         achieved, unit = pair.flops / fused_us * 1e-6, "TFLOP/s"      # flops / us = MFLOP/s
+        measured_peak = ceilings["mfma_bf16_TFLOPs" if pair.dtype == "bf16" else "mfma_f32_TFLOPs"]
     else:
         achieved, unit = (pair.bytes1 + pair.bytes2) / fused_us * 1e-3, "GB/s"
+        measured_peak = ceilings["hbm_copy_GBps"]
     res = {
         "workload": f"pair {pair.number}: {pair.title}",
         "dtype": pair.dtype,
@@ -260,7 +289,9 @@ def measure(number, K, W, spec):
         "ms_per_step": round(wall_ms, 6),
         "baseline_reps": R,
         "roofline": {"bound": pair.bound, "achieved": round(achieved, 2), "peak": pair.peak, "unit": unit,
-                     "frac": round(achieved / pair.peak, 4), "traffic": MEASURED_TRAFFIC.get(fused.name),
+                     "frac": round(achieved / pair.peak, 4),
+                     "measured_peak": measured_peak, "frac_of_measured_peak": round(achieved / measured_peak, 4),
+                     "traffic": MEASURED_TRAFFIC.get(fused.name),
                      "traffic_source": TRAFFIC_SOURCE.get(fused.name),
                      "kernel": fused.name, "avg_us": round(fused_us, 3),
                      "algorithmic": {"flops": pair.flops, "bytes": pair.bytes1 + pair.bytes2}},
@@ -315,8 +346,9 @@ def main():
     numbers = [args.pair] if args.pair else [1, 2, 3, 4, 5]
     top = numbers[-1]
     pairs, top_inputs, dev = {}, None, ""
+    ceilings = measured_ceilings()
     for n in numbers:
-        res, dev, inputs = measure(n, K, W, args.fusion)
+        res, dev, inputs = measure(n, K, W, args.fusion, ceilings)
         pairs[str(n)] = res
         if n == top:
             top_inputs = inputs
@@ -340,7 +372,8 @@ def main():
         "fused_over_back_to_back": t["fused_over_back_to_back"],
         "batched_fused_over_back_to_back": t["batched_fused_over_back_to_back"],
         "roofline": t["roofline"],
-        "hbm_copy_GBps": round(hbm_copy_rate(), 1),
+        "hbm_copy_GBps": ceilings["hbm_copy_GBps"],
+        "measured_ceilings": ceilings,
         "pairs": pairs,
     }
     if not args.pair:

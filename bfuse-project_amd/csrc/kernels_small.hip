@@ -4,6 +4,7 @@
 // prefetch, multi-group convolution, several K-steps / M-tiles of the bf16 GEMM), sides with
 // different grid sizes under horizontal fusion, and the ratio / proportional block patterns.
 #include "fuse.h"
+#include "ops_ceiling.h"
 #include "ops_conv.h"
 #include "ops_gemm_bf16.h"
 #include "ops_gemm_f32.h"
@@ -87,6 +88,13 @@ BFUSE_KERNEL(rmsnorm_rope_bf16_6x1024, NormRopeS, ({{6, 1024, 1, 1}, 2}), ({{(in
 // calibration kernel for the memory counters: 64 MiB read, 64 MiB written
 using Copy64M = CopyF32<16777216, 256>;
 BFUSE_KERNEL(copy_f32_16777216, Copy64M, ({{16777216, 1, 1, 1}, 4}), ({{1, 1, 1, 1}, 4}), ({{16777216, 1, 1, 1}, 4}))
+
+// what the matrix cores sustain with nothing else going on: 2000 (bf16) / 1000 (fp32) rounds of 14
+// independent MFMAs per wave, 0.94 TFLOP / 0.059 TFLOP per launch (about 0.6 / 0.4 ms)
+using MfmaStreamBf16 = MfmaStream<true, 2000>;
+using MfmaStreamF32 = MfmaStream<false, 1000>;
+BFUSE_KERNEL(mfma_stream_bf16_2000, MfmaStreamBf16, ({{1, 1, 1, 1}, 4}), ({{1, 1, 1, 1}, 4}), ({{256, 512, 1, 1}, 4}))
+BFUSE_KERNEL(mfma_stream_f32_1000, MfmaStreamF32, ({{1, 1, 1, 1}, 4}), ({{1, 1, 1, 1}, 4}), ({{256, 512, 1, 1}, 4}))
 
 // horizontal fusion with unequal grids (9 GEMM tiles, 4 element-wise blocks) and a barrier side
 BFUSE_HFUSE_KERNEL(gemm_gelu_f32_96x128x192, GemmS2, bias_relu_4096, BiasReluS)

@@ -39,6 +39,10 @@ def test_one_json_line_covering_all_five_pairs():
     assert abs(rf["frac"] - rf["achieved"] / rf["peak"]) < 1e-3
     assert abs(rf["achieved"] - rf["algorithmic"]["flops"] / d["value"] * 1e-6) < 0.5
     assert rf["traffic"] and rf["traffic_source"].startswith("profiles/") and os.path.exists(os.path.join(ROOT, rf["traffic_source"]))
+    mc = d["measured_ceilings"]
+    assert 2000 < mc["hbm_copy_GBps"] <= 8000 * 1.05 and 800 < mc["mfma_bf16_TFLOPs"] <= 2500 and 50 < mc["mfma_f32_TFLOPs"] <= 157.3 * 1.02
+    assert rf["measured_peak"] == mc["mfma_bf16_TFLOPs"] and abs(rf["frac_of_measured_peak"] - rf["achieved"] / rf["measured_peak"]) < 1e-3
+    assert d["pairs"]["1"]["roofline"]["measured_peak"] == mc["hbm_copy_GBps"] and d["pairs"]["2"]["roofline"]["measured_peak"] == mc["mfma_f32_TFLOPs"]
     cb = d["cpu_baseline"]
     assert cb["kind"] == "port" and cb["cores"] >= 1 and cb["value"] > 0 and cb["sample"]
     for n, p in d["pairs"].items():

@@ -48,3 +48,28 @@ def test_placement_probe_shows_the_round_robin_the_dispatch_patterns_rely_on():
     assert len(cus) == 256 and counts.min() == 2 and counts.max() == 2
     with pytest.raises(Exception):
         probe_placement(0)
+
+
+@pytest.mark.parametrize("name,flops,nominal", [("mfma_stream_bf16_2000", 256 * 8 * 14 * 2000 * 16384.0, 2500.0),
+                                                 ("mfma_stream_f32_1000", 256 * 8 * 14 * 1000 * 2048.0, 157.3)])
+def test_mfma_only_kernels_give_a_ceiling_below_the_published_peak(name, flops, nominal):
+    """The measured-ceiling kernels of the bench line: the same bytes on every launch, finite and not all
+    zero, and a rate between a third of the published peak and the peak itself."""
+    import numpy as np
+    import bfuse_project_amd as bf
+    print(name, flush=True)
+    with bf.Operation(name, "bias_relu_4096") as op:
+        z = np.zeros(1, np.float32)
+        op.upload(0, z, z)
+        op.zero_outputs()
+        op.launch("kernel1")
+        a = op.download(0).copy()
+        op.zero_outputs()
+        op.launch("kernel1")
+        b = op.download(0)
+        t = op.time("kernel1", warmup=5, reps=20)[0]
+    assert a.size == 256 * 512 and np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    assert np.all(np.isfinite(a)) and np.count_nonzero(a) > a.size // 2
+    tflops = flops / float(np.mean(t)) * 1e-6
+    print(f"{name}: {tflops:.1f} TFLOP/s of {nominal}", flush=True)
+    assert nominal / 3 < tflops <= nominal * 1.02
