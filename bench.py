@@ -29,7 +29,10 @@ Per pair:
                     (includes dispatch gaps, lets consecutive launches overlap their ramp-up)
   roofline          algorithmic flops (or bytes) of the pair / fused duration vs the MI355X peak;
                     `traffic` is HBM bytes per launch from the rocprofv3 --pmc summary named in
-                    `traffic_source` (not measured by this run)
+                    `traffic_source` (not measured by this run); `same_kernel_constant_operands` (pairs with a
+                    matrix-core bound): the same fused kernel timed over all-ones contraction inputs -- same
+                    instructions and traffic, no operand bits toggling -- i.e. what the code sustains when the
+                    chip's power management is not holding the clock down for the data
 Top level only:
   groups            fusions of more than two kernels (one: the fp32 QKV GEMM, LayerNorm and causal softmax
                     as one block-fused kernel) against their standalone kernels queued back to back
@@ -233,6 +236,22 @@ def measure(number, K, W, spec, ceilings):
         b_k1 = op.time_batched("kernel1", warmup=BW, reps=R)
         b_k2 = op.time_batched("kernel2", warmup=BW, reps=R)
 
+        # The same fused kernel over constant operands (every element of the contraction's two inputs = 1):
+        # the same instructions and the same memory traffic, but no bits toggle in the matrix cores'
+        # operands, so the power management grants a higher clock.  What this reads is what the kernel's
+        # code sustains; the distance to `fused_us` is what the data costs in power on this chip.
+        const = None
+        if pair.bound == "mfma":
+            side = 0 if k1.startswith(("gemm", "conv")) else 1
+            ones = [np.full(x.shape, 0x3f80, np.uint16) if x.dtype == np.uint16 else np.ones(x.shape, np.float32)
+                    for x in (inputs[2 * side], inputs[2 * side + 1])]
+            op.upload(side, *ones)
+            t_c = op.time(kind, fused, warmup=BW, reps=R)[0]
+            const = {"fused_us": round(float(t_c.mean()), 3), "contraction_side": side + 1,
+                     "achieved": round(pair.flops / float(t_c.mean()) * 1e-6, 2),
+                     "frac": round(pair.flops / float(t_c.mean()) * 1e-6 / pair.peak, 4)}
+            op.upload(side, inputs[2 * side], inputs[2 * side + 1])
+
     # fused forms the configuration names that are not the measured kernel, timed beside it
     extra = {}
     for label, a1, a2, akind, asuffix in BESIDE.get(number, []):
@@ -297,6 +316,8 @@ def measure(number, K, W, spec, ceilings):
                      "algorithmic": {"flops": pair.flops, "bytes": pair.bytes1 + pair.bytes2}},
         **extra,
     }
+    if const:
+        res["roofline"]["same_kernel_constant_operands"] = const
     if number in FLOORS:
         res["floor"] = FLOORS[number]
     return res, dev, inputs

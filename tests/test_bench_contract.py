@@ -43,6 +43,9 @@ def test_one_json_line_covering_all_five_pairs():
     assert 2000 < mc["hbm_copy_GBps"] <= 8000 * 1.05 and 800 < mc["mfma_bf16_TFLOPs"] <= 2500 and 50 < mc["mfma_f32_TFLOPs"] <= 157.3 * 1.02
     assert rf["measured_peak"] == mc["mfma_bf16_TFLOPs"] and abs(rf["frac_of_measured_peak"] - rf["achieved"] / rf["measured_peak"]) < 1e-3
     assert d["pairs"]["1"]["roofline"]["measured_peak"] == mc["hbm_copy_GBps"] and d["pairs"]["2"]["roofline"]["measured_peak"] == mc["mfma_f32_TFLOPs"]
+    ck = rf["same_kernel_constant_operands"]      # the power check: same kernel, operands that toggle no bits
+    assert 0 < ck["fused_us"] < d["value"] and abs(ck["frac"] - ck["achieved"] / rf["peak"]) < 1e-3
+    assert "same_kernel_constant_operands" not in d["pairs"]["1"]["roofline"]
     cb = d["cpu_baseline"]
     assert cb["kind"] == "port" and cb["cores"] >= 1 and cb["value"] > 0 and cb["sample"]
     for n, p in d["pairs"].items():
