@@ -2,7 +2,7 @@
 """Headline benchmark: the five fused pairs on one MI355X, each against the same two kernels
 launched back to back.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--pair N] [--fusion SPEC] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--pair N] [--fusion SPEC] [--no-cpu] [--no-power-check]
 
 A step is one launch of a fused kernel over device-resident synthetic inputs.  By default all
 five pairs are measured in one run (the reference profiles its whole pair matrix,
@@ -175,7 +175,7 @@ def pick_fusion(number, spec):
     return k1, k2, hk, sfx, note
 
 
-def measure(number, K, W, spec, ceilings):
+def measure(number, K, W, spec, ceilings, power_check=True):
     import bfuse_project_amd as bf
     from bfuse_project_amd import tuner
     from bfuse_project_amd.workloads import PAIRS, MEASURED_TRAFFIC, TRAFFIC_SOURCE, CONFIG_KINDS, BESIDE, FLOORS
@@ -241,7 +241,7 @@ def measure(number, K, W, spec, ceilings):
         # operands, so the power management grants a higher clock.  What this reads is what the kernel's
         # code sustains; the distance to `fused_us` is what the data costs in power on this chip.
         const = None
-        if pair.bound == "mfma":
+        if pair.bound == "mfma" and power_check:
             side = 0 if k1.startswith(("gemm", "conv")) else 1
             ones = [np.full(x.shape, 0x3f80, np.uint16) if x.dtype == np.uint16 else np.ones(x.shape, np.float32)
                     for x in (inputs[2 * side], inputs[2 * side + 1])]
@@ -356,6 +356,8 @@ def main():
     ap.add_argument("--pair", type=int, default=0, help="measure this pair only (default: all five, pair 5 on top)")
     ap.add_argument("--fusion", default="", help="'' = headline, 'auto' = the tuner's choice, or kind[:suffix][@k1,k2] with --pair")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-power-check", action="store_true",
+                    help="skip the launches over constant operands (under a kernel trace they would be averaged into the fused kernel's figure)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures fused pairs on ONE GPU: the path has no cross-device data flow and "
@@ -369,7 +371,7 @@ def main():
     pairs, top_inputs, dev = {}, None, ""
     ceilings = measured_ceilings()
     for n in numbers:
-        res, dev, inputs = measure(n, K, W, args.fusion, ceilings)
+        res, dev, inputs = measure(n, K, W, args.fusion, ceilings, not args.no_power_check)
         pairs[str(n)] = res
         if n == top:
             top_inputs = inputs
