@@ -432,6 +432,10 @@ int bfuse_init(int device)
         return fail(BFUSE_ERR_HIP, "no HIP device available (%s); this library has no CPU path",
                     st == hipSuccess ? "device count is 0" : hipGetErrorString(st));
     if (device < 0 || device >= n) return fail(BFUSE_ERR_ARG, "device %d out of range (0..%d)", device, n - 1);
+    if (g.inited && device != g.device)
+        for (int i = 0; i < kMaxKernels; ++i)
+            if (g.side[i].live)
+                return fail(BFUSE_ERR_STATE, "side %d holds buffers on device %d: finalize it before moving to device %d", i + 1, g.device, device);
     HIP_TRY(hipSetDevice(device));
     // the allocation-free entry point's staging array: its address on this device, looked up now so
     // that the entry point itself calls nothing that could allocate
@@ -445,13 +449,22 @@ int bfuse_init(int device)
 
 int bfuse_shutdown(void)
 {
+    if (!g.inited) return BFUSE_OK;
+    // nothing may still run on buffers or code objects that are about to go
+    int rc = sync_and_check();
+    if (rc && rc != BFUSE_ERR_SYNC) return rc;
     for (int i = 0; i < kMaxKernels; ++i)
         if (g.side[i].live) {
-            int rc = fini_side(i);
-            if (rc) return rc;
+            int rc2 = fini_side(i);
+            if (rc2) return rc2;
+        }
+    for (auto& m : modules())
+        if (m) {
+            HIP_TRY(hipModuleUnload(m));
+            m = nullptr;
         }
     g.inited = false;
-    return BFUSE_OK;
+    return rc;
 }
 
 int bfuse_device_info(char* name, size_t name_len, int* cus, int* lds, int* wave)
@@ -494,6 +507,11 @@ int bfuse_plan_blocks(int pattern, int n, const bfuse_launch_dims* k, int p0, in
 
 int bfuse_map_block(const bfuse_block_plan* plan, int bid, int* virt)
 {
+    if (!plan) {
+        if (virt) *virt = -1;
+        (void)fail(BFUSE_ERR_ARG, "null plan");
+        return -1;
+    }
     int v = -1;
     const int k = map_block(*reinterpret_cast<const BlockPlan*>(plan), bid, &v);
     if (virt) *virt = v;
@@ -502,6 +520,11 @@ int bfuse_map_block(const bfuse_block_plan* plan, int bid, int* virt)
 
 int bfuse_map_thread(const bfuse_thread_plan* plan, int bid, int tid, int* local)
 {
+    if (!plan) {
+        if (local) *local = -1;
+        (void)fail(BFUSE_ERR_ARG, "null plan");
+        return -1;
+    }
     int l = -1;
     const int k = map_thread(*reinterpret_cast<const ThreadPlan*>(plan), bid, tid, &l);
     if (local) *local = l;

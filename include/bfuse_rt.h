@@ -37,6 +37,9 @@ const char* bfuse_last_error(void);
 /* Selects the device and creates the two streams the harness uses (S1, S2 of
  * operation_cu.py:126).  Fails if no HIP device is present: there is no CPU fallback. */
 int bfuse_init(int device);
+/* Waits for everything launched, frees the buffers of every side still initialized and unloads every code
+ * object still loaded.  Calling it before bfuse_init (or twice) is harmless.  bfuse_init may be called again
+ * afterwards; calling it for another device while a side still holds buffers is refused. */
 int bfuse_shutdown(void);
 /* name, CU count, LDS bytes per workgroup, wavefront size of the selected device */
 int bfuse_device_info(char* name, size_t name_len, int* compute_units, int* lds_bytes, int* wave_size);
@@ -81,7 +84,7 @@ enum {
 int bfuse_plan_threads(int n, const bfuse_launch_dims* kernels, int pad, bfuse_thread_plan* out);
 int bfuse_plan_blocks(int pattern, int n, const bfuse_launch_dims* kernels, int p0, int p1,
                       bfuse_block_plan* out);
-/* Return the kernel index owning the id (or -1 if none) */
+/* Return the kernel index owning the id (or -1 if none, or if plan is null) */
 int bfuse_map_block(const bfuse_block_plan* plan, int bid, int* virt_block);
 int bfuse_map_thread(const bfuse_thread_plan* plan, int bid, int tid, int* local_tid);
 /* Evaluates bfuse_map_block for bid in [lo,hi) ON THE GPU with the device build of the map

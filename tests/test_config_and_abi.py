@@ -105,6 +105,22 @@ def test_launch_lists_and_generic_sides_refuse_work_before_init():
     assert len(rcs) == 5 and all(rc < 0 for rc in rcs), (out.stdout, out.stderr[-500:])
 
 
+def test_null_plans_and_shutdown_before_init_are_errors_not_crashes():
+    import ctypes as C
+    from bfuse_project_amd import _lib
+    l = _lib.lib()
+    v = C.c_int(7)
+    assert l.bfuse_map_block(None, 0, C.byref(v)) == -1 and v.value == -1
+    v = C.c_int(7)
+    assert l.bfuse_map_thread(None, 0, 0, C.byref(v)) == -1 and v.value == -1
+    assert b"null plan" in l.bfuse_last_error()
+    import subprocess
+    import sys
+    code = ("import sys; sys.path.insert(0, %r); from bfuse_project_amd import _lib; l = _lib.lib(); print(l.bfuse_shutdown(), l.bfuse_shutdown())" % ROOT)
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env={**os.environ, "HIP_VISIBLE_DEVICES": "-1"})
+    assert out.stdout.split() == ["0", "0"], (out.stdout, out.stderr[-500:])
+
+
 def test_reference_yaml_files_load(golden_dir):
     d = os.path.join(golden_dir, "config_sample")
     kernels = bf.load_kernels_yaml(os.path.join(d, "kernels.yaml"))          # written by PyYAML

@@ -73,3 +73,26 @@ def test_mfma_only_kernels_give_a_ceiling_below_the_published_peak(name, flops, 
     tflops = flops / float(np.mean(t)) * 1e-6
     print(f"{name}: {tflops:.1f} TFLOP/s of {nominal}", flush=True)
     assert nominal / 3 < tflops <= nominal * 1.02
+
+
+def test_shutdown_releases_everything_and_the_library_can_be_initialized_again():
+    """bfuse_shutdown with a side still live and a launch still queued: it waits, frees the buffers, and a
+    later bfuse_init + operation works as before."""
+    import numpy as np
+    import bfuse_project_amd as bf
+    from bfuse_project_amd import _lib
+    print("shutdown / re-init", flush=True)
+    x = np.arange(4096, dtype=np.float32) - 2048.0
+    b = np.ones(4096, np.float32)
+    op = bf.Operation("bias_relu_4096", "layernorm_8x256")
+    op.upload(0, x, b)
+    op.launch("kernel1")
+    _lib.check(_lib.lib().bfuse_shutdown())          # side buffers of `op` are gone now
+    op.live = False
+    _lib.check(_lib.lib().bfuse_shutdown())          # twice is harmless
+    with bf.Operation("bias_relu_4096", "layernorm_8x256") as op2:
+        op2.upload(0, x, b)
+        op2.zero_outputs()
+        op2.launch("kernel1")
+        y = op2.download(0)
+    assert np.array_equal(y.ravel(), np.maximum(x + b, 0.0))
