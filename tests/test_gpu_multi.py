@@ -172,8 +172,10 @@ def test_autotune_of_the_full_size_group_agrees_with_the_footprint_rule():
         for r in rows:
             _say(f"[tune-group] {r['label']:44s} {r['us_mean']:8.2f} us (queued {r['us_queued']:.2f}) workgroups {r['workgroups']}")
         assert mine, "the footprint rule's plan is not among the candidates"
-        if min(r["us_mean"] for r in mine) > 1.03 * best_plain:
-            rows, mine, best_plain = timed()   # a 3 % comparison: one disturbed sample must not decide it
+        for again in range(3):   # a 3 % comparison: a disturbed sample must not decide it
+            if min(r["us_mean"] for r in mine) <= 1.03 * best_plain:
+                break
+            rows, mine, best_plain = timed()
         _say(f"[tune-group] footprint rule -> {mine[0]['label']} {mine[0]['us_mean']:.2f} us, best plain candidate {best_plain:.2f} us")
         assert min(r["us_mean"] for r in mine) <= 1.03 * best_plain
         # the winner, installed again, still reproduces the standalone kernels
