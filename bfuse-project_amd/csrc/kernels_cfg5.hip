@@ -3,6 +3,7 @@
 // 32 heads x 128.
 #include "fuse.h"
 #include "ops_gemm_bf16.h"
+#include "ops_layout.h"
 #include "ops_rowwise.h"
 
 using namespace bfuse;
@@ -44,3 +45,7 @@ BFUSE_BFUSE_KERNEL(gemm_bf16_512x4096x14336, GemmGate, rmsnorm_rope_bf16_512x409
 // dense inputs, small enough for the CPU reference to evaluate the whole matrix
 using GemmGateK256 = GemmBf16NTDma<512, 14336, 256, 128, 224, 3, 4, 4, 2, 2, 11>;
 BFUSE_KERNEL(gemm_bf16_512x256x14336, GemmGateK256, ({{512, 256, 1, 1}, 2}), ({{14336, 256, 1, 1}, 2}), ({{512, 14336, 1, 1}, 2}))
+
+// a weight held as [K, N] = [4096, 14336] is brought into the GEMM's [N, K] layout once, when it is loaded
+using WeightToNK = Transpose16<4096, 14336>;
+BFUSE_KERNEL(transpose16_4096x14336, WeightToNK, ({{4096, 14336, 1, 1}, 2}), ({{1, 1, 1, 1}, 2}), ({{14336, 4096, 1, 1}, 2}))

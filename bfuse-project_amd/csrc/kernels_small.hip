@@ -9,6 +9,7 @@
 #include "ops_gemm_bf16.h"
 #include "ops_gemm_f32.h"
 #include "ops_gemm_f32_dma.h"
+#include "ops_layout.h"
 #include "ops_pool.h"
 #include "ops_rowwise.h"
 
@@ -84,6 +85,10 @@ BFUSE_KERNEL(gemm_bf16_256x320x1792_w8, GemmB5, ({{256, 320, 1, 1}, 2}), ({{1792
 BFUSE_KERNEL(gemm_bf16_256x384x1792_p, GemmB8, ({{256, 384, 1, 1}, 2}), ({{1792, 384, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
 BFUSE_KERNEL(gemm_bf16_256x448x1792_p2, GemmB9, ({{256, 448, 1, 1}, 2}), ({{1792, 448, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
 BFUSE_KERNEL(rmsnorm_rope_bf16_6x1024, NormRopeS, ({{6, 1024, 1, 1}, 2}), ({{(int)NormRopeS::F_BYTES, 1, 1, 1}, 1}), ({{6, 1024, 1, 1}, 2}))
+
+// [128, 192] -> [192, 128], 16-bit elements: 2 x 3 tiles
+using TransposeS = Transpose16<128, 192>;
+BFUSE_KERNEL(transpose16_128x192, TransposeS, ({{128, 192, 1, 1}, 2}), ({{1, 1, 1, 1}, 2}), ({{192, 128, 1, 1}, 2}))
 
 // calibration kernel for the memory counters: 64 MiB read, 64 MiB written
 using Copy64M = CopyF32<16777216, 256>;
