@@ -46,6 +46,9 @@ def test_one_json_line_covering_all_five_pairs():
     ck = rf["same_kernel_constant_operands"]      # the power check: same kernel, operands that toggle no bits
     assert 0 < ck["fused_us"] < d["value"] and abs(ck["frac"] - ck["achieved"] / rf["peak"]) < 1e-3
     assert "same_kernel_constant_operands" not in d["pairs"]["1"]["roofline"]
+    tg = d["target"]          # the 0.9 target of configurations 1-4, stated whether met or not
+    assert sorted(tg["pairs"]) == ["1", "2", "3", "4"] and tg["met"] == all(v <= 0.9 for v in tg["pairs"].values())
+    assert all(len(p["batched_rounds"]["fused_us"]) == len(p["batched_rounds"]["back_to_back_us"]) >= 3 for p in d["pairs"].values())
     cb = d["cpu_baseline"]
     assert cb["kind"] == "port" and cb["cores"] >= 1 and cb["value"] > 0 and cb["sample"]
     for n, p in d["pairs"].items():
