@@ -1,0 +1,194 @@
+"""Suite configuration from the reference's user config: the host-side half of
+scripts/configure_kernels.py (:150-166 get_fusion_info, :229-320 get_test_suite).
+
+The reference reads `FusionSet` (two `Set` lists of operator ids) and `KernelInfo` (id -> argument
+list; the id's prefix names the operator: `dense` = (batch, in, out), `conv2d` = (N, H, W, CO, CI, KH,
+KW, stride, padding), `bgemm` = (batch, M, K, N); :14-38), generates one kernel per id with TVM and
+writes `<out>/cuda/kernels.cu` and `<out>/config/{kernels,fusions,info}.yaml`.  Here kernels are not
+generated: every id is resolved against the library's registry of hand-written gfx950 kernels, whose
+shapes are compile-time, and the same three config files are written for what resolved:
+
+    python -m bfuse_project_amd.configure example.yaml -o OUT [--dtype f32|bf16] [--skip-missing]
+
+  OUT/config/kernels.yaml   id -> {KernelName (registry name), HasBarriers, GridDim, BlockDim, Reg, ExecTime}
+                            in the fuser's schema (horizontal-fuser/include/fuse/Utils.h:70-112); launch shape and
+                            barrier flag are the kernel's own, Reg is the reference's don't-care 32 unless a
+                            device is present
+  OUT/config/fusions.yaml   every (set 0, set 1) pair as {File, Kernels}; File names the library
+  OUT/config/info.yaml      the suite description for `python -m bfuse_project_amd.suite`: the two sets
+                            with registry names, the user's KernelInfo block kept beside them
+  OUT/config/fused.yaml     for every pair, the fused kernels the library holds for it
+
+An id no registry kernel matches is reported with the lines that would instantiate it; the run then
+fails (exit status 1) unless --skip-missing drops such ids from the sets.
+"""
+import argparse
+import os
+import sys
+from typing import Dict, List, Optional, Tuple
+
+import yaml
+
+OPERATORS = ("bgemm", "conv2d", "dense")     # configure_kernels.py:176-187
+
+
+def operator_of(kernel_id: str) -> str:
+    for op in OPERATORS:
+        if kernel_id.startswith(op):
+            return op
+    raise ValueError(f"{kernel_id}: function and schedule with given kernel's name do not exist "
+                     f"(ids start with one of {', '.join(OPERATORS)})")
+
+
+def shapes_of(kernel_id: str, args) -> Tuple[tuple, tuple, tuple]:
+    """(data, weight, output) shapes as the reference computes them (configure_kernels.py:14-38)."""
+    op = operator_of(kernel_id)
+    want = {"dense": 3, "bgemm": 4, "conv2d": 9}[op]
+    if not isinstance(args, (list, tuple)) or len(args) != want or not all(isinstance(a, int) and a >= 0 for a in args):
+        raise ValueError(f"{kernel_id}: {op} takes {want} non-negative integers, got {args!r}")
+    if op == "dense":
+        b, i, o = args
+        return (b, i), (o, i), (b, o)
+    if op == "bgemm":
+        b, m, k, n = args
+        return (b, m, k), (b, n, k), (b, m, n)
+    n, h, w, co, ci, kh, kw, stride, pad = args
+    if stride < 1:
+        raise ValueError(f"{kernel_id}: stride must be at least 1")
+    return (n, ci, h, w), (co, ci, kh, kw), (n, co, (h - kh + 2 * pad) // stride + 1, (w - kw + 2 * pad) // stride + 1)
+
+
+def candidate_names(kernel_id: str, args, dtype: Optional[str]) -> List[str]:
+    """Registry names that implement the operator at exactly these arguments, in order of preference."""
+    op = operator_of(kernel_id)
+    shapes_of(kernel_id, args)   # validates
+    types = [dtype] if dtype else ["f32", "bf16"]
+    if op == "dense":
+        b, i, o = args
+        return [f"gemm_{t}_{b}x{i}x{o}" for t in types]
+    if op == "conv2d":
+        n, h, w, co, ci, kh, kw, stride, pad = args
+        if (n, kh, kw, stride, pad) == (1, 3, 3, 1, 1):
+            return [f"conv3x3_{t}_{ci}x{h}x{w}_{co}" for t in types]
+    return []
+
+
+def instantiation_hint(kernel_id: str, args) -> str:
+    op = operator_of(kernel_id)
+    if op == "dense":
+        b, i, o = args
+        return (f"using Dense = GemmF32Dma<{b}, {o}, {i}, BM, BN, 4>;  BFUSE_KERNEL(gemm_f32_{b}x{i}x{o}, Dense, "
+                f"({{{{{b}, {i}, 1, 1}}, 4}}), ({{{{{i}, {o}, 1, 1}}, 4}}), ({{{{{b}, {o}, 1, 1}}, 4}}))  in csrc/kernels_*.hip")
+    if op == "conv2d":
+        n, h, w, co, ci, kh, kw, stride, pad = args
+        if (n, kh, kw, stride, pad) == (1, 3, 3, 1, 1):
+            return (f"using Conv = Conv3x3F32Lds<{ci}, {co}, {h}, {w}, ...>;  BFUSE_KERNEL(conv3x3_f32_{ci}x{h}x{w}_{co}, Conv, ...)  "
+                    f"in csrc/kernels_*.hip")
+        return "the library's convolution is 3x3, stride 1, padding 1, batch 1 (csrc/ops_conv.h)"
+    return "the library has no batched-GEMM operator"
+
+
+def load_user_config(path: str) -> dict:
+    with open(path) as f:
+        doc = yaml.safe_load(f)
+    if not isinstance(doc, dict) or "FusionSet" not in doc or "KernelInfo" not in doc:
+        raise ValueError("the config needs a FusionSet and a KernelInfo block")
+    sets = doc["FusionSet"]
+    if not isinstance(sets, list) or len(sets) != 2:
+        raise ValueError("Number of fusion sets are only 2.")            # configure_kernels.py:155-157
+    for s in sets:
+        if not isinstance(s, dict) or not isinstance(s.get("Set"), list):
+            raise ValueError("every FusionSet entry needs a 'Set' list")
+        s["Set"] = [k for k in s["Set"] if k is not None]               # the examples ship with one empty item
+        for k in s["Set"]:
+            if k not in doc["KernelInfo"]:
+                raise ValueError(f"{k} is in a fusion set but has no KernelInfo entry")
+    if not isinstance(doc["KernelInfo"], dict):
+        raise ValueError("KernelInfo must map ids to argument lists")
+    return doc
+
+
+def resolve(doc: dict, registry: Dict[str, object], dtype: Optional[str] = None):
+    """({id: registry kernel}, {id: hint}) for every id the two sets name."""
+    found, missing = {}, {}
+    for s in doc["FusionSet"]:
+        for kid in s["Set"]:
+            if kid in found or kid in missing:
+                continue
+            args = doc["KernelInfo"][kid]
+            hit = next((registry[n] for n in candidate_names(kid, args, dtype) if n in registry), None)
+            if hit is not None:
+                found[kid] = hit
+            else:
+                missing[kid] = instantiation_hint(kid, args)
+    return found, missing
+
+
+def configure(path: str, out: str, dtype: Optional[str] = None, skip_missing: bool = False, registry=None) -> dict:
+    """Writes OUT/config/*.yaml and returns {"found", "missing", "pairs", "fused"}."""
+    from . import config as cfg
+    if registry is None:
+        from .operation import list_kernels
+        registry = {k.name: k for k in list_kernels()}
+    doc = load_user_config(path)
+    found, missing = resolve(doc, registry, dtype)
+    if missing and not skip_missing:
+        lines = [f"  {kid} {doc['KernelInfo'][kid]}: {hint}" for kid, hint in missing.items()]
+        raise LookupError("no kernel of the library implements:\n" + "\n".join(lines))
+    sets = [[k for k in s["Set"] if k in found] for s in doc["FusionSet"]]
+    if not sets[0] or not sets[1]:
+        raise LookupError("a fusion set is empty" + (" after dropping the ids the library has no kernel for" if missing else ""))
+    config_dir = os.path.join(out, "config")
+    if os.path.exists(out):
+        raise FileExistsError(f'"{out}" already exists.')                # configure_kernels.py:239-241
+    os.makedirs(config_dir)
+
+    infos = {}
+    for kid, k in found.items():
+        infos[kid] = cfg.KernelInfo(k.name, bool(k.has_barriers), tuple(k.grid), tuple(k.block), k.regs if k.regs > 0 else 32)
+    cfg.dump_kernels_yaml(infos, os.path.join(config_dir, "kernels.yaml"))
+
+    pairs = [(a, b) for a in sets[0] for b in sets[1]]                    # configure_kernels.py:159-163
+    with open(os.path.join(config_dir, "fusions.yaml"), "w") as f:
+        yaml.safe_dump([{"File": "libbfuse_rt.so", "Kernels": [a, b]} for a, b in pairs], f, sort_keys=False)
+
+    fused = {}
+    for a, b in pairs:
+        ka, kb = found[a].name, found[b].name
+        fused[f"{a} + {b}"] = sorted(k.name for k in registry.values() if k.kind in (1, 2, 3) and tuple(k.sides[:2]) == (ka, kb) and k.n_sides == 2)
+    with open(os.path.join(config_dir, "fused.yaml"), "w") as f:
+        yaml.safe_dump(fused, f, sort_keys=False)
+
+    info = {"FusionSet": [{"Set": [found[k].name for k in s]} for s in sets],
+            "KernelInfo": {kid: list(doc["KernelInfo"][kid]) for kid in found},
+            "Resolved": {kid: found[kid].name for kid in found}}
+    with open(os.path.join(config_dir, "info.yaml"), "w") as f:
+        yaml.safe_dump(info, f, sort_keys=False)
+    return {"found": {k: v.name for k, v in found.items()}, "missing": missing, "pairs": pairs, "fused": fused}
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
+    ap.add_argument("config", help="config file path for generate test suite")
+    ap.add_argument("-o", dest="file", default="test-suite", help="output directory of the generated suite configuration")
+    ap.add_argument("--dtype", choices=("f32", "bf16"), default=None, help="arithmetic type of the kernels to resolve to (default: f32, else bf16)")
+    ap.add_argument("--skip-missing", action="store_true", help="drop ids the library has no kernel for instead of failing")
+    args = ap.parse_args(argv)
+    if not os.path.exists(args.config):
+        print(f'Given config path "{args.config}" doesn\'t exist.', file=sys.stderr)
+        return 1
+    try:
+        r = configure(args.config, args.file, args.dtype, args.skip_missing)
+    except (ValueError, LookupError, FileExistsError) as e:
+        print(f"configure: {e}", file=sys.stderr)
+        return 1
+    for kid, name in r["found"].items():
+        print(f"{kid} -> {name}")
+    for kid, hint in r["missing"].items():
+        print(f"{kid}: dropped, no kernel ({hint})", file=sys.stderr)
+    print(f"{len(r['pairs'])} pairs, {sum(1 for v in r['fused'].values() if v)} with a fused kernel; wrote {os.path.join(args.file, 'config')}")
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

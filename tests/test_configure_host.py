@@ -1,0 +1,104 @@
+"""The suite configuration step (the host half of the reference's scripts/configure_kernels.py): operator
+ids of a user config resolve to registry kernels and the fuser's config files come out in its schema."""
+import os
+import subprocess
+import sys
+
+import pytest
+import yaml
+
+import bfuse_project_amd as bf
+from bfuse_project_amd import configure, suite
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+EXAMPLE = os.path.join(ROOT, "bfuse-project_amd", "examples", "baseline_models.yaml")
+REF_EXAMPLES = "/root/reference/test-utils/examples"
+
+
+def test_shapes_follow_the_reference_formulas():
+    # configure_kernels.py:14-38
+    assert configure.shapes_of("dense_1", [512, 768, 3072]) == ((512, 768), (3072, 768), (512, 3072))
+    assert configure.shapes_of("bgemm_0", [12, 512, 64, 512]) == ((12, 512, 64), (12, 512, 64), (12, 512, 512))
+    assert configure.shapes_of("conv2d_0", [1, 224, 224, 64, 3, 7, 7, 2, 3]) == ((1, 3, 224, 224), (64, 3, 7, 7), (1, 64, 112, 112))
+    assert configure.shapes_of("conv2d_1", [1, 56, 56, 64, 64, 3, 3, 1, 1])[2] == (1, 64, 56, 56)
+    with pytest.raises(ValueError):
+        configure.shapes_of("pool_0", [1, 2, 3])
+    with pytest.raises(ValueError):
+        configure.shapes_of("dense_0", [512, 512])
+
+
+def test_example_config_resolves_and_writes_the_fusers_files(tmp_path):
+    out = str(tmp_path / "suite")
+    r = configure.configure(EXAMPLE, out)
+    assert r["found"] == {"dense_0": "gemm_f32_512x512x512", "dense_3": "gemm_f32_512x768x2304",
+                          "conv2d_1": "conv3x3_f32_64x56x56_64", "dense_6": "gemm_bf16_512x4096x14336"}
+    assert r["missing"] == {} and len(r["pairs"]) == 4
+    kernels = bf.load_kernels_yaml(os.path.join(out, "config", "kernels.yaml"))      # the fuser's schema loads it
+    fusions = bf.load_fusions_yaml(os.path.join(out, "config", "fusions.yaml"))
+    assert kernels["dense_3"].KernelName == "gemm_f32_512x768x2304" and kernels["dense_3"].GridDim == (256, 1, 1)
+    assert kernels["dense_6"].BlockDim == (640, 1, 1) and kernels["dense_6"].HasBarriers is True
+    assert [f.Kernels for f in fusions] == [["dense_0", "conv2d_1"], ["dense_0", "dense_6"], ["dense_3", "conv2d_1"], ["dense_3", "dense_6"]]
+    # the block-fusion context of the reference's live pattern over two resolved kernels
+    ctx = bf.FusionContext.create(fusions[2], kernels, bfuse=True)
+    assert ctx.fused_kernel_info().GridDim == (256 + 196, 1, 1)
+    # the suite driver takes the info.yaml as it is
+    info = suite.load_info(os.path.join(out, "config", "info.yaml"))
+    assert suite.set_names(info) == (["gemm_f32_512x512x512", "gemm_f32_512x768x2304"], ["conv3x3_f32_64x56x56_64", "gemm_bf16_512x4096x14336"])
+    with open(os.path.join(out, "config", "fused.yaml")) as f:
+        fused = yaml.safe_load(f)
+    assert set(fused) == {"dense_0 + conv2d_1", "dense_0 + dense_6", "dense_3 + conv2d_1", "dense_3 + dense_6"}
+    with pytest.raises(FileExistsError):
+        configure.configure(EXAMPLE, out)
+
+
+def test_unknown_shapes_are_reported_with_the_line_that_would_add_them(tmp_path):
+    cfg = tmp_path / "c.yaml"
+    cfg.write_text("FusionSet:\n  - Set: [dense_0, dense_9]\n  - Set: [conv2d_0, conv2d_1, bgemm_0]\n"
+                   "KernelInfo:\n  dense_0: [512, 512, 512]\n  dense_9: [512, 100, 100]\n  conv2d_0: [1, 224, 224, 64, 3, 7, 7, 2, 3]\n"
+                   "  conv2d_1: [1, 56, 56, 64, 64, 3, 3, 1, 1]\n  bgemm_0: [12, 512, 64, 512]\n")
+    with pytest.raises(LookupError) as e:
+        configure.configure(str(cfg), str(tmp_path / "a"))
+    assert "dense_9" in str(e.value) and "gemm_f32_512x100x100" in str(e.value) and "bgemm_0" in str(e.value) and not (tmp_path / "a").exists()
+    r = configure.configure(str(cfg), str(tmp_path / "b"), skip_missing=True)
+    assert r["found"] == {"dense_0": "gemm_f32_512x512x512", "conv2d_1": "conv3x3_f32_64x56x56_64"} and sorted(r["missing"]) == ["bgemm_0", "conv2d_0", "dense_9"]
+    assert r["pairs"] == [("dense_0", "conv2d_1")]
+    # the bf16 kernel only when asked for, or when there is no fp32 one
+    r2 = configure.configure(EXAMPLE, str(tmp_path / "c2"), dtype="f32", skip_missing=True)
+    assert "dense_6" in r2["missing"] and r2["found"]["dense_3"] == "gemm_f32_512x768x2304"
+
+
+def test_malformed_configs_are_refused(tmp_path):
+    for text in ("KernelInfo: {}\n", "FusionSet: [{Set: [a]}]\nKernelInfo: {a: [1, 2, 3]}\n",
+                 "FusionSet: [{Set: [dense_0]}, {Set: [dense_1]}]\nKernelInfo: {dense_0: [1, 2, 3]}\n"):
+        p = tmp_path / "bad.yaml"
+        p.write_text(text)
+        with pytest.raises(ValueError):
+            configure.load_user_config(str(p))
+
+
+def test_command_line(tmp_path):
+    out = str(tmp_path / "cli")
+    r = subprocess.run([sys.executable, "-m", "bfuse_project_amd.configure", EXAMPLE, "-o", out], capture_output=True, text=True, cwd=ROOT)
+    assert r.returncode == 0 and "dense_6 -> gemm_bf16_512x4096x14336" in r.stdout and os.path.exists(os.path.join(out, "config", "kernels.yaml"))
+    r = subprocess.run([sys.executable, "-m", "bfuse_project_amd.configure", os.path.join(out, "nope.yaml")], capture_output=True, text=True, cwd=ROOT)
+    assert r.returncode == 1 and "doesn't exist" in r.stderr
+
+
+@pytest.mark.skipif(not os.path.isdir(REF_EXAMPLES), reason="the reference's example configs are not on this machine")
+@pytest.mark.parametrize("name,want", [("llm.yaml", {"dense_3": "gemm_f32_512x768x2304", "dense_6": "gemm_bf16_512x4096x14336"}),
+                                       ("resnet-18.yaml", {"conv2d_1": "conv3x3_f32_64x56x56_64"})])
+def test_the_references_own_example_configs(tmp_path, name, want):
+    """The reference's examples (read in place) ship with empty fusion sets: every id goes into both
+    sets, as its benchmark.yaml does, and the ids of the benchmark configurations resolve."""
+    with open(os.path.join(REF_EXAMPLES, name)) as f:
+        doc = yaml.safe_load(f)
+    ids = list(doc["KernelInfo"])
+    doc["FusionSet"] = [{"Set": ids}, {"Set": ids}]
+    p = tmp_path / name
+    p.write_text(yaml.safe_dump(doc))
+    for kid in ids:
+        configure.shapes_of(kid, doc["KernelInfo"][kid])          # every entry is well formed
+    r = configure.configure(str(p), str(tmp_path / "o"), skip_missing=True)
+    for kid, kname in want.items():
+        assert r["found"][kid] == kname
+    assert set(r["found"]) | set(r["missing"]) == set(ids)

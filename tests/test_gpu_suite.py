@@ -29,3 +29,21 @@ def test_small_matrix(tmp_path):
     # the traces hold the warm-ups too; the analysis drops them
     assert len(suite.read_trace(str(tmp_path / "exec" / "0_0_0.csv"))) == suite.WARMUP_TRIALS + suite.TIMED_TRIALS
     print(suite.to_markdown(rows))
+
+
+def test_from_a_user_config_to_the_speed_up_table(tmp_path):
+    """The reference's front door end to end: operator ids and shapes in, resolved against the registry
+    (configure), the pair matrix run and tabulated (suite)."""
+    from bfuse_project_amd import configure
+    cfg = tmp_path / "models.yaml"
+    cfg.write_text("FusionSet:\n  - Set: [dense_3]\n  - Set: [conv2d_1, dense_0]\n"
+                   "KernelInfo:\n  dense_3: [512, 768, 2304]\n  dense_0: [512, 512, 512]\n  conv2d_1: [1, 56, 56, 64, 64, 3, 3, 1, 1]\n")
+    out = tmp_path / "suite"
+    r = configure.configure(str(cfg), str(out))
+    assert r["found"]["dense_3"] == "gemm_f32_512x768x2304"
+    info = suite.load_info(str(out / "config" / "info.yaml"))
+    print("suite from a user config", flush=True)
+    rows = suite.run_suite(info, str(out / "run"), validate=True, log=lambda m: print(m, flush=True))
+    assert [(x["kernel1"], x["kernel2"]) for x in rows] == [("gemm_f32_512x768x2304", "conv3x3_f32_64x56x56_64"),
+                                                             ("gemm_f32_512x768x2304", "gemm_f32_512x512x512")]
+    assert all(x["serial_ns"] > 0 and x["parallel_ns"] > 0 for x in rows)
