@@ -47,3 +47,20 @@ def test_from_a_user_config_to_the_speed_up_table(tmp_path):
     assert [(x["kernel1"], x["kernel2"]) for x in rows] == [("gemm_f32_512x768x2304", "conv3x3_f32_64x56x56_64"),
                                                              ("gemm_f32_512x768x2304", "gemm_f32_512x512x512")]
     assert all(x["serial_ns"] > 0 and x["parallel_ns"] > 0 for x in rows)
+
+
+def test_quick_start_command(tmp_path):
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cfg = tmp_path / "m.yaml"
+    cfg.write_text("FusionSet:\n  - Set: [dense_3]\n  - Set: [conv2d_1]\nKernelInfo:\n  dense_3: [512, 768, 2304]\n  conv2d_1: [1, 56, 56, 64, 64, 3, 3, 1, 1]\n")
+    out = tmp_path / "qs"
+    print("quick_start", flush=True)
+    r = subprocess.run([sys.executable, "-m", "bfuse_project_amd.quick_start", str(cfg), "-o", str(out)], capture_output=True, text=True, cwd=root, timeout=120)
+    assert r.returncode == 0, r.stdout[-1500:] + r.stderr[-1500:]
+    assert "[1/3]" in r.stdout and "[3/3]" in r.stdout and "gemm_f32_512x768x2304" in r.stdout
+    assert os.path.exists(out / "summary.md") and os.path.exists(out / "config" / "kernels.yaml") and os.path.exists(out / "exec" / "2_0_0.csv")
+    # a second run into the same directory is refused, as the reference's configure step refuses it
+    r = subprocess.run([sys.executable, "-m", "bfuse_project_amd.quick_start", str(cfg), "-o", str(out)], capture_output=True, text=True, cwd=root, timeout=120)
+    assert r.returncode == 1 and "already exists" in r.stderr
