@@ -1,0 +1,32 @@
+// Further dense layers of the reference's example models (test-utils/examples/llm.yaml:7-41), beyond the
+// ones the five benchmark configurations use: the same fp32 GEMM template at other shapes, so that the ids
+// of that file resolve to kernels of the library (bfuse_project_amd.configure).  Tiles are chosen as one per
+// CU (256 workgroups) where the shape allows it.
+#include "fuse.h"
+#include "ops_gemm_f32_dma.h"
+#include "ops_rowwise.h"
+
+using namespace bfuse;
+
+BFUSE_MODULE_PROLOGUE()
+
+// dense_0: BERT attention output projection, [512 x 768] . [768 x 768]: 16 x 16 tiles of 32 x 48
+using Dense0 = GemmF32Dma<512, 768, 768, 32, 48, 4>;
+// dense_1: BERT / GPT-2 MLP up-projection without the activation, [512 x 768] . [768 x 3072]: pair 4's tiling
+using Dense1 = GemmF32Dma<512, 3072, 768, 32, 96, 4, kEpiNone, 2>;
+// dense_2: MLP down-projection, [512 x 3072] . [3072 x 768]
+using Dense2 = GemmF32Dma<512, 768, 3072, 32, 48, 4>;
+// dense_5: Llama-3-8B key / value projection, [512 x 4096] . [4096 x 1024]: 16 x 16 tiles of 32 x 64
+using Dense5 = GemmF32Dma<512, 1024, 4096, 32, 64, 4>;
+
+BFUSE_KERNEL(gemm_f32_512x768x768, Dense0, ({{512, 768, 1, 1}, 4}), ({{768, 768, 1, 1}, 4}), ({{512, 768, 1, 1}, 4}))
+BFUSE_KERNEL(gemm_f32_512x768x3072, Dense1, ({{512, 768, 1, 1}, 4}), ({{768, 3072, 1, 1}, 4}), ({{512, 3072, 1, 1}, 4}))
+BFUSE_KERNEL(gemm_f32_512x3072x768, Dense2, ({{512, 3072, 1, 1}, 4}), ({{3072, 768, 1, 1}, 4}), ({{512, 768, 1, 1}, 4}))
+BFUSE_KERNEL(gemm_f32_512x4096x1024, Dense5, ({{512, 4096, 1, 1}, 4}), ({{4096, 1024, 1, 1}, 4}), ({{512, 1024, 1, 1}, 4}))
+
+// each with the LayerNorm of pair 2 as its memory-bound partner, block-fused one chunk per round over the CUs
+using LayerNormW1 = LayerNorm<512, 768, 1, 1>;
+BFUSE_BFUSE_KERNEL(gemm_f32_512x768x768, Dense0, layernorm_512x768, LayerNormW1, _c256, bfuse::kChunked, 256, 1)
+BFUSE_BFUSE_KERNEL(gemm_f32_512x768x3072, Dense1, layernorm_512x768, LayerNormW1, _c256, bfuse::kChunked, 256, 1)
+BFUSE_BFUSE_KERNEL(gemm_f32_512x3072x768, Dense2, layernorm_512x768, LayerNormW1, _c256, bfuse::kChunked, 256, 1)
+BFUSE_BFUSE_KERNEL(gemm_f32_512x4096x1024, Dense5, layernorm_512x768, LayerNormW1, _c256, bfuse::kChunked, 256, 1)
