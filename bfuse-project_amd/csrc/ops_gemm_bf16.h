@@ -77,10 +77,11 @@ struct GemmBf16NTDma {
     static_assert(TM == 2 || TM == 4, "the hand-written LDS wait lists two or four A fragments");
     static_assert(OCHUNKS % CTHREADS == 0 && NSTG >= 2 && NSTG <= 4 && NKT >= NSTG - 1, "pipeline shape");
     static_assert(PD_ >= 1 && PD_ < (BK / 32) * (BN / WGN_ / 16), "read-ahead distance");
-    // the hand-written wait counts (allowed()) assume that the next substep's A fragments, requested after
-    // group ks*TN+1, are waited for by a later group of the same substep: with fewer than three column blocks
-    // per wave they are not (the build's check of the assembly finds the MFMAs that would read them early)
-    static_assert(BN / WGN_ / 16 >= 3, "a wave needs at least three 16-column blocks");
+    // the hand-written wait counts (allowed()) count the next substep's A fragments, requested after group
+    // ks*TN+1, as reads that may still be in flight for the PD groups that follow: the substep must be
+    // longer than that, or its successor's first group would use them unwaited (the build's check of the
+    // assembly finds such MFMAs: seen with TN = 2 and with TN = PD = 4)
+    static_assert(BN / WGN_ / 16 > PD_ + 1, "column blocks per wave must exceed the read-ahead distance + 1");
     static constexpr int MT = M / BM, NT = N / BN;
     static_assert((MT * NT) % 8 == 0 && NT % 8 == 0, "tiles are dealt to 8 XCDs");
 
