@@ -1,8 +1,9 @@
 // Further dense layers of the reference's example models (test-utils/examples/llm.yaml:7-41), beyond the
-// ones the five benchmark configurations use: the same fp32 GEMM template at other shapes, so that the ids
+// ones the five benchmark configurations use: the same fp32 and bf16 GEMM templates at other shapes, so that the ids
 // of that file resolve to kernels of the library (bfuse_project_amd.configure).  Tiles are chosen as one per
 // CU (256 workgroups) where the shape allows it.
 #include "fuse.h"
+#include "ops_gemm_bf16.h"
 #include "ops_gemm_f32_dma.h"
 #include "ops_rowwise.h"
 
@@ -30,3 +31,17 @@ BFUSE_BFUSE_KERNEL(gemm_f32_512x768x768, Dense0, layernorm_512x768, LayerNormW1,
 BFUSE_BFUSE_KERNEL(gemm_f32_512x768x3072, Dense1, layernorm_512x768, LayerNormW1, _c256, bfuse::kChunked, 256, 1)
 BFUSE_BFUSE_KERNEL(gemm_f32_512x3072x768, Dense2, layernorm_512x768, LayerNormW1, _c256, bfuse::kChunked, 256, 1)
 BFUSE_BFUSE_KERNEL(gemm_f32_512x4096x1024, Dense5, layernorm_512x768, LayerNormW1, _c256, bfuse::kChunked, 256, 1)
+
+// Llama-3-8B, bf16 as pair 5's GEMM, weights [N, K]: dense_4 (query / output projection,
+// [512 x 4096] . [4096 x 4096]^T) and dense_7 (MLP down-projection, [512 x 14336] . [4096 x 14336]^T).
+// N = 4096 over 256 CUs leaves each a 64 x 128 tile: four compute waves (2 x 2) of 32 x 64 and two
+// producer waves, ring of three 64-k stages (72 KB), read-ahead of two fragments, the next step's barrier
+// before MFMA group 6 of 8.
+using Dense4 = GemmBf16NTDma<512, 4096, 4096, 64, 128, 3, 2, 2, 2, 2, 6>;
+using Dense7 = GemmBf16NTDma<512, 4096, 14336, 64, 128, 3, 2, 2, 2, 2, 6>;
+BFUSE_KERNEL(gemm_bf16_512x4096x4096, Dense4, ({{512, 4096, 1, 1}, 2}), ({{4096, 4096, 1, 1}, 2}), ({{512, 4096, 1, 1}, 2}))
+BFUSE_KERNEL(gemm_bf16_512x14336x4096, Dense7, ({{512, 14336, 1, 1}, 2}), ({{4096, 14336, 1, 1}, 2}), ({{512, 4096, 1, 1}, 2}))
+// each with pair 5's RMSNorm + RoPE side (one row per one-wave workgroup), block-fused one chunk per round
+using NormRopeW1 = RmsNormRope<512, 32, 128, 1>;
+BFUSE_BFUSE_KERNEL(gemm_bf16_512x4096x4096, Dense4, rmsnorm_rope_bf16_512x4096, NormRopeW1, _c256, bfuse::kChunked, 256, 1)
+BFUSE_BFUSE_KERNEL(gemm_bf16_512x14336x4096, Dense7, rmsnorm_rope_bf16_512x4096, NormRopeW1, _c256, bfuse::kChunked, 256, 1)

@@ -64,6 +64,7 @@ using GemmB3 = GemmBf16NTDma<256, 1792, 320, 128, 224, 3>;            // two M-t
 using GemmB5 = GemmBf16NTDma<256, 1792, 320, 128, 224, 3, 4, 4, 2>;   // the same with eight waves (uneven load groups per wave)
 using GemmB8 = GemmBf16NTDma<256, 1792, 384, 128, 224, 3, 4, 4, 2, 4, 11>;   // eight compute + four producer waves, early barrier, six K-steps (all after the rolled loop)
 using GemmB9 = GemmBf16NTDma<256, 1792, 448, 128, 224, 3, 4, 4, 2, 2, 10>;   // eight compute + two producer waves, early barrier, seven K-steps (one round of the rolled loop, then the last step)
+using GemmB11 = GemmBf16NTDma<128, 1024, 320, 64, 128, 3, 2, 2, 2, 2, 6>;   // 64 x 128 tiles, four compute waves (2 x 2) of 32 x 64 + two producer waves, read-ahead of two, early barrier
 using NormRopeS = RmsNormRope<6, 8, 128, 2>;
 
 BFUSE_KERNEL(gemm_f32_64x32x48, GemmS1, ({{64, 32, 1, 1}, 4}), ({{32, 48, 1, 1}, 4}), ({{64, 48, 1, 1}, 4}))
@@ -84,6 +85,7 @@ BFUSE_KERNEL(gemm_bf16_256x320x1792, GemmB3, ({{256, 320, 1, 1}, 2}), ({{1792, 3
 BFUSE_KERNEL(gemm_bf16_256x320x1792_w8, GemmB5, ({{256, 320, 1, 1}, 2}), ({{1792, 320, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
 BFUSE_KERNEL(gemm_bf16_256x384x1792_p, GemmB8, ({{256, 384, 1, 1}, 2}), ({{1792, 384, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
 BFUSE_KERNEL(gemm_bf16_256x448x1792_p2, GemmB9, ({{256, 448, 1, 1}, 2}), ({{1792, 448, 1, 1}, 2}), ({{256, 1792, 1, 1}, 2}))
+BFUSE_KERNEL(gemm_bf16_128x320x1024_t64, GemmB11, ({{128, 320, 1, 1}, 2}), ({{1024, 320, 1, 1}, 2}), ({{128, 1024, 1, 1}, 2}))
 BFUSE_KERNEL(rmsnorm_rope_bf16_6x1024, NormRopeS, ({{6, 1024, 1, 1}, 2}), ({{(int)NormRopeS::F_BYTES, 1, 1, 1}, 1}), ({{6, 1024, 1, 1}, 2}))
 
 // [128, 192] -> [192, 128], 16-bit elements: 2 x 3 tiles

@@ -39,3 +39,40 @@ def test_dense_layer_against_the_oracle_and_fused_with_layernorm(kid, m, k, n):
           f"GEMM {t_g:.1f} us = {2.0 * m * n * k / t_g * 1e-6:.1f} TFLOP/s, fused with LayerNorm {t_f:.1f} us", flush=True)
     assert st["n_fail"] == 0
     assert oracle_cases.rel_error(y, orf.layernorm(x.reshape(512, 768), gb[:768], gb[768:], 1e-12)) <= 1e-5
+
+
+@pytest.mark.parametrize("kid,m,k,n", [("dense_4", 512, 4096, 4096), ("dense_7", 512, 14336, 4096)])
+def test_llama_bf16_dense_layer_against_the_oracle_and_fused_with_rmsnorm_rope(kid, m, k, n):
+    """bf16 in, fp32 accumulate, bf16 out, weight [N, K]: a strided 64 x 512 sample of the outputs over
+    the full K against the oracle (1e-2), selector inputs that hit every output element exactly, and the
+    kernel block-fused with RMSNorm + RoPE bit-exact against the two kernels launched back to back."""
+    from bfuse_project_amd.operation import f32_to_bf16, bf16_to_f32
+    from bfuse_project_amd.workloads import PAIRS
+    name = f"gemm_bf16_{m}x{k}x{n}"
+    print(f"[models] {kid} -> {name}", flush=True)
+    a = f32_to_bf16(fill_normal(0xA0 + k, m * k, 0.0, 1.0))
+    w = f32_to_bf16(fill_normal(0xB0 + k, n * k, 0.0, 0.02))
+    _, _, x, f2 = PAIRS[5].inputs()
+    with bf.Operation(name, "rmsnorm_rope_bf16_512x4096") as op:
+        c = op.run_kernel(0, a, w)
+        y = op.run_kernel(1, x, f2)
+        fused = op.fused("bfuse", "_c256")
+        q1, q2 = op.run_fuse(fused, a, w, x, f2)
+        # selector inputs: A[r, :] has a single 1 at k = r mod K, so C[r, j] = W[j, r mod K] exactly
+        sel = np.zeros((m, k), np.float32)
+        sel[np.arange(m), (np.arange(m) * 37) % k] = 1.0
+        cs = op.run_kernel(0, f32_to_bf16(sel.ravel()), w)
+        op.upload(0, a, w)
+        op.upload(1, x, f2)
+        t_g = float(np.mean(op.time("kernel1", warmup=10, reps=50)[0]))
+        t_f = float(np.mean(op.time("bfuse", fused, warmup=10, reps=50)[0]))
+    assert q1.tobytes() == c.tobytes() and q2.tobytes() == y.tobytes(), "fused output differs from the unfused kernels"
+    W = w.reshape(n, k)
+    assert np.array_equal(cs.reshape(m, n), W[:, (np.arange(m) * 37) % k].T), "selector inputs: an output element is not the weight it selects"
+    rows, cols = np.arange(3, m, 8), np.arange(5, n, 8)
+    want = orf.gemm_bf16(np.ascontiguousarray(a.reshape(m, k)[rows]), np.ascontiguousarray(W[cols]), b_is_nk=True)
+    got = np.ascontiguousarray(c.reshape(m, n)[np.ix_(rows, cols)])
+    e = oracle_cases.rel_error(bf16_to_f32(got).ravel(), bf16_to_f32(want).ravel())
+    print(f"[parity] {name}: sample {len(rows)} x {len(cols)} over K = {k}: max rel err {e:.3e}; "
+          f"GEMM {t_g:.1f} us = {2.0 * m * n * k / t_g * 1e-6:.0f} TFLOP/s, fused with RMSNorm+RoPE {t_f:.1f} us", flush=True)
+    assert e <= 1e-2

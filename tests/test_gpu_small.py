@@ -69,6 +69,8 @@ def _cases():
                                      lambda I, F: orf.gemm_bf16(I.reshape(256, 384), F.reshape(1792, 384), b_is_nk=True), 1e-2, True),
         "gemm_bf16_256x448x1792_p2": (lambda s: (f32_to_bf16(fill_normal(s, 256 * 448, 0, 1)), f32_to_bf16(fill_normal(s + 1, 1792 * 448, 0, 0.1))),
                                       lambda I, F: orf.gemm_bf16(I.reshape(256, 448), F.reshape(1792, 448), b_is_nk=True), 1e-2, True),
+        "gemm_bf16_128x320x1024_t64": (lambda s: (f32_to_bf16(fill_normal(s, 128 * 320, 0, 1)), f32_to_bf16(fill_normal(s + 1, 1024 * 320, 0, 0.1))),
+                                       lambda I, F: orf.gemm_bf16(I.reshape(128, 320), F.reshape(1024, 320), b_is_nk=True), 1e-2, True),
         "rmsnorm_rope_bf16_6x1024": (lambda s: (f32_to_bf16(fill_normal(s, 6 * 1024, 0, 1.5)), _norm_rope_operand(6, 1024, 128, s + 1)),
                                      lambda I, F: orf.rmsnorm_rope_bf16(I.reshape(6, 1024), *wl.unpack_norm_rope_operand(F, 6, 1024, 128), heads=8, eps=1e-5), 1e-2, True),
     }
