@@ -3,6 +3,7 @@
 // of that file resolve to kernels of the library (bfuse_project_amd.configure).  Tiles are chosen as one per
 // CU (256 workgroups) where the shape allows it.
 #include "fuse.h"
+#include "ops_conv.h"
 #include "ops_gemm_bf16.h"
 #include "ops_gemm_f32_dma.h"
 #include "ops_rowwise.h"
@@ -45,3 +46,10 @@ BFUSE_KERNEL(gemm_bf16_512x14336x4096, Dense7, ({{512, 14336, 1, 1}, 2}), ({{409
 using NormRopeW1 = RmsNormRope<512, 32, 128, 1>;
 BFUSE_BFUSE_KERNEL(gemm_bf16_512x4096x4096, Dense4, rmsnorm_rope_bf16_512x4096, NormRopeW1, _c256, bfuse::kChunked, 256, 1)
 BFUSE_BFUSE_KERNEL(gemm_bf16_512x14336x4096, Dense7, rmsnorm_rope_bf16_512x4096, NormRopeW1, _c256, bfuse::kChunked, 256, 1)
+
+// ResNet-18 (test-utils/examples/resnet-18.yaml): conv2d_4, the second 3x3 / stride 1 / padding 1 convolution the
+// template's row alignment allows (128 -> 128 channels on 28 x 28): 32 output channels x 16 pixels per workgroup,
+// four waves take two 16-channel groups each, 49 x 4 = 196 workgroups
+using Conv128 = Conv3x3F32Lds<128, 128, 28, 28, 32, 1, 4>;
+BFUSE_KERNEL(conv3x3_f32_128x28x28_128, Conv128, ({{1, 128, 28, 28}, 4}), ({{128, 128, 3, 3}, 4}), ({{1, 128, 28, 28}, 4}))
+BFUSE_BFUSE_KERNEL(conv3x3_f32_128x28x28_128, Conv128, layernorm_512x768, LayerNormW1, _c256, bfuse::kChunked, 256, 1)

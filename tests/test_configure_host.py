@@ -88,7 +88,7 @@ def test_command_line(tmp_path):
 @pytest.mark.parametrize("name,want", [("llm.yaml", {"dense_0": "gemm_f32_512x768x768", "dense_1": "gemm_f32_512x768x3072", "dense_2": "gemm_f32_512x3072x768",
                                                      "dense_3": "gemm_f32_512x768x2304", "dense_4": "gemm_bf16_512x4096x4096", "dense_5": "gemm_f32_512x4096x1024",
                                                      "dense_6": "gemm_bf16_512x4096x14336", "dense_7": "gemm_bf16_512x14336x4096"}),
-                                       ("resnet-18.yaml", {"conv2d_1": "conv3x3_f32_64x56x56_64"})])
+                                       ("resnet-18.yaml", {"conv2d_1": "conv3x3_f32_64x56x56_64", "conv2d_4": "conv3x3_f32_128x28x28_128"})])
 def test_the_references_own_example_configs(tmp_path, name, want):
     """The reference's examples (read in place) ship with empty fusion sets: every id goes into both
     sets, as its benchmark.yaml does, and the ids of the benchmark configurations resolve."""

@@ -76,3 +76,24 @@ def test_llama_bf16_dense_layer_against_the_oracle_and_fused_with_rmsnorm_rope(k
     print(f"[parity] {name}: sample {len(rows)} x {len(cols)} over K = {k}: max rel err {e:.3e}; "
           f"GEMM {t_g:.1f} us = {2.0 * m * n * k / t_g * 1e-6:.0f} TFLOP/s, fused with RMSNorm+RoPE {t_f:.1f} us", flush=True)
     assert e <= 1e-2
+
+
+def test_resnet_conv2d_4_against_the_oracle_and_fused_with_layernorm():
+    """conv2d_4 of the reference's resnet-18.yaml: 3x3, stride 1, padding 1, 128 -> 128 channels on 28 x 28."""
+    name = "conv3x3_f32_128x28x28_128"
+    print(f"[models] conv2d_4 -> {name}", flush=True)
+    xin = np.maximum(fill_normal(0xC4, 128 * 28 * 28, 0.0, 1.0), 0.0)
+    w = fill_normal(0xC5, 128 * 128 * 9, 0.0, 0.05)
+    x = fill_normal(0xF0, 512 * 768, 0.0, 1.0)
+    gb = np.concatenate([fill_normal(0xF1, 768, 1.0, 0.1), fill_normal(0xF2, 768, 0.0, 0.1)])
+    with bf.Operation(name, "layernorm_512x768") as op:
+        c = op.run_kernel(0, xin, w)
+        y = op.run_kernel(1, x, gb)
+        q1, q2 = op.run_fuse(op.fused("bfuse", "_c256"), xin, w, x, gb)
+        op.upload(0, xin, w)
+        t = float(np.mean(op.time("kernel1", warmup=10, reps=50)[0]))
+    assert q1.tobytes() == c.tobytes() and q2.tobytes() == y.tobytes(), "fused output differs from the unfused kernels"
+    want = orf.conv2d(xin.reshape(1, 128, 28, 28), w.reshape(128, 128, 3, 3), s=1, p=1)
+    st = oracle_cases.rel_stats(c, want, 1e-5)
+    print(f"[parity] {name}: worst |d|/max(|ref|,rms) {st['worst_floor_rel']:.3e}; {st['n_fail']} fail; {t:.1f} us", flush=True)
+    assert st["n_fail"] == 0
