@@ -70,7 +70,9 @@ def candidate_names(kernel_id: str, args, dtype: Optional[str]) -> List[str]:
         n, h, w, co, ci, kh, kw, stride, pad = args
         if (n, kh, kw, stride, pad) == (1, 3, 3, 1, 1):
             return [f"conv3x3_{t}_{ci}x{h}x{w}_{co}" for t in types]
-    return []
+        return []
+    b, m, k, n = args
+    return [f"bgemm_{t}_{b}x{m}x{k}x{n}" for t in types]
 
 
 def instantiation_hint(kernel_id: str, args) -> str:
@@ -85,7 +87,9 @@ def instantiation_hint(kernel_id: str, args) -> str:
             return (f"using Conv = Conv3x3F32Lds<{ci}, {co}, {h}, {w}, ...>;  BFUSE_KERNEL(conv3x3_f32_{ci}x{h}x{w}_{co}, Conv, ...)  "
                     f"in csrc/kernels_*.hip")
         return "the library's convolution is 3x3, stride 1, padding 1, batch 1 (csrc/ops_conv.h)"
-    return "the library has no batched-GEMM operator"
+    b, m, k, n = args
+    return (f"using Bgemm = GemmF32<{m}, {n}, {k}, BM, BN, KS, kEpiNone, 2, 1, true, {b}>;  BFUSE_KERNEL(bgemm_f32_{b}x{m}x{k}x{n}, Bgemm, "
+            f"({{{{{b}, {m}, {k}, 1}}, 4}}), ({{{{{b}, {n}, {k}, 1}}, 4}}), ({{{{{b}, {m}, {n}, 1}}, 4}}))  in csrc/kernels_*.hip")
 
 
 def load_user_config(path: str) -> dict:

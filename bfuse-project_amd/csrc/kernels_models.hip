@@ -5,6 +5,7 @@
 #include "fuse.h"
 #include "ops_conv.h"
 #include "ops_gemm_bf16.h"
+#include "ops_gemm_f32.h"
 #include "ops_gemm_f32_dma.h"
 #include "ops_rowwise.h"
 
@@ -53,3 +54,22 @@ BFUSE_BFUSE_KERNEL(gemm_bf16_512x14336x4096, Dense7, rmsnorm_rope_bf16_512x4096,
 using Conv128 = Conv3x3F32Lds<128, 128, 28, 28, 32, 1, 4>;
 BFUSE_KERNEL(conv3x3_f32_128x28x28_128, Conv128, ({{1, 128, 28, 28}, 4}), ({{128, 128, 3, 3}, 4}), ({{1, 128, 28, 28}, 4}))
 BFUSE_BFUSE_KERNEL(conv3x3_f32_128x28x28_128, Conv128, layernorm_512x768, LayerNormW1, _c256, bfuse::kChunked, 256, 1)
+
+// Batched GEMMs of the attention layers (the reference's bgemm, scripts/configure_kernels.py:14-19,40-48:
+// C[b] = A[b] . B[b]^T with A [b, M, K] and B [b, N, K]): bgemm_0 / bgemm_1 are BERT's and GPT-2's scores and
+// context products (12 heads, sequence 512, head size 64), bgemm_2 / bgemm_3 Llama-3-8B's (32 heads, head size 128).
+// Operands go global -> VGPR in MFMA layout (both are contiguous along K); a short reduction (K = 64, 128) is
+// one wave's, a long one (K = 512) is split over two.
+using Bgemm0 = GemmF32<512, 512, 64, 32, 64, 1, kEpiNone, 2, 1, true, 12>;     // 16 x 8 tiles x 12 = 1536 one-wave workgroups
+using Bgemm1 = GemmF32<512, 64, 512, 16, 64, 2, kEpiNone, 2, 1, true, 12>;     // 32 x 1 tiles x 12 = 384 two-wave workgroups
+using Bgemm2 = GemmF32<512, 512, 128, 32, 64, 1, kEpiNone, 2, 1, true, 32>;    // 4096 one-wave workgroups
+using Bgemm3 = GemmF32<512, 128, 512, 32, 64, 2, kEpiNone, 2, 1, true, 32>;    // 16 x 2 tiles x 32 = 1024 two-wave workgroups
+BFUSE_KERNEL(bgemm_f32_12x512x64x512, Bgemm0, ({{12, 512, 64, 1}, 4}), ({{12, 512, 64, 1}, 4}), ({{12, 512, 512, 1}, 4}))
+BFUSE_KERNEL(bgemm_f32_12x512x512x64, Bgemm1, ({{12, 512, 512, 1}, 4}), ({{12, 64, 512, 1}, 4}), ({{12, 512, 64, 1}, 4}))
+BFUSE_KERNEL(bgemm_f32_32x512x128x512, Bgemm2, ({{32, 512, 128, 1}, 4}), ({{32, 512, 128, 1}, 4}), ({{32, 512, 512, 1}, 4}))
+BFUSE_KERNEL(bgemm_f32_32x512x512x128, Bgemm3, ({{32, 512, 512, 1}, 4}), ({{32, 128, 512, 1}, 4}), ({{32, 512, 128, 1}, 4}))
+// the scores product of BERT / GPT-2 with the causal softmax that follows it in the model as its partner,
+// and with the LayerNorm
+using Softmax4W = SoftmaxCausal<12, 512, 4, 1>;
+BFUSE_BFUSE_KERNEL(bgemm_f32_12x512x64x512, Bgemm0, softmax_causal_12x512x512, Softmax4W, _c256, bfuse::kChunked, 256, 1)
+BFUSE_BFUSE_KERNEL(bgemm_f32_12x512x512x64, Bgemm1, layernorm_512x768, LayerNormW1, _c256, bfuse::kChunked, 256, 1)

@@ -50,8 +50,16 @@ __device__ __forceinline__ float gelu_tanh(float x)
     return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 
-template <int M_, int N_, int K_, int BM_, int BN_, int KS_, int EPI_ = kEpiNone, int NBUF_ = 2, int SCHED_ = 1>
+// B_NK_: the second operand is stored [N, K] (the reference's `dense` / `batch_matmul` layout, both operands
+// contiguous along K): a lane then loads, for each of its four columns 4j+e, the four k it needs with ONE
+// 128-bit load (component t is MFMA step t) where the [K, N] layout gives it, for each k-step t, four columns
+// with one load -- the same number of loads and registers, indexed the other way round.
+// BATCH_ > 1: BATCH_ independent products A[b] . B[b] of the same shape (the reference's bgemm,
+// scripts/configure_kernels.py:14-19,40-48); workgroup v works on batch v / tiles, tile v % tiles.
+template <int M_, int N_, int K_, int BM_, int BN_, int KS_, int EPI_ = kEpiNone, int NBUF_ = 2, int SCHED_ = 1, bool B_NK_ = false, int BATCH_ = 1>
 struct GemmF32 {
+    static constexpr bool B_NK = B_NK_;
+    static constexpr int BATCH = BATCH_;
     static constexpr int M = M_, N = N_, K = K_, BM = BM_, BN = BN_, KS = KS_, EPI = EPI_;
     static constexpr int TM = BM / 16;          // 16-row blocks per tile
     static constexpr int G4 = BN / 64;          // 64-column groups
@@ -67,7 +75,8 @@ struct GemmF32 {
     static_assert(N % 4 == 0 && K % 4 == 0, "rows must be 16-byte aligned");
     static_assert(NSTAGE >= NBUF - 1, "k-range shorter than the prefetch depth");
 
-    static constexpr Dims3 GRID{N / BN, M / BM, 1};
+    static constexpr int TILES = (N / BN) * (M / BM);
+    static constexpr Dims3 GRID{N / BN, M / BM, BATCH};
     static constexpr Dims3 BLOCK{64 * KS, 1, 1};
     static constexpr int THREADS = 64 * KS;
     static constexpr bool HAS_BARRIERS = KS > 1;
@@ -83,6 +92,9 @@ struct GemmF32 {
         f32x4 b4[G4 > 0 ? G4 : 1][4];  // [group][t] -> 4 columns
         f32x2 b2[G2 > 0 ? G2 : 1][4];  // [group][t] -> 2 columns
         float b1[G1 > 0 ? G1 : 1][4];  // [group][t]
+        // B_NK: b4[group][e] holds the four k of column 4j+e; the narrower groups likewise
+        f32x4 n2[(B_NK && G2 > 0) ? G2 : 1][2];  // [group][e] -> 4 k of column 2j+e
+        f32x4 n1[(B_NK && G1 > 0) ? G1 : 1];     // [group]    -> 4 k of column j
     };
 
     // Every address is a wave-uniform part (tile origin, k, the row block, the k-step t: scalar
@@ -98,10 +110,31 @@ struct GemmF32 {
         const unsigned b2_off = (unsigned)(4 * kq * N + 2 * i) * 4u;
         const unsigned b1_off = (unsigned)(4 * kq * N + i) * 4u;
         const char* a_ub = reinterpret_cast<const char*>(A + (size_t)m0 * K + k);
-        const char* b_ub = reinterpret_cast<const char*>(B + (size_t)k * N + n0);
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm)
             f.a[tm] = *reinterpret_cast<const f32x4*>(a_ub + (size_t)tm * 16 * K * 4 + a_off);
+        if constexpr (B_NK) {
+            // rows of B are columns of the product: lane (j = i, kq) reads B[n][k + 4kq .. + 3]
+            const char* n_ub = reinterpret_cast<const char*>(B + (size_t)n0 * K + k);
+            const unsigned n4_off = (unsigned)(4 * i * K + 4 * kq) * 4u;
+            const unsigned n2_off = (unsigned)(2 * i * K + 4 * kq) * 4u;
+            const unsigned n1_off = (unsigned)(i * K + 4 * kq) * 4u;
+#pragma unroll
+            for (int g = 0; g < G4; ++g)
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    f.b4[g][e] = *reinterpret_cast<const f32x4*>(n_ub + ((size_t)(g * 64 + e) * K) * 4 + n4_off);
+#pragma unroll
+            for (int g = 0; g < G2; ++g)
+#pragma unroll
+                for (int e = 0; e < 2; ++e)
+                    f.n2[g][e] = *reinterpret_cast<const f32x4*>(n_ub + ((size_t)(G4 * 64 + g * 32 + e) * K) * 4 + n2_off);
+#pragma unroll
+            for (int g = 0; g < G1; ++g)
+                f.n1[g] = *reinterpret_cast<const f32x4*>(n_ub + ((size_t)(G4 * 64 + G2 * 32 + g * 16) * K) * 4 + n1_off);
+            return;
+        }
+        const char* b_ub = reinterpret_cast<const char*>(B + (size_t)k * N + n0);
 #pragma unroll
         for (int g = 0; g < G4; ++g)
 #pragma unroll
@@ -130,17 +163,17 @@ struct GemmF32 {
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
                         acc[tm][4 * g + e] = __builtin_amdgcn_mfma_f32_16x16x4f32(
-                            f.a[tm][t], f.b4[g][t][e], acc[tm][4 * g + e], 0, 0, 0);
+                            f.a[tm][t], B_NK ? f.b4[g][e][t] : f.b4[g][t][e], acc[tm][4 * g + e], 0, 0, 0);
 #pragma unroll
                 for (int g = 0; g < G2; ++g)
 #pragma unroll
                     for (int e = 0; e < 2; ++e)
                         acc[tm][4 * G4 + 2 * g + e] = __builtin_amdgcn_mfma_f32_16x16x4f32(
-                            f.a[tm][t], f.b2[g][t][e], acc[tm][4 * G4 + 2 * g + e], 0, 0, 0);
+                            f.a[tm][t], B_NK ? f.n2[g][e][t] : f.b2[g][t][e], acc[tm][4 * G4 + 2 * g + e], 0, 0, 0);
 #pragma unroll
                 for (int g = 0; g < G1; ++g)
                     acc[tm][4 * G4 + 2 * G2 + g] = __builtin_amdgcn_mfma_f32_16x16x4f32(
-                        f.a[tm][t], f.b1[g][t], acc[tm][4 * G4 + 2 * G2 + g], 0, 0, 0);
+                        f.a[tm][t], B_NK ? f.n1[g][t] : f.b1[g][t], acc[tm][4 * G4 + 2 * G2 + g], 0, 0, 0);
             }
         }
     }
@@ -192,10 +225,11 @@ struct GemmF32 {
     __device__ static __forceinline__ void run(int vblock, int tid, Smem& sm, const void* I, const void* F,
                                                void* O, Sync sync)
     {
-        const float* __restrict__ A = static_cast<const float*>(I);
-        const float* __restrict__ B = static_cast<const float*>(F);
-        float* __restrict__ C = static_cast<float*>(O);
-        const Dims3 vb = XcdTiles<N / BN, M / BM, BM, BN>::tile(vblock);   // tiles dealt so that each XCD's L2 fetches as little as possible
+        const int batch = BATCH > 1 ? vblock / TILES : 0;
+        const float* __restrict__ A = static_cast<const float*>(I) + (size_t)batch * M * K;
+        const float* __restrict__ B = static_cast<const float*>(F) + (size_t)batch * K * N;
+        float* __restrict__ C = static_cast<float*>(O) + (size_t)batch * M * N;
+        const Dims3 vb = XcdTiles<N / BN, M / BM, BM, BN>::tile(BATCH > 1 ? vblock % TILES : vblock);   // tiles dealt so that each XCD's L2 fetches as little as possible
         const int m0 = vb.y * BM, n0 = vb.x * BN;
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;   // wave-uniform: addresses built on it stay in scalar registers
         const int kbeg = wave * KW;

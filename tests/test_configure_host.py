@@ -53,14 +53,14 @@ def test_example_config_resolves_and_writes_the_fusers_files(tmp_path):
 
 def test_unknown_shapes_are_reported_with_the_line_that_would_add_them(tmp_path):
     cfg = tmp_path / "c.yaml"
-    cfg.write_text("FusionSet:\n  - Set: [dense_0, dense_9]\n  - Set: [conv2d_0, conv2d_1, bgemm_0]\n"
+    cfg.write_text("FusionSet:\n  - Set: [dense_0, dense_9]\n  - Set: [conv2d_0, conv2d_1, bgemm_9]\n"
                    "KernelInfo:\n  dense_0: [512, 512, 512]\n  dense_9: [512, 100, 100]\n  conv2d_0: [1, 224, 224, 64, 3, 7, 7, 2, 3]\n"
-                   "  conv2d_1: [1, 56, 56, 64, 64, 3, 3, 1, 1]\n  bgemm_0: [12, 512, 64, 512]\n")
+                   "  conv2d_1: [1, 56, 56, 64, 64, 3, 3, 1, 1]\n  bgemm_9: [16, 208, 208, 64]\n")
     with pytest.raises(LookupError) as e:
         configure.configure(str(cfg), str(tmp_path / "a"))
-    assert "dense_9" in str(e.value) and "gemm_f32_512x100x100" in str(e.value) and "bgemm_0" in str(e.value) and not (tmp_path / "a").exists()
+    assert "dense_9" in str(e.value) and "gemm_f32_512x100x100" in str(e.value) and "bgemm_9" in str(e.value) and not (tmp_path / "a").exists()
     r = configure.configure(str(cfg), str(tmp_path / "b"), skip_missing=True)
-    assert r["found"] == {"dense_0": "gemm_f32_512x512x512", "conv2d_1": "conv3x3_f32_64x56x56_64"} and sorted(r["missing"]) == ["bgemm_0", "conv2d_0", "dense_9"]
+    assert r["found"] == {"dense_0": "gemm_f32_512x512x512", "conv2d_1": "conv3x3_f32_64x56x56_64"} and sorted(r["missing"]) == ["bgemm_9", "conv2d_0", "dense_9"]
     assert r["pairs"] == [("dense_0", "conv2d_1")]
     # the bf16 kernel only when asked for, or when there is no fp32 one
     r2 = configure.configure(EXAMPLE, str(tmp_path / "c2"), dtype="f32", skip_missing=True)
@@ -87,7 +87,9 @@ def test_command_line(tmp_path):
 @pytest.mark.skipif(not os.path.isdir(REF_EXAMPLES), reason="the reference's example configs are not on this machine")
 @pytest.mark.parametrize("name,want", [("llm.yaml", {"dense_0": "gemm_f32_512x768x768", "dense_1": "gemm_f32_512x768x3072", "dense_2": "gemm_f32_512x3072x768",
                                                      "dense_3": "gemm_f32_512x768x2304", "dense_4": "gemm_bf16_512x4096x4096", "dense_5": "gemm_f32_512x4096x1024",
-                                                     "dense_6": "gemm_bf16_512x4096x14336", "dense_7": "gemm_bf16_512x14336x4096"}),
+                                                     "dense_6": "gemm_bf16_512x4096x14336", "dense_7": "gemm_bf16_512x14336x4096",
+                                                     "bgemm_0": "bgemm_f32_12x512x64x512", "bgemm_1": "bgemm_f32_12x512x512x64",
+                                                     "bgemm_2": "bgemm_f32_32x512x128x512", "bgemm_3": "bgemm_f32_32x512x512x128"}),
                                        ("resnet-18.yaml", {"conv2d_1": "conv3x3_f32_64x56x56_64", "conv2d_4": "conv3x3_f32_128x28x28_128"})])
 def test_the_references_own_example_configs(tmp_path, name, want):
     """The reference's examples (read in place) ship with empty fusion sets: every id goes into both

@@ -97,3 +97,46 @@ def test_resnet_conv2d_4_against_the_oracle_and_fused_with_layernorm():
     st = oracle_cases.rel_stats(c, want, 1e-5)
     print(f"[parity] {name}: worst |d|/max(|ref|,rms) {st['worst_floor_rel']:.3e}; {st['n_fail']} fail; {t:.1f} us", flush=True)
     assert st["n_fail"] == 0
+
+
+@pytest.mark.parametrize("kid,b,m,k,n,partner,fuse", [
+    ("bgemm_0", 12, 512, 64, 512, "softmax_causal_12x512x512", True),
+    ("bgemm_1", 12, 512, 512, 64, "layernorm_512x768", True),
+    ("bgemm_2", 32, 512, 128, 512, "layernorm_512x768", False),
+    ("bgemm_3", 32, 512, 512, 128, "layernorm_512x768", False)])
+def test_attention_batched_gemm_against_the_oracle(kid, b, m, k, n, partner, fuse):
+    """The reference's bgemm, C[b] = A[b] . B[b]^T with B stored [b, N, K]: every batch at full size against the
+    oracle; selector inputs that would expose a batch or a row of B read from the wrong place; and, where a
+    fused kernel is built, bit-exactness against the two kernels launched back to back."""
+    name = f"bgemm_f32_{b}x{m}x{k}x{n}"
+    print(f"[models] {kid} -> {name}", flush=True)
+    a = fill_normal(0x1B0 + k, b * m * k, 0.0, 1.0)
+    w = fill_normal(0x2B0 + n, b * n * k, 0.0, 0.125)
+    if partner.startswith("softmax"):
+        x, f2 = fill_normal(0x3B0, 12 * 512 * 512, 0.0, 0.125), np.zeros(1, np.float32)
+    else:
+        x = fill_normal(0xF0, 512 * 768, 0.0, 1.0)
+        f2 = np.concatenate([fill_normal(0xF1, 768, 1.0, 0.1), fill_normal(0xF2, 768, 0.0, 0.1)])
+    with bf.Operation(name, partner) as op:
+        c = op.run_kernel(0, a, w)
+        # A[b, r, :] = one-hot at k = (r + b) mod K  =>  C[b, r, j] = B[b, j, (r + b) mod K] exactly
+        sel = np.zeros((b, m, k), np.float32)
+        bi, ri = np.meshgrid(np.arange(b), np.arange(m), indexing="ij")
+        sel[bi, ri, (ri + bi) % k] = 1.0
+        cs = op.run_kernel(0, sel.ravel(), w)
+        if fuse:
+            y = op.run_kernel(1, x, f2)
+            q1, q2 = op.run_fuse(op.fused("bfuse", "_c256"), a, w, x, f2)
+            assert q1.tobytes() == c.tobytes() and q2.tobytes() == y.tobytes(), "fused output differs from the unfused kernels"
+        op.upload(0, a, w)
+        t = float(np.mean(op.time("kernel1", warmup=10, reps=50)[0]))
+    W = w.reshape(b, n, k)
+    want_sel = np.stack([W[i][:, (np.arange(m) + i) % k].T for i in range(b)])
+    assert np.array_equal(cs.reshape(b, m, n), want_sel), "selector inputs: an output element is not the B element it selects"
+    A = a.reshape(b, m, k)
+    want = np.stack([orf.gemm_f32(A[i], W[i], b_is_nk=True) for i in range(b)])
+    st = oracle_cases.rel_stats(c, want, 1e-5)
+    mb = 4.0 * b * (m * k + n * k + m * n) / 1e6
+    print(f"[parity] {name}: worst |d|/max(|ref|,rms) {st['worst_floor_rel']:.3e}; {st['n_fail']} fail; {t:.1f} us "
+          f"({2.0 * b * m * n * k / t * 1e-6:.1f} TFLOP/s, {mb / t * 1e3:.0f} GB/s)", flush=True)
+    assert st["n_fail"] == 0
