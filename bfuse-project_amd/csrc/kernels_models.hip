@@ -60,9 +60,11 @@ BFUSE_BFUSE_KERNEL(conv3x3_f32_128x28x28_128, Conv128, layernorm_512x768, LayerN
 // context products (12 heads, sequence 512, head size 64), bgemm_2 / bgemm_3 Llama-3-8B's (32 heads, head size 128).
 // Operands go global -> VGPR in MFMA layout (both are contiguous along K); a short reduction (K = 64, 128) is
 // one wave's, a long one (K = 512) is split over two.
-using Bgemm0 = GemmF32<512, 512, 64, 32, 64, 1, kEpiNone, 2, 1, true, 12>;     // 16 x 8 tiles x 12 = 1536 one-wave workgroups
-using Bgemm1 = GemmF32<512, 64, 512, 16, 64, 2, kEpiNone, 2, 1, true, 12>;     // 32 x 1 tiles x 12 = 384 two-wave workgroups
-using Bgemm2 = GemmF32<512, 512, 128, 32, 64, 1, kEpiNone, 2, 1, true, 32>;    // 4096 one-wave workgroups
+// (tiles measured on bgemm_0 / bgemm_1: 64 x 64 one-wave 8.0 us, 32 x 64 8.3-9.0, 32 x 128 8.0, 16 x 64 10.1, 64 x 128 11.1;
+//  32 x 64 two-wave 9.7 us, 16 x 64 two-wave 11.3, four-wave 11.3, 16 x 32 10.1)
+using Bgemm0 = GemmF32<512, 512, 64, 64, 64, 1, kEpiNone, 2, 1, true, 12>;     // 8 x 8 tiles x 12 = 768 one-wave workgroups
+using Bgemm1 = GemmF32<512, 64, 512, 32, 64, 2, kEpiNone, 2, 1, true, 12>;     // 16 x 1 tiles x 12 = 192 two-wave workgroups
+using Bgemm2 = GemmF32<512, 512, 128, 64, 64, 1, kEpiNone, 2, 1, true, 32>;    // 2048 one-wave workgroups
 using Bgemm3 = GemmF32<512, 128, 512, 32, 64, 2, kEpiNone, 2, 1, true, 32>;    // 16 x 2 tiles x 32 = 1024 two-wave workgroups
 BFUSE_KERNEL(bgemm_f32_12x512x64x512, Bgemm0, ({{12, 512, 64, 1}, 4}), ({{12, 512, 64, 1}, 4}), ({{12, 512, 512, 1}, 4}))
 BFUSE_KERNEL(bgemm_f32_12x512x512x64, Bgemm1, ({{12, 512, 512, 1}, 4}), ({{12, 64, 512, 1}, 4}), ({{12, 512, 64, 1}, 4}))
