@@ -140,3 +140,22 @@ def test_attention_batched_gemm_against_the_oracle(kid, b, m, k, n, partner, fus
     print(f"[parity] {name}: worst |d|/max(|ref|,rms) {st['worst_floor_rel']:.3e}; {st['n_fail']} fail; {t:.1f} us "
           f"({2.0 * b * m * n * k / t * 1e-6:.1f} TFLOP/s, {mb / t * 1e3:.0f} GB/s)", flush=True)
     assert st["n_fail"] == 0
+
+
+def test_pair_matrix_of_the_model_operators(tmp_path):
+    """The reference's benchmark arrangement over the operators the library holds: every dense layer with every
+    attention product and convolution, 48 pairs, each fused kernel validated bit for bit against the unfused
+    pair inside the run (the suite's validation), speed-ups tabulated by the reference's definitions."""
+    import os
+    from bfuse_project_amd import configure, suite
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = tmp_path / "matrix"
+    r = configure.configure(os.path.join(root, "bfuse-project_amd", "examples", "model_operators.yaml"), str(out))
+    assert not r["missing"] and len(r["pairs"]) == 48 and all(r["fused"][f"{a} + {b}"] for a, b in r["pairs"])
+    print("[models] pair matrix, 48 pairs", flush=True)
+    rows = suite.run_suite(suite.load_info(str(out / "config" / "info.yaml")), str(out), validate=True, log=lambda m: None)
+    assert len(rows) == 48 and all("bfuse_ns" in x and "parallel_ns" in x for x in rows)
+    g = suite.geomean([x["bfuse_speedup"] for x in rows])
+    print(f"[models] geomean speed-up over serial: bfuse {g:.3f}x, two streams {suite.geomean([x['parallel_speedup'] for x in rows]):.3f}x; "
+          f"best {max(x['bfuse_speedup'] for x in rows):.2f}x, worst {min(x['bfuse_speedup'] for x in rows):.2f}x", flush=True)
+    assert 0.8 < g < 2.0
