@@ -1,17 +1,23 @@
 // benchmark -- command-line driver over libbfuse_rt, the counterpart of the reference's
 // generated main.cc (test-utils/test-suite-files/main_cc.py:22-36,139-299):
 //
-//     benchmark [-vh] [-n num_iterations] [-s seed] [-x suffix] T K1 K2
+//     benchmark [-vhd] [-n num_iterations] [-s seed] [-x suffix] [-i info.yaml] T K1 K2
 //
 //      T : type of operation: 0 kernel1, 1 kernel2, 2 parallel (two streams), 3 hfuse, 4 bfuse,
 //          5 serial (kernel1 then kernel2 on one stream; not in the reference)
-//  K1,K2 : index into the first / second fusion set, or a kernel name.  The sets are the
-//          distinct first / second sides of the fused kernels the library was built with.
+//  K1,K2 : a number is the position in the first / second `FusionSet` of the suite's info.yaml,
+//          exactly what the reference's ASSIGN_* tables switch on (macro_h.py:296-320; the
+//          command matrix of scripts/profile_test_suite.py:13-47 passes such positions); the
+//          set members are kernel names of the library.  Anything else is a kernel name.
+//     -i : the suite's info.yaml; default ./config/info.yaml when that file exists.  Without an
+//          info file a numeric K1 / K2 is an error, not a guess.
 //     -v : validate: run the variant, then each unfused kernel on the same inputs, and compare
 //          (the reference's check, main_cc.py:82-122,246-268).  Fused and parallel outputs
 //          must be bit-identical to the unfused ones; check_matrix (eps 1e-3) is reported too.
 //          Exit status 1 on mismatch (main_cc.py:288-292).
-//     -x : variant suffix of a bfuse kernel (e.g. _c256); default is the plain name.
+//     -d : dry run: print the kernels T K1 K2 resolve to and exit (needs no device).
+//     -x : variant suffix of a bfuse kernel (e.g. _c256); default is the plain name, or the
+//          only fused kernel of that kind the library holds for the pair.
 //
 // Inputs are seeded U(-0.5, 0.5) (the reference uses rand()/RAND_MAX - 0.5, utils_cc.py:28-31).
 // Prints the GPU-side duration of every timed launch set (3 warm-up launches are discarded,
@@ -22,6 +28,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <fstream>
 #include <string>
 #include <vector>
 
@@ -31,20 +38,24 @@ static bool validation = false;
 static size_t num_iterations = 1;
 static unsigned long long seed = 0xB5F05E;
 static std::string suffix;
+static std::string info_path;
+static bool dry_run = false;
 static const char* operation_type_string[] = {"kernel1", "kernel2", "parallel", "hfuse", "bfuse", "serial"};
 
 static void print_help(const char* prog)
 {
-    printf("Usage: %s [-vh] [-n num_iterations] [-s seed] [-x suffix] T K1 K2\n", prog);
+    printf("Usage: %s [-vhd] [-n num_iterations] [-s seed] [-x suffix] [-i info.yaml] T K1 K2\n", prog);
     printf("Options:\n");
     printf("     -v : validate test.                (default: off)\n");
     printf("     -h : print this page.\n");
     printf("     -n : number of iterations.         (default: 1)\n");
     printf("     -s : seed of the synthetic inputs.\n");
     printf("     -x : suffix of the bfuse variant.   (default: none)\n");
+    printf("     -i : info.yaml of the suite.        (default: ./config/info.yaml if present)\n");
+    printf("     -d : only print the kernels the command resolves to (no device needed).\n");
     printf("      T : type of operation (0 kernel1, 1 kernel2, 2 parallel, 3 hfuse, 4 bfuse, 5 serial).\n");
-    printf("     K1 : idx or name of kernel1.\n");
-    printf("     K2 : idx or name of kernel2.\n");
+    printf("     K1 : idx (position in the first FusionSet of info.yaml) or name of kernel1.\n");
+    printf("     K2 : idx (position in the second FusionSet of info.yaml) or name of kernel2.\n");
 }
 
 #define CHECK(call)                                                                \
@@ -56,34 +67,113 @@ static void print_help(const char* prog)
         }                                                                          \
     } while (0)
 
-static std::vector<std::string> fusion_set(int which)
+// The two `Set` lists under `FusionSet:` of an info.yaml, in block style (what PyYAML and LLVM's YAML
+// writer emit, scripts/configure_kernels.py:316-318) or flow style (`Set: [a, b]`).  Other top-level
+// keys (KernelInfo, ...) are skipped.
+static std::string trimmed(const std::string& s)
 {
-    std::vector<std::string> out;
-    for (int i = 0; i < bfuse_kernel_count(); ++i) {
-        bfuse_kernel_info ki;
-        CHECK(bfuse_kernel_at(i, &ki));
-        if (ki.kind == BFUSE_KIND_SINGLE) continue;
-        std::string s = ki.side[which];
-        bool seen = false;
-        for (auto& o : out) seen |= (o == s);
-        if (!seen) out.push_back(s);
+    size_t a = s.find_first_not_of(" \t\r"), b = s.find_last_not_of(" \t\r");
+    if (a == std::string::npos) return "";
+    std::string t = s.substr(a, b - a + 1);
+    if (t.size() >= 2 && (t.front() == '"' || t.front() == '\'') && t.back() == t.front()) t = t.substr(1, t.size() - 2);
+    return t;
+}
+
+static bool read_fusion_sets(const std::string& path, std::vector<std::vector<std::string>>& sets)
+{
+    std::ifstream in(path);
+    if (!in) return false;
+    std::string line;
+    bool inside = false;
+    while (std::getline(in, line)) {
+        const size_t hash = line.find(" #");
+        if (hash != std::string::npos) line.erase(hash);
+        if (trimmed(line).empty() || trimmed(line)[0] == '#') continue;
+        const bool top_level = line[0] != ' ' && line[0] != '-' && line[0] != '\t';
+        if (top_level) {
+            inside = trimmed(line).rfind("FusionSet:", 0) == 0;
+            continue;
+        }
+        if (!inside) continue;
+        std::string t = trimmed(line);
+        if (t[0] == '-') t = trimmed(t.substr(1));
+        if (t.rfind("Set:", 0) == 0) {
+            sets.emplace_back();
+            std::string rest = trimmed(t.substr(4));
+            if (!rest.empty() && rest.front() == '[') {          // flow list on the same line
+                rest = rest.substr(1, rest.find(']') == std::string::npos ? std::string::npos : rest.find(']') - 1);
+                size_t pos = 0;
+                while (pos <= rest.size()) {
+                    const size_t comma = rest.find(',', pos);
+                    const std::string item = trimmed(rest.substr(pos, comma == std::string::npos ? std::string::npos : comma - pos));
+                    if (!item.empty()) sets.back().push_back(item);
+                    if (comma == std::string::npos) break;
+                    pos = comma + 1;
+                }
+            }
+        } else if (!sets.empty() && !t.empty() && t.find(':') == std::string::npos) {
+            sets.back().push_back(t);
+        }
     }
-    return out;
+    return true;
 }
 
 static std::string resolve(const char* arg, int which)
 {
     char* end = nullptr;
     long idx = strtol(arg, &end, 10);
-    if (end && *end == '\0') {
-        auto set = fusion_set(which);
-        if (idx < 0 || idx >= (long)set.size()) {
-            fprintf(stderr, "K%d index %ld out of range (set has %zu kernels)\n", which + 1, idx, set.size());
-            exit(EXIT_FAILURE);
-        }
-        return set[idx];
+    if (!(end && *end == '\0' && end != arg)) return arg;          // a kernel name
+    std::string path = info_path;
+    if (path.empty()) {
+        std::ifstream probe("./config/info.yaml");
+        if (probe) path = "./config/info.yaml";
     }
-    return arg;
+    if (path.empty()) {
+        fprintf(stderr, "K%d = %ld is a position in the suite's info.yaml: pass it with -i (no ./config/info.yaml here), or name the kernel\n",
+                which + 1, idx);
+        exit(EXIT_FAILURE);
+    }
+    std::vector<std::vector<std::string>> sets;
+    if (!read_fusion_sets(path, sets)) {
+        fprintf(stderr, "cannot read %s\n", path.c_str());
+        exit(EXIT_FAILURE);
+    }
+    if (sets.size() != 2) {
+        fprintf(stderr, "%s: Number of fusion sets are only 2. (found %zu)\n", path.c_str(), sets.size());   // profile_test_suite.py:19-21
+        exit(EXIT_FAILURE);
+    }
+    if (idx < 0 || idx >= (long)sets[which].size()) {
+        fprintf(stderr, "K%d index %ld out of range (set %d of %s has %zu kernels)\n", which + 1, idx, which, path.c_str(), sets[which].size());
+        exit(EXIT_FAILURE);
+    }
+    return sets[which][idx];
+}
+
+// The fused kernel of `kind` for (k1, k2): the plain name (+ -x suffix) when the library holds it, else the
+// only variant it holds for the pair; several variants and no -x is an error that lists them.
+static void find_fused(const std::string& k1, const std::string& k2, int kind, bfuse_kernel_info* out)
+{
+    const std::string fname = k1 + "_" + k2 + (kind == BFUSE_KIND_HFUSE ? "_fused_hfuse" : "_fused_bfuse") + (kind == BFUSE_KIND_BFUSE ? suffix : "");
+    if (bfuse_kernel_find(fname.c_str(), out) == 0) return;
+    std::vector<bfuse_kernel_info> hits;
+    if (suffix.empty() || kind == BFUSE_KIND_HFUSE)
+        for (int i = 0; i < bfuse_kernel_count(); ++i) {
+            bfuse_kernel_info ki;
+            CHECK(bfuse_kernel_at(i, &ki));
+            if (ki.kind == kind && ki.n_sides == 2 && k1 == ki.side[0] && k2 == ki.side[1]) hits.push_back(ki);
+        }
+    if (hits.size() == 1) {
+        *out = hits[0];
+        return;
+    }
+    fprintf(stderr, "unknown kernel %s", fname.c_str());
+    if (hits.size() > 1) {
+        fprintf(stderr, "; the library holds");
+        for (auto& h : hits) fprintf(stderr, " %s", h.name);
+        fprintf(stderr, " -- choose one with -x");
+    }
+    fprintf(stderr, "\n");
+    exit(EXIT_FAILURE);
 }
 
 struct HostSide {
@@ -157,7 +247,7 @@ static void stats(const char* label, const std::vector<float>& v)
 int main(int argc, char** argv)
 {
     int c;
-    while ((c = getopt(argc, argv, "vhn:s:x:")) != -1) {
+    while ((c = getopt(argc, argv, "vhdn:s:x:i:")) != -1) {
         switch (c) {
             case 'v': validation = true; break;
             case 'n': {
@@ -172,6 +262,8 @@ int main(int argc, char** argv)
             }
             case 's': seed = strtoull(optarg, nullptr, 0); break;
             case 'x': suffix = optarg; break;
+            case 'i': info_path = optarg; break;
+            case 'd': dry_run = true; break;
             case 'h':
             default: print_help(argv[0]); exit(0);
         }
@@ -187,8 +279,20 @@ int main(int argc, char** argv)
         return EXIT_FAILURE;
     }
     const size_t T = (size_t)t_arg;
-    CHECK(bfuse_init(0));
     const std::string k1 = resolve(argv[optind + 1], 0), k2 = resolve(argv[optind + 2], 1);
+    if (dry_run) {
+        // what the command would launch, from the registry alone (no device needed)
+        bfuse_kernel_info ki;
+        CHECK(bfuse_kernel_find(k1.c_str(), &ki));
+        CHECK(bfuse_kernel_find(k2.c_str(), &ki));
+        printf("- Type of operation: %s\n- Kernel1: %s\n- Kernel2: %s\n", operation_type_string[T], k1.c_str(), k2.c_str());
+        if (T == BFUSE_MODE_HFUSE || T == BFUSE_MODE_BFUSE) {
+            find_fused(k1, k2, T == BFUSE_MODE_HFUSE ? BFUSE_KIND_HFUSE : BFUSE_KIND_BFUSE, &ki);
+            printf("- Fused kernel: %s\n", ki.name);
+        }
+        return 0;
+    }
+    CHECK(bfuse_init(0));
 
     HostSide a, b;
     setup(a, k1, 1);
@@ -199,8 +303,7 @@ int main(int argc, char** argv)
     bfuse_kernel_info fused;
     memset(&fused, 0, sizeof(fused));
     if (T == BFUSE_MODE_HFUSE || T == BFUSE_MODE_BFUSE) {
-        const std::string fname = k1 + "_" + k2 + (T == BFUSE_MODE_HFUSE ? "_fused_hfuse" : "_fused_bfuse" + suffix);
-        CHECK(bfuse_kernel_find(fname.c_str(), &fused));
+        find_fused(k1, k2, T == BFUSE_MODE_HFUSE ? BFUSE_KIND_HFUSE : BFUSE_KIND_BFUSE, &fused);
     }
     printf("============= Benchmark =============\n");
     printf("- Number of iterations: %zu\n- Type of operation: %s\n- Kernel1: %s\n- Kernel2: %s\n", num_iterations,

@@ -60,31 +60,58 @@ def combos(info: dict, triangular: bool = False) -> List[Tuple[int, int]]:
 
 
 # ---- command matrix (profile_test_suite.py:13-140) ----------------------------------------------
-def valid_commands(info: dict, benchmark_path: str, triangular: bool = False) -> List[List[str]]:
+def _ids(info: dict, info_path: Optional[str]):
+    """How a command names its kernels: with the suite's info.yaml at hand by position in the two sets
+    (`-i info.yaml T idx1 idx2`, the reference's form: its benchmark switches on those positions,
+    macro_h.py:296-320), without it by kernel name."""
     a, b = set_names(info)
-    common = [os.path.abspath(benchmark_path), "-v"]
+    if info_path:
+        return ["-i", os.path.abspath(info_path)], (lambda i: str(i)), (lambda j: str(j))
+    return [], (lambda i: a[i]), (lambda j: b[j])
+
+
+def bfuse_suffix(k1: str, k2: str) -> List[str]:
+    """`-x suffix` selecting the block-fused variant of (k1, k2) when the library holds several and none
+    under the plain name: the one the footprint rule selects, else the first registered."""
+    from . import tuner
+    from .operation import kernel_info
+    variants = [h for h in tuner.built_variants(k1, k2) if h.kind == 1]
+    stem = f"{k1}_{k2}_fused_bfuse"
+    if len(variants) <= 1 or any(h.name == stem for h in variants):
+        return []
+    a, b = kernel_info(k1), kernel_info(k2)
+    pick = tuner.find_variant(a, b, {"kind": "bfuse", "pattern": "chunked", "p0": 256, "p1": 1}) or variants[0]
+    return ["-x", pick.name[len(stem):]]
+
+
+def valid_commands(info: dict, benchmark_path: str, triangular: bool = False, info_path: Optional[str] = None) -> List[List[str]]:
+    """`benchmark -v T K1 K2` for every method and pair (profile_test_suite.py:13-47)."""
+    a, b = set_names(info)
+    opts, k1, k2 = _ids(info, info_path)
+    common = [os.path.abspath(benchmark_path), "-v"] + opts
     out = []
     for idx, _ in enumerate(METHODS):
         if idx == 0:
-            out += [common + [str(idx), k, b[0]] for k in a]
+            out += [common + [str(idx), k1(i), k2(0)] for i in range(len(a))]
         elif idx == 1:
-            out += [common + [str(idx), a[0], k] for k in b]
+            out += [common + [str(idx), k1(0), k2(j)] for j in range(len(b))]
         else:
-            out += [common + [str(idx), a[i], b[j]] for i, j in combos(info, triangular)]
+            out += [common + (bfuse_suffix(a[i], b[j]) if idx == 4 else []) + [str(idx), k1(i), k2(j)] for i, j in combos(info, triangular)]
     return out
 
 
-def exec_commands(info: dict, benchmark_path: str, exec_path: str, triangular: bool = False) -> List[List[str]]:
+def exec_commands(info: dict, benchmark_path: str, exec_path: str, triangular: bool = False, info_path: Optional[str] = None) -> List[List[str]]:
     """One rocprofv3 kernel-trace run per (method, k1, k2); the trace lands in
     `<exec_path>/<method index>_<i>_<j>_kernel_trace.csv` (the reference's file naming with the
     profiler's suffix)."""
     a, b = set_names(info)
+    opts, k1, k2 = _ids(info, info_path)
     bench = os.path.abspath(benchmark_path)
     n = str(WARMUP_TRIALS + TIMED_TRIALS)
 
     def one(idx, i, j):
         return ["rocprofv3", "--kernel-trace", "--output-format", "csv", "-d", exec_path, "-o", f"{idx}_{i}_{j}", "--",
-                bench, "-n", n, str(idx), a[i], b[j]]
+                bench, "-n", n] + opts + (bfuse_suffix(a[i], b[j]) if idx == 4 else []) + [str(idx), k1(i), k2(j)]
     out = []
     for idx, _ in enumerate(METHODS):
         if idx == 0:
@@ -330,7 +357,7 @@ def main(argv=None) -> int:
         return 1
     exec_dir = os.path.join(args.out, "exec")
     if args.commands:
-        for c in exec_commands(info, args.benchmark, exec_dir, args.triangular):
+        for c in exec_commands(info, args.benchmark, exec_dir, args.triangular, args.file):
             print(" ".join(c))
         return 0
     rows = analyze(info, exec_dir, args.triangular) if args.analyze else run_suite(info, args.out, not args.no_validate, args.triangular)

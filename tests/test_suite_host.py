@@ -9,6 +9,8 @@ import numpy as np
 import pytest
 import yaml
 
+import bfuse_project_amd as bf
+
 from bfuse_project_amd import suite
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -111,3 +113,84 @@ def test_analyze_and_tables(tmp_path, info):
     assert "geomean speed-up over serial" in md and "1.25x" in md
     assert suite.geomean([2.0, 8.0]) == pytest.approx(4.0)
     assert suite.main([os.path.join(ROOT, "bfuse-project_amd", "examples", "headline_pairs.yaml"), "--commands", "-o", str(tmp_path)]) == 0
+
+
+# ---- numeric K1 / K2 of the command-line driver ----------------------------------------------
+EXE = os.path.join(ROOT, "bfuse-project_amd", "benchmark")
+
+
+def _dry(args, cwd=None):
+    import subprocess
+    r = subprocess.run([EXE, "-d", *args], capture_output=True, text=True, timeout=60, cwd=cwd)
+    got = {}
+    for line in r.stdout.splitlines():
+        if line.startswith("- ") and ": " in line:
+            k, v = line[2:].split(": ", 1)
+            got[k] = v.split()[0] if k == "Fused kernel" else v
+    return r, got
+
+
+def test_numeric_ids_are_positions_in_the_suites_info_yaml(tmp_path):
+    """The reference's command matrix (scripts/profile_test_suite.py:13-47) passes positions in the two
+    FusionSets of info.yaml, and its benchmark switches on them (macro_h.py:296-320).  Restated here for
+    a `configure` output and resolved command by command (dry run: needs no device)."""
+    from bfuse_project_amd import configure, tuner
+    out = tmp_path / "s"
+    configure.configure(os.path.join(ROOT, "bfuse-project_amd", "examples", "model_operators.yaml"), str(out))
+    info_path = str(out / "config" / "info.yaml")
+    with open(info_path) as f:
+        info_yaml = yaml.safe_load(f)
+    fusion_sets = info_yaml["FusionSet"]
+    kernel1_size, kernel2_size = len(fusion_sets[0]["Set"]), len(fusion_sets[1]["Set"])
+    assert kernel1_size >= 2 and kernel2_size >= 2 and fusion_sets[0]["Set"] != fusion_sets[1]["Set"]
+    # the reference's loops, upper triangle included
+    want = []
+    for idx in range(5):
+        if idx == 0:
+            want += [[str(idx), str(k), "0"] for k in range(kernel1_size)]
+        if idx == 1:
+            want += [[str(idx), "0", str(k)] for k in range(kernel2_size)]
+        if idx in (2, 3, 4):
+            want += [[str(idx), str(k1), str(k2)] for k1 in range(kernel1_size) for k2 in range(k1, kernel2_size)]
+    ours = suite.valid_commands(suite.load_info(info_path), EXE, triangular=True, info_path=info_path)
+    assert [c[-3:] for c in ours] == want
+    assert all(c[:4] == [EXE, "-v", "-i", info_path] for c in ours)
+    checked_fused = 0
+    for c in ours:
+        t, i, j = int(c[-3]), int(c[-2]), int(c[-1])
+        k1, k2 = fusion_sets[0]["Set"][i], fusion_sets[1]["Set"][j]
+        built = tuner.built_variants(k1, k2)
+        if t in (3, 4) and not [h for h in built if h.kind == (2 if t == 3 else 1)]:
+            r, got = _dry(c[2:])
+            assert r.returncode != 0 and "unknown kernel" in r.stderr      # no fused kernel of that kind for the pair
+            continue
+        r, got = _dry(c[2:])
+        assert r.returncode == 0, (c, r.stderr)
+        assert got["Kernel1"] == k1 and got["Kernel2"] == k2, (c, got)
+        if t in (3, 4):
+            h = bf.kernel_info(got["Fused kernel"])
+            assert h.sides == (k1, k2) and h.kind == (2 if t == 3 else 1)
+            checked_fused += 1
+    assert checked_fused >= 4
+
+
+def test_numeric_ids_without_an_info_file_are_an_error_and_names_keep_working(tmp_path):
+    r, _ = _dry(["4", "0", "1"], cwd=str(tmp_path))
+    assert r.returncode != 0 and "info.yaml" in r.stderr
+    r, got = _dry(["4", "gemm_f32_512x768x2304", "layernorm_512x768"], cwd=str(tmp_path))
+    assert r.returncode == 0 and got["Fused kernel"] == "gemm_f32_512x768x2304_layernorm_512x768_fused_bfuse"
+    # ./config/info.yaml is the default; flow-style lists and quoted names are read too
+    (tmp_path / "config").mkdir()
+    (tmp_path / "config" / "info.yaml").write_text(
+        "# suite\nFusionSet:\n  - Set: [bias_relu_4096, 'gemm_f32_512x768x2304']\n  - Set:\n      - layernorm_8x256\n      - layernorm_512x768\n"
+        "KernelInfo:\n  dense_3: [512, 768, 2304]\n")
+    r, got = _dry(["4", "1", "1"], cwd=str(tmp_path))
+    assert r.returncode == 0 and (got["Kernel1"], got["Kernel2"]) == ("gemm_f32_512x768x2304", "layernorm_512x768")
+    r, got = _dry(["0", "0", "0"], cwd=str(tmp_path))
+    assert r.returncode == 0 and (got["Kernel1"], got["Kernel2"]) == ("bias_relu_4096", "layernorm_8x256")
+    r, _ = _dry(["0", "2", "0"], cwd=str(tmp_path))
+    assert r.returncode != 0 and "out of range" in r.stderr
+    one = tmp_path / "one.yaml"
+    one.write_text("FusionSet:\n- Set:\n  - bias_relu_4096\n")
+    r, _ = _dry(["-i", str(one), "0", "0", "0"], cwd=str(tmp_path))
+    assert r.returncode != 0 and "only 2" in r.stderr
