@@ -56,7 +56,7 @@ class LaunchDescC(C.Structure):
 
 # every symbol include/bfuse_rt.h declares
 EXPORTS = [
-    "bfuse_last_error", "bfuse_init", "bfuse_shutdown", "bfuse_device_info",
+    "bfuse_last_error", "bfuse_init", "bfuse_shutdown", "bfuse_device_info", "bfuse_device_memory",
     "bfuse_plan_threads", "bfuse_plan_blocks", "bfuse_map_block", "bfuse_map_thread", "bfuse_map_blocks_device", "bfuse_map_blocks_device_noalloc", "bfuse_probe_placement", "bfuse_set_plan",
     "bfuse_set_sync_spin_limit",
     "bfuse_kernel_count", "bfuse_kernel_at", "bfuse_kernel_find",

@@ -135,6 +135,6 @@ BFUSE_BFUSE_KERNEL(conv3x3_f32_64x8x16_16, ConvS3, layernorm_8x256, LayerNormS, 
 // both sides synchronise (each split-K GEMM's reduction barriers): each side gets LDS arrival counters of its own
 BFUSE_HFUSE_KERNEL(gemm_f32_128x160x192_d, GemmS5, gemm_gelu_f32_64x192x288_d, GemmS6)
 // the give-up path of the side barrier, forced from the host with a small spin limit
-BFUSE_KERNEL(sync_probe_a, SyncProbeA, ({{512, 1, 1, 1}, 4}), ({{512, 1, 1, 1}, 4}), ({{512, 1, 1, 1}, 4}))
-BFUSE_KERNEL(sync_probe_b, SyncProbeB, ({{768, 1, 1, 1}, 4}), ({{768, 1, 1, 1}, 4}), ({{768, 1, 1, 1}, 4}))
-BFUSE_HFUSE_KERNEL(sync_probe_a, SyncProbeA, sync_probe_b, SyncProbeB)
+BFUSE_KERNEL(selftest_sync_a, SyncProbeA, ({{512, 1, 1, 1}, 4}), ({{512, 1, 1, 1}, 4}), ({{512, 1, 1, 1}, 4}))
+BFUSE_KERNEL(selftest_sync_b, SyncProbeB, ({{768, 1, 1, 1}, 4}), ({{768, 1, 1, 1}, 4}), ({{768, 1, 1, 1}, 4}))
+BFUSE_HFUSE_KERNEL(selftest_sync_a, SyncProbeA, selftest_sync_b, SyncProbeB)

@@ -43,6 +43,8 @@ int bfuse_init(int device);
 int bfuse_shutdown(void);
 /* name, CU count, LDS bytes per workgroup, wavefront size of the selected device */
 int bfuse_device_info(char* name, size_t name_len, int* compute_units, int* lds_bytes, int* wave_size);
+/* free and total device memory of the selected device in bytes (hipMemGetInfo); either may be NULL */
+int bfuse_device_memory(size_t* free_bytes, size_t* total_bytes);
 
 /* ------------------------------------------------------------------------------------------
  * Fusion index maps -- horizontal-fuser/src/Algorithms.cc.  Pure host arithmetic, usable
@@ -111,12 +113,14 @@ int bfuse_set_plan(const void* func, const bfuse_block_plan* plan);
 int bfuse_map_blocks_device(const bfuse_block_plan* plan, int lo, int hi, int* kernel_out, int* virt_out);
 
 /* bfuse_map_blocks_device without any allocation.  No counterpart in the reference: it is for
- * callers that cannot allocate device memory where they call -- code under HIP graph capture, tight
- * serving loops, harnesses that forbid hipMalloc.  Same arguments and results; the two tables are
- * staged in a fixed device array of the library (2 x BFUSE_NOALLOC_MAX_IDS ints = 2 MiB per GPU,
- * held until the process ends) whose address is looked up in bfuse_init.  hi - lo above
- * BFUSE_NOALLOC_MAX_IDS is refused (BFUSE_ERR_ARG).  Calls on one GPU share that array: calls
- * that overlap on one GPU race. */
+ * callers that cannot allocate device memory where they call -- tight serving loops, harnesses that
+ * forbid hipMalloc.  Same arguments and results; the two tables are staged in a fixed device array of
+ * the library (2 x BFUSE_NOALLOC_MAX_IDS ints = 2 MiB per GPU, held until the process ends) whose
+ * address is looked up in bfuse_init.  Like the allocating entry point it is synchronous: it launches
+ * on the default stream and copies the tables into the caller's host arrays before it returns, so it
+ * is not a call to make while a stream is being captured into a graph.  hi - lo above
+ * BFUSE_NOALLOC_MAX_IDS is refused (BFUSE_ERR_ARG).  Calls on one GPU share that array: calls that
+ * overlap on one GPU race. */
 #define BFUSE_NOALLOC_MAX_IDS 262144
 int bfuse_map_blocks_device_noalloc(const bfuse_block_plan* plan, int lo, int hi, int* kernel_out, int* virt_out);
 
@@ -149,6 +153,8 @@ typedef struct {
     char side_more[BFUSE_MAX_KERNELS - 2][64];   /* fused kernels of more than two: the third, fourth standalone kernel */
 } bfuse_kernel_info;
 
+/* bfuse_kernel_count / bfuse_kernel_at enumerate every kernel except the library's self-test operators
+ * (names starting with `selftest_`), which bfuse_kernel_find still finds by name. */
 int bfuse_kernel_count(void);
 int bfuse_kernel_at(int index, bfuse_kernel_info* out);
 int bfuse_kernel_find(const char* name, bfuse_kernel_info* out);

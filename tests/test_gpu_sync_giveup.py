@@ -1,7 +1,7 @@
 """The give-up path of the per-side barrier (the gfx950 replacement for the reference's
 `bar.sync id, n`, horizontal-fuser/src/Matchers.cc:288-320), forced from the host.
 
-`sync_probe_a` / `sync_probe_b` are two-wave test operators whose wave 0 takes one barrier more
+`selftest_sync_a` / `selftest_sync_b` are two-wave test operators whose wave 0 takes one barrier more
 than wave 1 when they run under the side barrier.  The wait is bounded, so every kernel ends
 normally; the host lowers the bound so that the give-up comes at once, and every entry point that
 synchronises after such a launch must report BFUSE_ERR_SYNC -- once, with the counter cleared for
@@ -27,7 +27,7 @@ def _want(I, F):
 def test_side_barrier_give_up_is_reported_by_every_synchronising_entry_point():
     I1, F1 = fill_normal(11, 512, 0, 1), fill_normal(12, 512, 0, 1)
     I2, F2 = fill_normal(13, 768, 0, 1), fill_normal(14, 768, 0, 1)
-    with bf.Operation("sync_probe_a", "sync_probe_b") as op:
+    with bf.Operation("selftest_sync_a", "selftest_sync_b") as op:
         # standalone (hardware barrier): well formed
         O1, O2 = op.run_kernel(0, I1, F1).ravel(), op.run_kernel(1, I2, F2).ravel()
         assert bool(np.array_equal(O1, _want(I1, F1))) and bool(np.array_equal(O2, _want(I2, F2)))

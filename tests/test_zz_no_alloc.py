@@ -57,3 +57,21 @@ def test_noalloc_entry_point_limits():
     k_new, v_new = big.table_device_noalloc(0, 1000)
     k_host, v_host = big.table(0, 1000)
     assert np.array_equal(k_new, k_host) and np.array_equal(v_new, v_host)
+
+
+def test_noalloc_entry_point_leaves_free_device_memory_unchanged():
+    """Free device memory as the runtime reports it, before and after repeated calls (one call first, so
+    that whatever the first launch of the kernel loads is already there)."""
+    l = _lib.lib()
+    _lib.check(l.bfuse_init(0))
+    plan = _plan("zigzag", (4, 1), (65536, 1858560))
+    plan.table_device_noalloc(0, MAX_IDS)
+    before = C.c_size_t()
+    _lib.check(l.bfuse_device_memory(C.byref(before), None))
+    for lo in (0, 1000, 500000):
+        plan.table_device_noalloc(lo, lo + MAX_IDS)
+        plan.table_device_noalloc(lo, lo + 77)
+    after = C.c_size_t()
+    _lib.check(l.bfuse_device_memory(C.byref(after), None))
+    print(f"[noalloc] free device memory {before.value} -> {after.value} bytes", flush=True)
+    assert after.value == before.value
