@@ -59,13 +59,16 @@ def test_driver_rejects_unknown_kernels():
 
 
 def test_placement_probe_shows_the_round_robin_the_dispatch_patterns_rely_on():
-    """Consecutive workgroup ids go to consecutive XCDs, and an XCD deals its share evenly over
+    """Consecutive workgroup ids go to consecutive XCDs (starting wherever the hardware's round-robin
+    stands), and an XCD deals its share evenly over
     its CUs -- why chunk = 256 (one chunk per round over all CUs) is the pattern used here and
     why the 1:1 zig-zag parks one operator on the even XCDs."""
     import numpy as np
     from bfuse_project_amd.operation import probe_placement
     p = probe_placement(512, 256, 3000)
-    assert np.all(p["xcc"] == np.arange(512) % 8)
+    # round-robin over the eight XCDs; the XCD the first workgroup lands on depends on where the
+    # previous dispatch stopped, so only the rotation is fixed
+    assert np.all((p["xcc"].astype(np.int64) - int(p["xcc"][0])) % 8 == np.arange(512) % 8)
     key = p["xcc"].astype(np.int64) * 10000 + p["se"].astype(np.int64) * 100 + p["cu"]
     cus, counts = np.unique(key, return_counts=True)
     assert len(cus) <= 256
