@@ -69,15 +69,23 @@ struct GemmF32Dma {
     static constexpr Dims3 BLOCK{64 * NW, 1, 1};
     static constexpr int THREADS = 64 * NW;
     static constexpr bool HAS_BARRIERS = NW > 1;
-    static constexpr int NUNIT = TM * (G4 + G1);
     static constexpr int RING_BYTES = KS * WAVE_BYTES;
-    // The partial tiles meet in LDS in ROUNDS rounds of TMR row blocks each, so that the reduction
-    // buffer is no larger than the rings it reuses: the static LDS size decides whether a second
-    // workgroup (of either side of a fused kernel) fits on the CU.
-    static constexpr int FULL_PART_BYTES = KS * TM * NB * 64 * 16;
+    // The partial tiles meet in LDS.  Component v of every f32x4 accumulator (row 4*rg + v of its
+    // 16-row block) is finished by wave v / OWN: a wave writes the components that other waves own,
+    // reads the other waves' values of its own components and adds them in wave order 0 .. KS-1 with
+    // its register value in its own place -- the order of the sum is fixed, the work (sums, epilogue,
+    // stores) is the same for every wave whatever the tile's mix of 64- and 16-column groups, and a
+    // quarter (KS = 4) of the partial values never leaves its registers.  It happens in ROUNDS rounds of
+    // TMR row blocks each, so that the reduction buffer is no larger than the rings it reuses: the
+    // static LDS size decides whether a second workgroup (of either side of a fused kernel) fits on
+    // the CU.
+    static_assert(KS == 1 || KS == 2 || KS == 4, "the reduction deals the four accumulator components to the waves");
+    static constexpr int OWN = 4 / KS;          // accumulator components a wave finishes
+    static constexpr int FOREIGN = 4 - OWN;     // components it hands to other waves
+    static constexpr int FULL_PART_BYTES = KS * TM * NB * FOREIGN * 256;
     static constexpr int ROUNDS = (KS > 1 && FULL_PART_BYTES > RING_BYTES && TM % 2 == 0) ? 2 : 1;
     static constexpr int TMR = TM / ROUNDS;
-    static constexpr int PART_BYTES = KS > 1 ? KS * TMR * NB * 64 * 16 : 16;
+    static constexpr int PART_BYTES = KS > 1 ? KS * TMR * NB * FOREIGN * 256 : 16;
 
     struct Smem {
         __attribute__((aligned(1024))) unsigned char t[RING_BYTES > PART_BYTES ? RING_BYTES : PART_BYTES];
@@ -331,40 +339,91 @@ struct GemmF32Dma {
         } else {
             // the rings are dead (every wave has consumed its last stage before it gets here, and
             // the barrier below orders the other waves' ring reads before this wave's writes)
-            f32x4(*part)[TMR * NB][64] = reinterpret_cast<f32x4(*)[TMR * NB][64]>(sm.t);
+            float* part = reinterpret_cast<float*>(sm.t) + lane;
 #pragma unroll
             for (int r = 0; r < ROUNDS; ++r) {
                 sync();   // first pass: the rings are dead; later passes: the previous sums have been read
+                if (wave == 0) hand_over<0>(acc, r, part);
+                else if (wave == 1) hand_over<1>(acc, r, part);
+                else if (wave == 2) hand_over<(KS > 2 ? 2 : 0)>(acc, r, part);
+                else hand_over<(KS > 2 ? 3 : 0)>(acc, r, part);
+                sync();
+                if (wave == 0) finish<0>(acc, r, part, C, m0, n0, lane);
+                else if (wave == 1) finish<1>(acc, r, part, C, m0, n0, lane);
+                else if (wave == 2) finish<(KS > 2 ? 2 : 0)>(acc, r, part, C, m0, n0, lane);
+                else finish<(KS > 2 ? 3 : 0)>(acc, r, part, C, m0, n0, lane);
+            }
+        }
+    }
+
+    // word index (before the lane) of component V of block `blk` in the area wave X writes
+    template <int X, int V>
+    static constexpr int part_index(int blk)
+    {
+        static_assert(V / OWN != X, "a wave keeps its own components in registers");
+        return ((X * (TMR * NB) + blk) * FOREIGN + (V < X * OWN ? V : V - OWN)) * 64;
+    }
+    template <int W, int V>
+    __device__ static __forceinline__ void hand_over_one(const f32x4 (&acc)[TM][NB], int r, float* part)
+    {
+        if constexpr (V < 4) {
+            if constexpr (V / OWN != W) {
 #pragma unroll
                 for (int tm = 0; tm < TMR; ++tm)
 #pragma unroll
-                    for (int b = 0; b < NB; ++b) part[wave][tm * NB + b][lane] = acc[r * TMR + tm][b];
-                sync();
-                // every wave of the workgroup finishes units
-#pragma unroll
-                for (int u0 = 0; u0 < NUNIT / ROUNDS; u0 += NW) {
-                    const int u = u0 + wave;
-                    if (u < NUNIT / ROUNDS) {
-                        const int tm = u / (G4 + G1), g = u % (G4 + G1);
-                        if (g < G4) {
-                            f32x4 blk[4];
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) {
-                                f32x4 s = part[0][tm * NB + 4 * g + e][lane];
-#pragma unroll
-                                for (int w = 1; w < KS; ++w) s += part[w][tm * NB + 4 * g + e][lane];
-                                blk[e] = s;
-                            }
-                            store_group4(C, m0, n0, r * TMR + tm, g, blk, lane);
-                        } else {
-                            f32x4 s = part[0][tm * NB + 4 * G4 + (g - G4)][lane];
-#pragma unroll
-                            for (int w = 1; w < KS; ++w) s += part[w][tm * NB + 4 * G4 + (g - G4)][lane];
-                            store_group1(C, m0, n0, r * TMR + tm, g - G4, s, lane);
-                        }
-                    }
-                }
+                    for (int b = 0; b < NB; ++b) part[part_index<W, V>(tm * NB + b)] = acc[r * TMR + tm][b][V];
             }
+            hand_over_one<W, V + 1>(acc, r, part);
+        }
+    }
+    template <int W>
+    __device__ static __forceinline__ void hand_over(const f32x4 (&acc)[TM][NB], int r, float* part)
+    {
+        hand_over_one<W, 0>(acc, r, part);
+    }
+    // sum over the waves in wave order, wave W's own value taken from its register
+    template <int W, int V>
+    __device__ static __forceinline__ float total(float own, const float* part, int blk)
+    {
+        float s;
+        if constexpr (W == 0) s = own;
+        else s = part[part_index<0, V>(blk)];
+        return total_rest<W, V, 1>(s, own, part, blk);
+    }
+    template <int W, int V, int X>
+    __device__ static __forceinline__ float total_rest(float s, float own, const float* part, int blk)
+    {
+        if constexpr (X < KS) {
+            if constexpr (X == W) s += own;
+            else s += part[part_index<X, V>(blk)];
+            return total_rest<W, V, X + 1>(s, own, part, blk);
+        } else {
+            return s;
+        }
+    }
+    template <int W, int T = 0>
+    __device__ static __forceinline__ void finish(const f32x4 (&acc)[TM][NB], int r, const float* part, float* __restrict__ C,
+                                                  int m0, int n0, int lane)
+    {
+        if constexpr (T < OWN) {
+            constexpr int V = W * OWN + T;
+            const int j = lane & 15, rg = lane >> 4;
+#pragma unroll
+            for (int tm = 0; tm < TMR; ++tm) {
+                float* __restrict__ row = C + (size_t)(m0 + (r * TMR + tm) * 16 + 4 * rg + V) * N + n0;
+#pragma unroll
+                for (int g = 0; g < G4; ++g) {
+                    f32x4 o;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        o[e] = epilogue(total<W, V>(acc[r * TMR + tm][4 * g + e][V], part, tm * NB + 4 * g + e));
+                    *reinterpret_cast<f32x4*>(row + g * 64 + 4 * j) = o;
+                }
+#pragma unroll
+                for (int g = 0; g < G1; ++g)
+                    row[G4 * 64 + g * 16 + j] = epilogue(total<W, V>(acc[r * TMR + tm][4 * G4 + g][V], part, tm * NB + 4 * G4 + g));
+            }
+            finish<W, T + 1>(acc, r, part, C, m0, n0, lane);
         }
     }
 
