@@ -26,7 +26,11 @@ Per pair:
   serial_sum_us     sum of the two unfused kernel durations (the reference's "serial",
                     scripts/analyze_test_suite.py:425-428)
   batched_*_us      wall-clock microseconds per launch with K launches queued back to back
-                    (includes dispatch gaps, lets consecutive launches overlap their ramp-up)
+                    (includes dispatch gaps, lets consecutive launches overlap their ramp-up);
+                    fused_over_back_to_back is the ratio of these queued figures
+  best_unfused      the fastest standalone kernels the library holds for the two operators (every
+                    registered tiling / schedule of each is timed queued), those two queued back to back,
+                    and the fused kernel's queued time over that: the baseline a user would really run
   roofline          algorithmic flops (or bytes) of the pair / fused duration vs the MI355X peak;
                     `traffic` is HBM bytes per launch from the rocprofv3 --pmc summary named in
                     `traffic_source` (not measured by this run); `same_kernel_constant_operands` (pairs with a
@@ -177,6 +181,42 @@ def pick_fusion(number, spec):
     return k1, k2, hk, sfx, note
 
 
+def best_unfused(k1, k2, inputs, R, BW, b_ser, b_k1, b_k2):
+    """Queued time of the fastest standalone kernels for the two operators of a pair.  Every registered
+    alternative of each side is timed queued on its own; if the fastest ones are not (k1, k2), that pair is
+    then timed queued back to back (median of three runs).  b_ser / b_k1 / b_k2: the figures already
+    measured for (k1, k2)."""
+    import bfuse_project_amd as bf
+    from bfuse_project_amd.workloads import BASELINE_NOTES, standalone_alternatives
+    I1, F1, I2, F2 = inputs
+    alone = [{k1: b_k1}, {k2: b_k2}]
+    for side, (mine, partner) in enumerate(((k1, k2), (k2, k1))):
+        for alt in standalone_alternatives(mine):
+            if alt == mine:
+                continue
+            pair = (alt, partner) if side == 0 else (partner, alt)
+            with bf.Operation(*pair) as op:
+                op.upload(0, I1, F1)
+                op.upload(1, I2, F2)
+                alone[side][alt] = op.time_batched("kernel1" if side == 0 else "kernel2", warmup=BW, reps=R)
+    pick = [min(d, key=d.get) for d in alone]
+    out = {"kernel1": pick[0], "kernel2": pick[1],
+           "alone_us": [{k: round(v, 3) for k, v in d.items()} for d in alone],
+           "is_the_fused_kernels_own_pair": (pick[0], pick[1]) == (k1, k2)}
+    if (pick[0], pick[1]) == (k1, k2):
+        out["batched_back_to_back_us"] = round(b_ser, 3)
+    else:
+        with bf.Operation(pick[0], pick[1]) as op:
+            op.upload(0, I1, F1)
+            op.upload(1, I2, F2)
+            q = [op.time_batched("serial", warmup=BW, reps=R) for _ in range(3)]
+        out["batched_back_to_back_us"] = round(float(np.median(q)), 3)
+    notes = [f"{k}: {BASELINE_NOTES[k]}" for k in pick if k in BASELINE_NOTES]
+    if notes:
+        out["notes"] = notes
+    return out
+
+
 def measure(number, K, W, spec, ceilings, power_check=True):
     import bfuse_project_amd as bf
     from bfuse_project_amd import tuner
@@ -260,6 +300,13 @@ def measure(number, K, W, spec, ceilings, power_check=True):
                      "frac": round(pair.flops / float(t_c.mean()) * 1e-6 / pair.peak, 4)}
             op.upload(side, inputs[2 * side], inputs[2 * side + 1])
 
+    # The honest baseline: for each side, the fastest standalone kernel the library holds for that operator
+    # at that shape (another tiling or schedule of it), found by timing them queued, and then those two
+    # queued back to back.  The headline sides are the kernels the fusion was built from, which is not
+    # always the fastest way to run each operator alone.
+    best = best_unfused(k1, k2, inputs, R, BW, b_ser, b_k1, b_k2)
+    best["batched_fused_over_best_unfused"] = round(b_f / best["batched_back_to_back_us"], 4)
+
     # fused forms the configuration names that are not the measured kernel, timed beside it
     extra = {}
     for label, a1, a2, akind, asuffix in BESIDE.get(number, []):
@@ -306,13 +353,17 @@ def measure(number, K, W, spec, ceilings, power_check=True):
         "kernel1_us": round(float(t_a.mean()), 3),
         "kernel2_us": round(float(t_b.mean()), 3),
         "parallel_streams_us": round(float(t_par.mean()), 3),
-        "fused_over_back_to_back": round(fused_us / back_to_back, 4),
+        # first start -> second end includes the gap between the two launches (several us when each launch
+        # waits for its own completion signal); the queued ratio below is the one quoted
+        "fused_over_back_to_back_incl_launch_gap": round(fused_us / back_to_back, 4),
         "fused_over_serial_sum": round(fused_us / serial_sum, 4),
         "batched_fused_us": round(b_f, 3),
         "batched_back_to_back_us": round(b_ser, 3),
         "batched_kernel1_us": round(b_k1, 3),
         "batched_kernel2_us": round(b_k2, 3),
         "batched_fused_over_back_to_back": round(b_f / b_ser, 4),
+        "fused_over_back_to_back": round(b_f / b_ser, 4),
+        "best_unfused": best,
         "batched_rounds": {"fused_us": [round(x, 3) for x in q_f], "back_to_back_us": [round(x, 3) for x in q_ser]},
         "ms_per_step": round(wall_ms, 6),
         "baseline_reps": R,
@@ -403,6 +454,7 @@ def main():
         "bit_exact_vs_unfused": all(p["bit_exact_vs_unfused"] for p in pairs.values()),
         "fused_over_back_to_back": t["fused_over_back_to_back"],
         "batched_fused_over_back_to_back": t["batched_fused_over_back_to_back"],
+        "batched_fused_over_best_unfused": t["best_unfused"]["batched_fused_over_best_unfused"],
         "roofline": t["roofline"],
         "hbm_copy_GBps": ceilings["hbm_copy_GBps"],
         "measured_ceilings": ceilings,
@@ -412,7 +464,11 @@ def main():
     # kernels launched back to back (queued: the strongest form of that baseline)
     tgt = {n: pairs[n]["batched_fused_over_back_to_back"] for n in ("1", "2", "3", "4") if n in pairs}
     if tgt:
-        out["target"] = {"queued_fused_over_back_to_back_at_most": 0.9, "pairs": tgt, "met": all(v <= 0.9 for v in tgt.values())}
+        # the same target against the fastest standalone kernels the library holds for each operator
+        # (not always the ones the fused kernel was built from): stated beside it
+        vs_best = {n: pairs[n]["best_unfused"]["batched_fused_over_best_unfused"] for n in tgt}
+        out["target"] = {"queued_fused_over_back_to_back_at_most": 0.9, "pairs": tgt, "met": all(v <= 0.9 for v in tgt.values()),
+                         "pairs_vs_best_unfused": vs_best, "met_vs_best_unfused": all(v <= 0.9 for v in vs_best.values())}
     if not args.pair:
         from bfuse_project_amd.workloads import GROUPS
         out["groups"] = {g: measure_group(g, K, W) for g in GROUPS}

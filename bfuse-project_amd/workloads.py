@@ -215,6 +215,27 @@ TRAFFIC_SOURCE = {
     "gemm_bf16_512x4096x14336_rmsnorm_rope_bf16_512x4096_w2_fused_hfuse": "profiles/pair5_gemm_bf16_rmsnorm_rope_hfuse.md",
 }
 
+def standalone_alternatives(name: str) -> List[str]:
+    """Every standalone kernel of the registry that computes what `name` computes: the same operator at the
+    same shapes (a variant suffix such as _s3, _k4, _w2 names another tiling or schedule of it)."""
+    import re
+    from .operation import kernel_info, list_kernels
+    me = kernel_info(name)
+    base = re.sub(r"_[a-z]+\d*$", "", name)
+    out = []
+    for k in list_kernels():
+        if k.kind != 0 or (k.name != base and not re.fullmatch(re.escape(base) + r"_[a-z]+\d*", k.name)):
+            continue
+        if tuple(map(tuple, k.shapes)) == tuple(map(tuple, me.shapes)) and tuple(k.elem_bytes) == tuple(me.elem_bytes):
+            out.append(k.name)
+    return out
+
+
+# Standalone kernels that are not a like-for-like baseline for a pair, with the reason (reported, still timed)
+BASELINE_NOTES = {
+    "gemm_f32_512x512x512_k4": "four waves split K: outside configuration 1's 128/128 thread split (its GEMM side is two waves)",
+}
+
 # what bounds a pair from below whatever the fusion does, stated in the benchmark line
 FLOORS = {
     1: {"us": 3.9, "why": "the configuration's 128/128 thread split gives the GEMM side two waves = two of a CU's four SIMDs; "

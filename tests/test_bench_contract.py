@@ -53,6 +53,13 @@ def test_one_json_line_covering_all_five_pairs():
     assert "same_kernel_constant_operands" not in d["pairs"]["1"]["roofline"]
     tg = d["target"]          # the 0.9 target of configurations 1-4, stated whether met or not
     assert sorted(tg["pairs"]) == ["1", "2", "3", "4"] and tg["met"] == all(v <= 0.9 for v in tg["pairs"].values())
+    assert sorted(tg["pairs_vs_best_unfused"]) == ["1", "2", "3", "4"] and tg["met_vs_best_unfused"] == all(v <= 0.9 for v in tg["pairs_vs_best_unfused"].values())
+    for n, p in d["pairs"].items():          # the fastest standalone kernels of each operator, and the fused kernel against them
+        bu = p["best_unfused"]
+        assert bu["kernel1"] in bu["alone_us"][0] and bu["kernel2"] in bu["alone_us"][1] and bu["batched_back_to_back_us"] > 0
+        assert abs(bu["batched_fused_over_best_unfused"] - p["batched_fused_us"] / bu["batched_back_to_back_us"]) < 1e-3
+        assert p["fused_over_back_to_back"] == p["batched_fused_over_back_to_back"]
+    assert "gemm_gelu_f32_512x768x3072_s3" in d["pairs"]["4"]["best_unfused"]["alone_us"][1]
     assert all(len(p["batched_rounds"]["fused_us"]) == len(p["batched_rounds"]["back_to_back_us"]) >= 3 for p in d["pairs"].values())
     cb = d["cpu_baseline"]
     assert cb["kind"] == "port" and cb["cores"] >= 1 and cb["value"] > 0 and cb["sample"]
