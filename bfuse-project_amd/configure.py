@@ -10,13 +10,22 @@ shapes are compile-time, and the same three config files are written for what re
 
     python -m bfuse_project_amd.configure example.yaml -o OUT [--dtype f32|bf16] [--skip-missing]
 
+Arithmetic and weight layout are part of what an id resolves to, and are written down per id: by default
+every id resolves to an fp32 kernel, the reference's arithmetic; `--dtype bf16` takes the bf16 kernel where
+the library holds one and says which ids stayed fp32.  The reference's `dense` weight is (out, in)
+(:21-26).  The bf16 GEMMs take it like that; the fp32 GEMMs take [in, out], so a weight in the reference's
+layout goes through the library's `transpose32_<out>x<in>` kernel once when it is loaded -- `info.yaml`
+names that kernel, and resolution fails if a kernel's registered shapes are not the reference's shapes up
+to that one stated transposition.
+
   OUT/config/kernels.yaml   id -> {KernelName (registry name), HasBarriers, GridDim, BlockDim, Reg, ExecTime}
                             in the fuser's schema (horizontal-fuser/include/fuse/Utils.h:70-112); launch shape and
                             barrier flag are the kernel's own, Reg is the reference's don't-care 32 unless a
                             device is present
   OUT/config/fusions.yaml   every (set 0, set 1) pair as {File, Kernels}; File names the library
   OUT/config/info.yaml      the suite description for `python -m bfuse_project_amd.suite`: the two sets
-                            with registry names, the user's KernelInfo block kept beside them
+                            with registry names, the user's KernelInfo block kept beside them, and `Resolved`:
+                            id -> {kernel, dtype, weight_layout, weight_transpose}
   OUT/config/fused.yaml     for every pair, the fused kernels the library holds for it
 
 An id no registry kernel matches is reported with the lines that would instantiate it; the run then
@@ -59,20 +68,64 @@ def shapes_of(kernel_id: str, args) -> Tuple[tuple, tuple, tuple]:
 
 
 def candidate_names(kernel_id: str, args, dtype: Optional[str]) -> List[str]:
-    """Registry names that implement the operator at exactly these arguments, in order of preference."""
+    """Registry names that implement the operator at exactly these arguments, in order of preference:
+    fp32 (the reference's arithmetic) unless bf16 is asked for, then bf16 first and fp32 behind it."""
     op = operator_of(kernel_id)
     shapes_of(kernel_id, args)   # validates
-    types = [dtype] if dtype else ["f32", "bf16"]
+    types = ["bf16", "f32"] if dtype == "bf16" else ["f32"]
     if op == "dense":
         b, i, o = args
         return [f"gemm_{t}_{b}x{i}x{o}" for t in types]
     if op == "conv2d":
         n, h, w, co, ci, kh, kw, stride, pad = args
-        if (n, kh, kw, stride, pad) == (1, 3, 3, 1, 1):
-            return [f"conv3x3_{t}_{ci}x{h}x{w}_{co}" for t in types]
-        return []
+        if n != 1:
+            return []
+        names = []
+        for t in types:
+            if (kh, kw, stride, pad) == (3, 3, 1, 1):
+                names.append(f"conv3x3_{t}_{ci}x{h}x{w}_{co}")       # the kernel tuned for this case, where instantiated
+            names.append(f"conv{kh}x{kw}s{stride}p{pad}_{t}_{ci}x{h}x{w}_{co}")
+        return names
     b, m, k, n = args
     return [f"bgemm_{t}_{b}x{m}x{k}x{n}" for t in types]
+
+
+# kernel families whose dense weight is stored [in, out] (= [K, N]) instead of the reference's (out, in): the
+# fp32 GEMM sides (csrc/ops_gemm_f32*.h); the bf16 GEMM takes (out, in) as it is
+WEIGHT_IS_IN_OUT = {"gemm_f32": True, "gemm_bf16": False}
+
+
+def _dims(shape) -> tuple:
+    """A shape without its padding of trailing ones."""
+    d = [int(x) for x in shape]
+    while len(d) > 1 and d[-1] == 1:
+        d.pop()
+    return tuple(d)
+
+
+def describe(kernel_id: str, args, kernel, registry) -> dict:
+    """What the id resolved to: kernel, arithmetic, weight layout.  The kernel's registered shapes must be the
+    reference's (shapes_of), except that a dense weight may be registered transposed -- [in, out] instead of
+    (out, in) -- when the library also holds the kernel that transposes it; anything else is an error."""
+    data, weight, out = shapes_of(kernel_id, args)
+    have = [_dims(sh) for sh in kernel.shapes]
+    want = [_dims(data), _dims(weight), _dims(out)]
+    dtype = {4: "f32", 2: "bf16"}.get(kernel.elem_bytes[0], f"{kernel.elem_bytes[0]} bytes")
+    if have[0] != want[0] or have[2] != want[2]:
+        raise ValueError(f"{kernel_id}: {kernel.name} is registered for data {have[0]} -> {have[2]}, the id asks for {want[0]} -> {want[2]}")
+    info = {"kernel": kernel.name, "dtype": dtype, "weight_layout": "reference", "weight_transpose": None}
+    if operator_of(kernel_id) == "dense" and WEIGHT_IS_IN_OUT.get(kernel.name.split("_")[0] + "_" + dtype, False):
+        # the kernel family takes [in, out]; a square weight has the same shape either way, so the family decides
+        if have[1] != want[1][::-1]:
+            raise ValueError(f"{kernel_id}: {kernel.name} takes a weight of shape {have[1]}, [in, out] of the id's is {want[1][::-1]}")
+        tname = f"transpose32_{want[1][0]}x{want[1][1]}"
+        if tname not in registry:
+            raise ValueError(f"{kernel_id}: {kernel.name} takes its weight as [in, out] {have[1]} (the reference's is (out, in)) and the library has no {tname}")
+        info.update(weight_layout="[in, out]: the reference's (out, in) weight transposed once on load", weight_transpose=tname)
+        return info
+    if have[1] != want[1]:
+        raise ValueError(f"{kernel_id}: {kernel.name} takes a weight of shape {have[1]}, the id's is {want[1]}")
+    return info
 
 
 def instantiation_hint(kernel_id: str, args) -> str:
@@ -83,10 +136,10 @@ def instantiation_hint(kernel_id: str, args) -> str:
                 f"({{{{{b}, {i}, 1, 1}}, 4}}), ({{{{{i}, {o}, 1, 1}}, 4}}), ({{{{{b}, {o}, 1, 1}}, 4}}))  in csrc/kernels_*.hip")
     if op == "conv2d":
         n, h, w, co, ci, kh, kw, stride, pad = args
-        if (n, kh, kw, stride, pad) == (1, 3, 3, 1, 1):
-            return (f"using Conv = Conv3x3F32Lds<{ci}, {co}, {h}, {w}, ...>;  BFUSE_KERNEL(conv3x3_f32_{ci}x{h}x{w}_{co}, Conv, ...)  "
-                    f"in csrc/kernels_*.hip")
-        return "the library's convolution is 3x3, stride 1, padding 1, batch 1 (csrc/ops_conv.h)"
+        if n != 1:
+            return "the library's convolutions are batch 1 (csrc/ops_conv_general.h)"
+        return (f"using Conv = ConvF32Lds<{ci}, {co}, {h}, {w}, {kh}, {kw}, {stride}, {pad}, BM, PB, KS>;  "
+                f"BFUSE_KERNEL(conv{kh}x{kw}s{stride}p{pad}_f32_{ci}x{h}x{w}_{co}, Conv, ...)  in csrc/kernels_*.hip")
     b, m, k, n = args
     return (f"using Bgemm = GemmF32<{m}, {n}, {k}, BM, BN, KS, kEpiNone, 2, 1, true, {b}>;  BFUSE_KERNEL(bgemm_f32_{b}x{m}x{k}x{n}, Bgemm, "
             f"({{{{{b}, {m}, {k}, 1}}, 4}}), ({{{{{b}, {n}, {k}, 1}}, 4}}), ({{{{{b}, {m}, {n}, 1}}, 4}}))  in csrc/kernels_*.hip")
@@ -113,7 +166,8 @@ def load_user_config(path: str) -> dict:
 
 
 def resolve(doc: dict, registry: Dict[str, object], dtype: Optional[str] = None):
-    """({id: registry kernel}, {id: hint}) for every id the two sets name."""
+    """({id: registry kernel}, {id: hint}) for every id the two sets name.  A kernel whose registered shapes are
+    not the id's (up to the stated weight transposition of fp32 dense kernels) raises ValueError."""
     found, missing = {}, {}
     for s in doc["FusionSet"]:
         for kid in s["Set"]:
@@ -122,6 +176,7 @@ def resolve(doc: dict, registry: Dict[str, object], dtype: Optional[str] = None)
             args = doc["KernelInfo"][kid]
             hit = next((registry[n] for n in candidate_names(kid, args, dtype) if n in registry), None)
             if hit is not None:
+                describe(kid, args, hit, registry)      # shapes checked here, before anything is written
                 found[kid] = hit
             else:
                 missing[kid] = instantiation_hint(kid, args)
@@ -163,19 +218,21 @@ def configure(path: str, out: str, dtype: Optional[str] = None, skip_missing: bo
     with open(os.path.join(config_dir, "fused.yaml"), "w") as f:
         yaml.safe_dump(fused, f, sort_keys=False)
 
+    resolved = {kid: describe(kid, doc["KernelInfo"][kid], found[kid], registry) for kid in found}
     info = {"FusionSet": [{"Set": [found[k].name for k in s]} for s in sets],
             "KernelInfo": {kid: list(doc["KernelInfo"][kid]) for kid in found},
-            "Resolved": {kid: found[kid].name for kid in found}}
+            "Resolved": resolved}
     with open(os.path.join(config_dir, "info.yaml"), "w") as f:
         yaml.safe_dump(info, f, sort_keys=False)
-    return {"found": {k: v.name for k, v in found.items()}, "missing": missing, "pairs": pairs, "fused": fused}
+    return {"found": {k: v.name for k, v in found.items()}, "missing": missing, "pairs": pairs, "fused": fused, "resolved": resolved}
 
 
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
     ap.add_argument("config", help="config file path for generate test suite")
     ap.add_argument("-o", dest="file", default="test-suite", help="output directory of the generated suite configuration")
-    ap.add_argument("--dtype", choices=("f32", "bf16"), default=None, help="arithmetic type of the kernels to resolve to (default: f32, else bf16)")
+    ap.add_argument("--dtype", choices=("f32", "bf16"), default=None,
+                    help="arithmetic type to resolve to: f32 (default, the reference's) or bf16 where the library holds a bf16 kernel (the others stay f32 and are listed)")
     ap.add_argument("--skip-missing", action="store_true", help="drop ids the library has no kernel for instead of failing")
     args = ap.parse_args(argv)
     if not os.path.exists(args.config):
@@ -186,8 +243,13 @@ def main(argv=None) -> int:
     except (ValueError, LookupError, FileExistsError) as e:
         print(f"configure: {e}", file=sys.stderr)
         return 1
-    for kid, name in r["found"].items():
-        print(f"{kid} -> {name}")
+    for kid, d in r["resolved"].items():
+        layout = f", weight {d['weight_layout']} ({d['weight_transpose']})" if d["weight_transpose"] else ""
+        print(f"{kid} -> {d['kernel']}  [{d['dtype']}{layout}]")
+    if args.dtype == "bf16":
+        kept = [kid for kid, d in r["resolved"].items() if d["dtype"] != "bf16"]
+        if kept:
+            print(f"no bf16 kernel, resolved to f32: {', '.join(kept)}", file=sys.stderr)
     for kid, hint in r["missing"].items():
         print(f"{kid}: dropped, no kernel ({hint})", file=sys.stderr)
     print(f"{len(r['pairs'])} pairs, {sum(1 for v in r['fused'].values() if v)} with a fused kernel; wrote {os.path.join(args.file, 'config')}")

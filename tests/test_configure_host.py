@@ -29,10 +29,18 @@ def test_shapes_follow_the_reference_formulas():
 
 def test_example_config_resolves_and_writes_the_fusers_files(tmp_path):
     out = str(tmp_path / "suite")
-    r = configure.configure(EXAMPLE, out)
+    # fp32, the reference's arithmetic, unless bf16 is asked for; what each id resolved to is written down
+    r32 = configure.configure(EXAMPLE, str(tmp_path / "suite32"))
+    assert r32["found"]["dense_6"] == "gemm_f32_512x4096x14336" and all(d["dtype"] == "f32" for d in r32["resolved"].values())
+    assert r32["resolved"]["dense_6"]["weight_transpose"] == "transpose32_14336x4096" and r32["resolved"]["conv2d_1"]["weight_transpose"] is None
+    r = configure.configure(EXAMPLE, out, dtype="bf16")
     assert r["found"] == {"dense_0": "gemm_f32_512x512x512", "dense_3": "gemm_f32_512x768x2304",
                           "conv2d_1": "conv3x3_f32_64x56x56_64", "dense_6": "gemm_bf16_512x4096x14336"}
     assert r["missing"] == {} and len(r["pairs"]) == 4
+    assert r["resolved"]["dense_6"] == {"kernel": "gemm_bf16_512x4096x14336", "dtype": "bf16", "weight_layout": "reference", "weight_transpose": None}
+    assert r["resolved"]["dense_3"]["dtype"] == "f32" and r["resolved"]["dense_3"]["weight_transpose"] == "transpose32_2304x768"
+    with open(os.path.join(out, "config", "info.yaml")) as f:
+        assert yaml.safe_load(f)["Resolved"] == r["resolved"]
     kernels = bf.load_kernels_yaml(os.path.join(out, "config", "kernels.yaml"))      # the fuser's schema loads it
     fusions = bf.load_fusions_yaml(os.path.join(out, "config", "fusions.yaml"))
     assert kernels["dense_3"].KernelName == "gemm_f32_512x768x2304" and kernels["dense_3"].GridDim == (256, 1, 1)
@@ -54,17 +62,18 @@ def test_example_config_resolves_and_writes_the_fusers_files(tmp_path):
 def test_unknown_shapes_are_reported_with_the_line_that_would_add_them(tmp_path):
     cfg = tmp_path / "c.yaml"
     cfg.write_text("FusionSet:\n  - Set: [dense_0, dense_9]\n  - Set: [conv2d_0, conv2d_1, bgemm_9]\n"
-                   "KernelInfo:\n  dense_0: [512, 512, 512]\n  dense_9: [512, 100, 100]\n  conv2d_0: [1, 224, 224, 64, 3, 7, 7, 2, 3]\n"
-                   "  conv2d_1: [1, 56, 56, 64, 64, 3, 3, 1, 1]\n  bgemm_9: [16, 208, 208, 64]\n")
+                   "KernelInfo:\n  dense_0: [512, 512, 512]\n  dense_9: [512, 100, 100]\n  conv2d_0: [1, 30, 30, 8, 16, 5, 5, 1, 2]\n"
+                   "  conv2d_1: [1, 56, 56, 64, 64, 3, 3, 1, 1]\n  bgemm_9: [3, 100, 100, 100]\n")
     with pytest.raises(LookupError) as e:
         configure.configure(str(cfg), str(tmp_path / "a"))
     assert "dense_9" in str(e.value) and "gemm_f32_512x100x100" in str(e.value) and "bgemm_9" in str(e.value) and not (tmp_path / "a").exists()
+    assert "conv5x5s1p2_f32_16x30x30_8" in str(e.value)
     r = configure.configure(str(cfg), str(tmp_path / "b"), skip_missing=True)
     assert r["found"] == {"dense_0": "gemm_f32_512x512x512", "conv2d_1": "conv3x3_f32_64x56x56_64"} and sorted(r["missing"]) == ["bgemm_9", "conv2d_0", "dense_9"]
     assert r["pairs"] == [("dense_0", "conv2d_1")]
-    # the bf16 kernel only when asked for, or when there is no fp32 one
-    r2 = configure.configure(EXAMPLE, str(tmp_path / "c2"), dtype="f32", skip_missing=True)
-    assert "dense_6" in r2["missing"] and r2["found"]["dense_3"] == "gemm_f32_512x768x2304"
+    # the bf16 kernel only when asked for
+    r2 = configure.configure(EXAMPLE, str(tmp_path / "c2"), dtype="f32")
+    assert r2["found"]["dense_6"] == "gemm_f32_512x4096x14336" and r2["found"]["dense_3"] == "gemm_f32_512x768x2304"
 
 
 def test_malformed_configs_are_refused(tmp_path):
@@ -79,30 +88,56 @@ def test_malformed_configs_are_refused(tmp_path):
 def test_command_line(tmp_path):
     out = str(tmp_path / "cli")
     r = subprocess.run([sys.executable, "-m", "bfuse_project_amd.configure", EXAMPLE, "-o", out], capture_output=True, text=True, cwd=ROOT)
-    assert r.returncode == 0 and "dense_6 -> gemm_bf16_512x4096x14336" in r.stdout and os.path.exists(os.path.join(out, "config", "kernels.yaml"))
+    assert r.returncode == 0 and "dense_6 -> gemm_f32_512x4096x14336  [f32, weight [in, out]" in r.stdout and os.path.exists(os.path.join(out, "config", "kernels.yaml"))
+    r = subprocess.run([sys.executable, "-m", "bfuse_project_amd.configure", EXAMPLE, "-o", out + "_bf16", "--dtype", "bf16"], capture_output=True, text=True, cwd=ROOT)
+    assert r.returncode == 0 and "dense_6 -> gemm_bf16_512x4096x14336  [bf16]" in r.stdout and "no bf16 kernel, resolved to f32: dense_0, dense_3, conv2d_1" in r.stderr
     r = subprocess.run([sys.executable, "-m", "bfuse_project_amd.configure", os.path.join(out, "nope.yaml")], capture_output=True, text=True, cwd=ROOT)
     assert r.returncode == 1 and "doesn't exist" in r.stderr
 
 
+def test_a_kernel_registered_for_other_shapes_than_the_ids_is_refused():
+    """The registry kernel's shapes are checked against the reference's shape formulas: a dense kernel of the
+    [in, out] family with a weight of another shape, or data of another shape, does not resolve silently."""
+    from types import SimpleNamespace as NS
+    reg = {"transpose32_96x64": NS(name="transpose32_96x64")}
+    good = NS(name="gemm_f32_32x64x96", shapes=((32, 64, 1, 1), (64, 96, 1, 1), (32, 96, 1, 1)), elem_bytes=(4, 4, 4))
+    d = configure.describe("dense_0", [32, 64, 96], good, reg)
+    assert d["dtype"] == "f32" and d["weight_transpose"] == "transpose32_96x64" and d["weight_layout"].startswith("[in, out]")
+    wrong_w = NS(name="gemm_f32_32x64x96", shapes=((32, 64, 1, 1), (96, 64, 1, 1), (32, 96, 1, 1)), elem_bytes=(4, 4, 4))
+    with pytest.raises(ValueError, match="weight"):
+        configure.describe("dense_0", [32, 64, 96], wrong_w, reg)
+    with pytest.raises(ValueError, match="no transpose32_96x64"):
+        configure.describe("dense_0", [32, 64, 96], good, {})
+    wrong_d = NS(name="gemm_f32_32x64x96", shapes=((16, 64, 1, 1), (64, 96, 1, 1), (16, 96, 1, 1)), elem_bytes=(4, 4, 4))
+    with pytest.raises(ValueError, match="registered for data"):
+        configure.describe("dense_0", [32, 64, 96], wrong_d, reg)
+    nk = NS(name="gemm_bf16_32x64x96", shapes=((32, 64, 1, 1), (96, 64, 1, 1), (32, 96, 1, 1)), elem_bytes=(2, 2, 2))
+    assert configure.describe("dense_0", [32, 64, 96], nk, {}) == {"kernel": "gemm_bf16_32x64x96", "dtype": "bf16", "weight_layout": "reference", "weight_transpose": None}
+    # a square weight has the same shape in both layouts: the kernel family decides, not the shape
+    sq = NS(name="gemm_f32_8x64x64", shapes=((8, 64, 1, 1), (64, 64, 1, 1), (8, 64, 1, 1)), elem_bytes=(4, 4, 4))
+    assert configure.describe("dense_1", [8, 64, 64], sq, {"transpose32_64x64": 1})["weight_transpose"] == "transpose32_64x64"
+
+
 @pytest.mark.skipif(not os.path.isdir(REF_EXAMPLES), reason="the reference's example configs are not on this machine")
-@pytest.mark.parametrize("name,want", [("llm.yaml", {"dense_0": "gemm_f32_512x768x768", "dense_1": "gemm_f32_512x768x3072", "dense_2": "gemm_f32_512x3072x768",
-                                                     "dense_3": "gemm_f32_512x768x2304", "dense_4": "gemm_bf16_512x4096x4096", "dense_5": "gemm_f32_512x4096x1024",
-                                                     "dense_6": "gemm_bf16_512x4096x14336", "dense_7": "gemm_bf16_512x14336x4096",
-                                                     "bgemm_0": "bgemm_f32_12x512x64x512", "bgemm_1": "bgemm_f32_12x512x512x64",
-                                                     "bgemm_2": "bgemm_f32_32x512x128x512", "bgemm_3": "bgemm_f32_32x512x512x128"}),
-                                       ("resnet-18.yaml", {"conv2d_1": "conv3x3_f32_64x56x56_64", "conv2d_4": "conv3x3_f32_128x28x28_128"})])
-def test_the_references_own_example_configs(tmp_path, name, want):
-    """The reference's examples (read in place) ship with empty fusion sets: every id goes into both
-    sets, as its benchmark.yaml does, and the ids of the benchmark configurations resolve."""
+@pytest.mark.parametrize("name,count", [("llm.yaml", 26), ("resnet-18.yaml", 12)])
+def test_the_references_own_example_configs_resolve_completely(tmp_path, name, count):
+    """The reference's examples (read in place) ship with empty fusion sets: every id goes into both sets, as its
+    benchmark.yaml does, and EVERY id resolves without --skip-missing -- in fp32, the reference's arithmetic."""
     with open(os.path.join(REF_EXAMPLES, name)) as f:
         doc = yaml.safe_load(f)
     ids = list(doc["KernelInfo"])
+    assert len(ids) == count
     doc["FusionSet"] = [{"Set": ids}, {"Set": ids}]
     p = tmp_path / name
     p.write_text(yaml.safe_dump(doc))
-    for kid in ids:
-        configure.shapes_of(kid, doc["KernelInfo"][kid])          # every entry is well formed
-    r = configure.configure(str(p), str(tmp_path / "o"), skip_missing=True)
-    for kid, kname in want.items():
-        assert r["found"][kid] == kname
-    assert set(r["found"]) | set(r["missing"]) == set(ids)
+    r = configure.configure(str(p), str(tmp_path / "o"))
+    assert set(r["found"]) == set(ids) and not r["missing"]
+    assert all(d["dtype"] == "f32" for d in r["resolved"].values())
+    reg = {k.name: k for k in bf.operation.list_kernels()}
+    for kid in ids:          # and each to a kernel of exactly the reference's shapes
+        data, weight, out = configure.shapes_of(kid, doc["KernelInfo"][kid])
+        k = reg[r["found"][kid]]
+        assert configure._dims(k.shapes[0]) == configure._dims(data) and configure._dims(k.shapes[2]) == configure._dims(out)
+    if name == "llm.yaml":
+        rb = configure.configure(str(p), str(tmp_path / "ob"), dtype="bf16")
+        assert {k for k, d in rb["resolved"].items() if d["dtype"] == "bf16"} == {"dense_4", "dense_6", "dense_7"}

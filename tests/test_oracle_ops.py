@@ -128,6 +128,28 @@ def test_conv2d():
     assert np.array_equal(y[1:, :-1], x[0, 0][:-1, 1:]) and np.all(y[0] == 0) and np.all(y[:, -1] == 0)
 
 
+@pytest.mark.parametrize("ci,co,h,w,kh,kw,s,p", [(3, 8, 20, 18, 7, 7, 2, 3), (6, 4, 9, 9, 1, 1, 1, 0), (6, 4, 10, 8, 1, 1, 2, 0),
+                                                 (5, 3, 14, 14, 3, 3, 2, 1), (4, 6, 7, 7, 3, 3, 1, 1), (2, 2, 11, 6, 5, 3, 3, 2)])
+def test_conv2d_for_every_argument_list_of_the_resnet_layers(ci, co, h, w, kh, kw, s, p):
+    """Filter sizes, strides and paddings of the reference's resnet-18.yaml (7x7 stride 2 padding 3; 1x1 with
+    stride 1 and 2 and no padding; 3x3 stride 2; 3x3 on 7x7 images) and an asymmetric one, against the library
+    routine, plus a closed form: a one-hot filter picks input pixels with the stride and the padding offset."""
+    r = _rng(80 + kh * 10 + s)
+    x = r.normal(0, 1, (1, ci, h, w)).astype(np.float32)
+    wt = r.normal(0, 0.1, (co, ci, kh, kw)).astype(np.float32)
+    want = F.conv2d(torch.from_numpy(x).double(), torch.from_numpy(wt).double(), stride=s, padding=p).float().numpy()
+    got = orf.conv2d(x, wt, s=s, p=p)
+    assert got.shape == want.shape == (1, co, (h - kh + 2 * p) // s + 1, (w - kw + 2 * p) // s + 1)
+    assert np.max(np.abs(got - want)) <= 1e-6
+    sel = np.zeros((1, ci, kh, kw), np.float32)
+    a, b = kh - 1, kw // 2
+    sel[0, ci - 1, a, b] = 1
+    y = orf.conv2d(x, sel, s=s, p=p)[0, 0]
+    xp = np.pad(x[0, ci - 1], p)
+    oh, ow = y.shape
+    assert np.array_equal(y, xp[a:a + s * oh:s, b:b + s * ow:s])
+
+
 def test_softmax_causal():
     r = _rng(9)
     x = (r.normal(0, 1, (3, 33, 33)) / 8).astype(np.float32)
