@@ -124,30 +124,84 @@ class FusionContext:
 
 
 def choose_fusion(a: KernelInfo, b: KernelInfo, lds_a: int, lds_b: int, cus: int = 256) -> dict:
-    """Picks hfuse vs bfuse and a block ratio from each side's footprint.
+    """Picks hfuse vs bfuse vs no fusion from each side's footprint (and its ExecTime where known).
 
     * Both sides with barriers -> block fusion (a wave-granular LDS barrier on both sides of
       one workgroup would have each side spin on issue slots the other needs).
     * Otherwise horizontal fusion is possible if the summed threads fit a workgroup and the
       summed LDS fits a CU.
-    * The bfuse ratio interleaves in proportion to how many workgroups of each side fit a CU
-      next to each other (VGPR- and LDS-limited), capped by the grid ratio.
+    * Does block fusion pay?  Every workgroup of a block-fused kernel is charged the LARGER side's
+      static LDS and registers.  `needed` = workgroups per CU each side has resident when it runs
+      alone (its grid over the CUs, capped by its own occupancy); `cap_lds` / `cap_waves` = what a
+      CU holds of the fused kernel.  If both sides' needs fit a CU at once (`side_by_side`), the
+      sides run in each other's shadow: fusion pays.  If not, the workgroups of the side that does
+      not fit run in rounds, in whatever slots the other side leaves: with the sides' ExecTime
+      known, a round of that side lasts its standalone time over its standalone rounds, and the
+      fusion pays only if those rounds end within the other side's time and the side keeps at
+      least half of the workgroups per CU it has alone (`bfuse_pays`).  A memory-bound side cut into short workgroups
+      (LayerNorm rows, softmax rows) passes; a side whose workgroups live as long as its kernel
+      (a batched GEMM resident in one round) does not: its displaced workgroups start when the
+      partner ends and the pair takes as long as serial, or longer.  Without times, a side that
+      does not fit is taken for short-lived only if it has neither barriers nor LDS.
     """
     ta, tb = a.dims.block[0] * a.dims.block[1] * a.dims.block[2], b.dims.block[0] * b.dims.block[1] * b.dims.block[2]
     wa, wb = -(-ta // 64), -(-tb // 64)
     hfuse_ok = not (a.HasBarriers and b.HasBarriers) and (wa + wb) * 64 <= 1024 and lds_a + lds_b <= LDS_PER_CU
 
+    def waves_per_cu(regs):
+        return 4 * min(MAX_WAVES_PER_SIMD, VGPRS_PER_SIMD // (-(-max(regs, 1) // 8) * 8))   # registers come in blocks of 8
+
     def wg_per_cu(waves, regs, lds):
-        by_reg = (VGPRS_PER_SIMD // max(regs, 1)) * 4 // max(waves, 1)
-        by_wave = MAX_WAVES_PER_SIMD * 4 // max(waves, 1)
+        by_reg = waves_per_cu(regs) // max(waves, 1)
         by_lds = LDS_PER_CU // lds if lds else 1 << 30
-        return max(1, min(by_reg, by_wave, by_lds))
+        return max(1, min(by_reg, by_lds))
 
     # the fused kernel allocates max(regs) for both sides
     regs = max(a.Reg, b.Reg)
-    na, nb = wg_per_cu(wa, regs, max(lds_a, lds_b)), wg_per_cu(wb, regs, max(lds_a, lds_b))
+    lds = max(lds_a, lds_b)
+    na, nb = wg_per_cu(wa, regs, lds), wg_per_cu(wb, regs, lds)
     ga, gb = a.dims.grid[0] * a.dims.grid[1] * a.dims.grid[2], b.dims.grid[0] * b.dims.grid[1] * b.dims.grid[2]
     rounds_a, rounds_b = -(-ga // (cus * na)), -(-gb // (cus * nb))
+
+    # ---- does block fusion pay? -----------------------------------------------------------------
+    alone = (wg_per_cu(wa, a.Reg, lds_a), wg_per_cu(wb, b.Reg, lds_b))          # occupancy of each side on its own
+    per_cu = (-(-ga // cus), -(-gb // cus))
+    needed = (min(alone[0], per_cu[0]), min(alone[1], per_cu[1]))
+    rounds_alone = (-(-per_cu[0] // alone[0]), -(-per_cu[1] // alone[1]))
+    cap_lds = LDS_PER_CU // lds if lds else 1 << 30
+    cap_waves = waves_per_cu(regs)
+    waves = (wa, wb)
+    side_by_side = needed[0] + needed[1] <= cap_lds and needed[0] * wa + needed[1] * wb <= cap_waves
+    times = (a.ExecTime, b.ExecTime)
+    known = times[0] > 0 and times[1] > 0
+    predicted = None
+    if side_by_side:
+        pays = True
+        if known:
+            predicted = max(times)
+    else:
+        # one side is dealt into the slots the other leaves; either may be that side: the better case counts
+        pays = False
+        for x in (0, 1):
+            o = 1 - x
+            slots = min(cap_lds - needed[o], (cap_waves - needed[o] * waves[o]) // waves[x])
+            if known:
+                life = times[x] / rounds_alone[x]                  # one round of side x's workgroups
+                if slots >= 1:
+                    p_x = max(times[o], -(-per_cu[x] // slots) * life)
+                else:                                              # nothing of x fits beside o: x runs after it
+                    p_x = times[o] + -(-per_cu[x] // max(1, min(cap_lds, cap_waves // waves[x]))) * life
+                # the displaced rounds must end in the partner's shadow; if they outlast it, what is left of side
+                # x runs alone at a fraction of its occupancy and the pair comes out no better than serial
+                # -- and it must keep at least half of the concurrency it has alone (a side squeezed into a third
+                # of its workgroups per CU, one wave at a time beside a barrier-synchronised GEMM, measured slower
+                # than serial although its rounds were short)
+                pays = pays or (2 * slots >= needed[x] and -(-per_cu[x] // slots) * life <= times[o])
+                predicted = p_x if predicted is None else min(predicted, p_x)
+            else:
+                kx = (a, b)[x]
+                pays = pays or (slots >= 1 and 2 * slots >= needed[x] and not kx.HasBarriers and (lds_a, lds_b)[x] == 0)
+    fuse = "hfuse" if hfuse_ok and ga == gb else ("bfuse" if pays else ("hfuse" if hfuse_ok and max(ga, gb) <= cus else "none"))
     return {"hfuse_ok": hfuse_ok, "prefer": "hfuse" if hfuse_ok and ga == gb else "bfuse",
             "wg_per_cu": (na, nb), "rounds": (rounds_a, rounds_b),
             # one chunk per round over the CUs (measured best on MI355X: the compute-bound side lands
@@ -155,4 +209,7 @@ def choose_fusion(a: KernelInfo, b: KernelInfo, lds_a: int, lds_b: int, cus: int
             # is then a single contiguous range, which the hardware itself deals round-robin over
             # the eight XCDs.
             "chunk": cus,
-            "ratio_M": max(1, max(ga, gb) // max(1, min(ga, gb)))}
+            "ratio_M": max(1, max(ga, gb) // max(1, min(ga, gb))),
+            "needed": needed, "cap_lds": min(cap_lds, 1 << 20), "cap_waves": cap_waves, "side_by_side": side_by_side,
+            "predicted_us": predicted, "serial_us": (times[0] + times[1]) if known else None,
+            "bfuse_pays": pays, "fuse": fuse}

@@ -214,9 +214,15 @@ def _synthetic(handle, seed):
     return out
 
 
+def read_own(path: str, name: str) -> List[float]:
+    """Durations (ns) of `name` in a trace, warm-ups dropped."""
+    return [r["Duration"] for r in read_trace(path) if r["Name"] == name][WARMUP_TRIALS:]
+
+
 def run_suite(info: dict, out_dir: str, validate: bool = True, triangular: bool = False, log=print) -> List[dict]:
     """Runs the matrix over resident buffers with the library's dispatch timestamps, writes one
     trace per (method, i, j) under `<out_dir>/exec/` and returns the analysed rows."""
+    from . import tuner
     from .operation import Operation
     a, b = set_names(info)
     exec_dir = os.path.join(out_dir, "exec")
@@ -254,6 +260,22 @@ def run_suite(info: dict, out_dir: str, validate: bool = True, triangular: bool 
             write_trace(os.path.join(exec_dir, f"1_0_{j}.csv"), trace_of(t[0], t[1], t[2], [k2]))
             t = op.time("parallel", warmup=0, reps=WARMUP_TRIALS + n_rep)
             write_trace(os.path.join(exec_dir, f"2_{i}_{j}.csv"), trace_of(t[0], t[1], t[2], [k1, k2]))
+            # The chooser decides BEFORE any fused kernel of the pair has run, from the two kernels' footprints
+            # (registers, LDS, barriers, launch shapes: the code objects' metadata) and their standalone
+            # times just measured (KernelInfo.ExecTime): thread-level fusion, block fusion, or leave the
+            # pair unfused.  The fused variants are all timed below for the table; `chooser` names the one
+            # form this suite would run.
+            t1 = float(np.mean(read_own(os.path.join(exec_dir, f"0_{i}_0.csv"), k1)))
+            t2 = float(np.mean(read_own(os.path.join(exec_dir, f"1_0_{j}.csv"), k2)))
+            choice = tuner.static_plan(op.k[0], op.k[1], kinds=("hfuse", "bfuse", "none"), times=(t1 / 1e3, t2 / 1e3))
+            picked = tuner.find_variant(op.k[0], op.k[1], choice)
+            st = choice["static"]
+            with open(os.path.join(exec_dir, f"choice_{i}_{j}.json"), "w") as f:
+                json.dump({"kind": choice["kind"] if picked is not None or choice["kind"] == "none" else "none",
+                           "kernel": picked.name if picked is not None else None,
+                           "not_built": picked is None and choice["kind"] != "none",
+                           "side_by_side": bool(st["side_by_side"]), "needed": list(st["needed"]),
+                           "cap_lds": st["cap_lds"], "cap_waves": st["cap_waves"], "predicted_us": st["predicted_us"]}, f)
             for kind, idx in (("hfuse", 3), ("bfuse", 4)):
                 best = None
                 for h in fused_variants(k1, k2)[kind]:
@@ -263,6 +285,8 @@ def run_suite(info: dict, out_dir: str, validate: bool = True, triangular: bool 
                         if not (np.array_equal(Q1.view(np.uint8), base[0].view(np.uint8)) and np.array_equal(Q2.view(np.uint8), base[1].view(np.uint8))):
                             raise RuntimeError(f"{h.name}: output differs from the unfused kernels")
                     t = op.time(kind, h, warmup=0, reps=WARMUP_TRIALS + n_rep)
+                    if picked is not None and h.name == picked.name:
+                        write_trace(os.path.join(exec_dir, f"chosen_{i}_{j}.csv"), trace_of(t[0], t[1], t[2], [h.name]))
                     m = float(np.mean(t[0][WARMUP_TRIALS:]))
                     if best is None or m < best[0]:
                         best = (m, h, t)
@@ -314,6 +338,24 @@ def analyze(info: dict, exec_dir: str, triangular: bool = False) -> List[dict]:
             row[f"{kind}_kernel"] = name
             row[f"{kind}_ns"] = single_statistics(tr, name)[2]
             row[f"{kind}_speedup"] = row["serial_ns"] / row[f"{kind}_ns"]
+        # what the chooser decided for the pair (written by run_suite before the fused kernels ran) and the
+        # time of that one form: the chosen fused kernel's, or the serial time when the pair is left unfused
+        cf = os.path.join(exec_dir, f"choice_{i}_{j}.json")
+        if os.path.exists(cf):
+            with open(cf) as f:
+                ch = json.load(f)
+            row["chooser"] = ch
+            row["chooser_ns"] = row["serial_ns"]
+            if ch["kind"] != "none" and ch["kernel"]:
+                pf = _find(exec_dir, f"{3 if ch['kind'] == 'hfuse' else 4}_{i}_{j}")
+                # the trace of a kind holds the fastest variant; the chooser's kernel is timed in its own file
+                own = _find(exec_dir, f"chosen_{i}_{j}")
+                src = own or pf
+                if src:
+                    d = [r["Duration"] for r in read_trace(src) if r["Name"] == ch["kernel"]][WARMUP_TRIALS:]
+                    if d:
+                        row["chooser_ns"] = float(np.mean(d))
+            row["chooser_speedup"] = row["serial_ns"] / row["chooser_ns"]
         rows.append(row)
     return rows
 
@@ -324,19 +366,34 @@ def geomean(values: Sequence[float]) -> float:
 
 
 def to_markdown(rows: Sequence[dict]) -> str:
-    head = "| kernel1 | kernel2 | k1 us | k2 us | serial us | parallel | hfuse | bfuse | bfuse kernel |\n|---|---|---|---|---|---|---|---|---|\n"
+    head = "| kernel1 | kernel2 | k1 us | k2 us | serial us | parallel | hfuse | bfuse | chooser | bfuse kernel |\n|---|---|---|---|---|---|---|---|---|---|\n"
     body = ""
+    def chooser(r):
+        if "chooser" not in r:
+            return "-"
+        c = r["chooser"]
+        what = "unfused" if c["kind"] == "none" else c["kind"]
+        if c.get("not_built"):
+            what += " (chosen form not built)"
+        return f"{what}: {r['chooser_ns'] / 1e3:.2f} ({r['chooser_speedup']:.2f}x)"
+
     for r in rows:
         def f(k):
             return f"{r[k + '_ns'] / 1e3:.2f} ({r[k + '_speedup']:.2f}x)" if k + "_ns" in r else "-"
         body += (f"| {r['kernel1']} | {r['kernel2']} | {r['kernel1_ns'] / 1e3:.2f} | {r['kernel2_ns'] / 1e3:.2f} | {r['serial_ns'] / 1e3:.2f} | "
-                 f"{f('parallel')} | {f('hfuse')} | {f('bfuse')} | {r.get('bfuse_kernel', '-')} |\n")
+                 f"{f('parallel')} | {f('hfuse')} | {f('bfuse')} | {chooser(r)} | {r.get('bfuse_kernel', '-')} |\n")
     kinds = [k for k in ("parallel", "hfuse", "bfuse") if any(k + "_speedup" in r for r in rows)]
     tail = "\ngeomean speed-up over serial: " + ", ".join(
         f"{k} {geomean([r.get(k + '_speedup') for r in rows]):.3f}x" for k in kinds)
     # what the table is for: each pair run in the fastest of its measured forms (serial counts as 1)
     best = [max([1.0] + [r[k + "_speedup"] for k in ("hfuse", "bfuse") if k + "_speedup" in r]) for r in rows]
-    tail += f"; fusing only the pairs it pays for: {geomean(best):.3f}x ({sum(1 for x in best if x > 1.0)} of {len(rows)} pairs fused)"
+    tail += f"; best form per pair, picked after the fact: {geomean(best):.3f}x ({sum(1 for x in best if x > 1.0)} of {len(rows)} pairs fused)"
+    ch = [r for r in rows if "chooser" in r]
+    if ch:
+        fusedn = sum(1 for r in ch if r["chooser"]["kind"] != "none")
+        tail += (f"\nthe chooser's form per pair (decided from the footprints and the two standalone times, before any fused kernel of the pair "
+                 f"ran): {geomean([r['chooser_speedup'] for r in ch]):.3f}x ({fusedn} of {len(ch)} pairs fused, {len(ch) - fusedn} left unfused; "
+                 f"worst {min(r['chooser_speedup'] for r in ch):.2f}x)")
     return head + body + tail + "\n"
 
 

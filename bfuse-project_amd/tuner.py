@@ -58,10 +58,13 @@ def default_candidates(g1: int, g2: int, cus: int = 256) -> List[Candidate]:
     return out
 
 
-def static_choice(a: KernelHandle, b: KernelHandle, cus: int = 256) -> dict:
-    """What the code-object metadata alone says (no launch)."""
-    ka = config.KernelInfo(a.name, a.has_barriers, a.grid, a.block, max(a.regs, 1))
-    kb = config.KernelInfo(b.name, b.has_barriers, b.grid, b.block, max(b.regs, 1))
+def static_choice(a: KernelHandle, b: KernelHandle, cus: int = 256, times: Optional[Sequence[float]] = None) -> dict:
+    """What the code-object metadata alone says (no launch).  `times`: the two kernels' standalone
+    durations in microseconds where they are known (KernelInfo.ExecTime, a field the reference
+    parses and never uses): with them the rule also predicts whether block fusion pays."""
+    ta, tb = (times if times is not None else (-1.0, -1.0))
+    ka = config.KernelInfo(a.name, a.has_barriers, a.grid, a.block, max(a.regs, 1), float(ta))
+    kb = config.KernelInfo(b.name, b.has_barriers, b.grid, b.block, max(b.regs, 1), float(tb))
     return config.choose_fusion(ka, kb, max(a.lds_bytes, 0), max(b.lds_bytes, 0), cus)
 
 
@@ -108,11 +111,19 @@ def same_dispatch(plan_a, plan_b) -> bool:
     return bool(np.array_equal(ka, kb) and np.array_equal(va, vb))
 
 
-def static_plan(a: KernelHandle, b: KernelHandle, cus: int = 256, kinds: Sequence[str] = ("hfuse", "bfuse")) -> dict:
+def static_plan(a: KernelHandle, b: KernelHandle, cus: int = 256, kinds: Sequence[str] = ("hfuse", "bfuse"),
+                times: Optional[Sequence[float]] = None) -> dict:
     """The fusion the metadata alone selects, among the allowed kinds: thread-level fusion when the
     footprints allow it and the grids match, else block fusion in chunks of `chunk` workgroups
-    (one chunk per round over the CUs).  Returns {"kind", "pattern", "p0", "p1", "static"}."""
-    st = static_choice(a, b, cus)
+    (one chunk per round over the CUs).  With "none" among the kinds the answer may be to leave the
+    pair unfused: when the footprint rule predicts that block fusion does not pay
+    (config.choose_fusion) and thread-level fusion is not possible either.
+    Returns {"kind", "pattern", "p0", "p1", "static"}."""
+    st = static_choice(a, b, cus, times)
+    if "none" in kinds and (st["fuse"] == "none" or st["fuse"] not in kinds):
+        return {"kind": "none", "pattern": None, "p0": 0, "p1": 0, "static": st}
+    if "none" in kinds and st["fuse"] == "hfuse":
+        return {"kind": "hfuse", "pattern": None, "p0": 0, "p1": 0, "static": st}
     if "hfuse" in kinds and (st["prefer"] == "hfuse" or "bfuse" not in kinds):
         if not st["hfuse_ok"]:
             raise ValueError(f"{a.name} + {b.name}: thread-level fusion is not possible (barriers on both sides, threads or LDS)")
@@ -123,6 +134,8 @@ def static_plan(a: KernelHandle, b: KernelHandle, cus: int = 256, kinds: Sequenc
 def find_variant(k1: KernelHandle, k2: KernelHandle, choice: dict) -> Optional[KernelHandle]:
     """The built compile-time kernel of (k1, k2) that realises `choice` (static_plan's or a row of
     autotune): for block fusion, the one whose dispatch table equals the chosen plan's."""
+    if choice["kind"] == "none":
+        return None
     built = built_variants(k1.name, k2.name)
     if choice["kind"] == "hfuse":
         hs = [k for k in built if k.kind == 2]

@@ -60,3 +60,69 @@ def test_footprint_rules():
     assert c["wg_per_cu"] == (5, 5) and c["chunk"] == 256
     c = config.choose_fusion(ki("a", True, 256, 768, 168), ki("b", False, 512, 64, 48), 135 * 1024, 0)
     assert c["wg_per_cu"][0] == 1 and c["wg_per_cu"][1] == 1      # 135 KB: nothing shares the CU with it
+
+
+def test_the_footprint_rule_on_the_48_pairs_of_the_model_operator_matrix(golden_dir):
+    """Footprints of the library's own kernels (registers and LDS from the build's resource remarks, launch
+    shapes from the registry) and one measured run of the 48-pair matrix (standalone times, speed-up of the
+    block-fused kernel over serial; tests/golden/model_matrix_footprints.json).  The rule sees footprints and
+    standalone times only.  It must leave unfused every pair whose block-fused kernel measured slower than
+    serial, fuse at least half of the pairs that gained 5 % or more, and its choices must come out ahead."""
+    import json
+    import math
+    import os
+    with open(os.path.join(golden_dir, "model_matrix_footprints.json")) as f:
+        data = json.load(f)
+
+    def ki(name):
+        k = data["kernels"][name]
+        return config.KernelInfo(name, k["barriers"], (k["grid"], 1, 1), (k["threads"], 1, 1), k["regs"], k["us"]), k["lds"]
+
+    assert len(data["pairs"]) == 48
+    log_gain, fused, missed = 0.0, 0, 0
+    for p in data["pairs"]:
+        (a, la), (b, lb) = ki(p["kernel1"]), ki(p["kernel2"])
+        c = config.choose_fusion(a, b, la, lb)
+        assert c["fuse"] in ("bfuse", "none")            # no pair of the matrix has matching grids
+        if p["bfuse_speedup"] < 0.98:
+            assert c["fuse"] == "none", (p, c)
+        if c["fuse"] == "bfuse":
+            assert p["bfuse_speedup"] >= 0.98, (p, c)
+            log_gain += math.log(p["bfuse_speedup"])
+            fused += 1
+        elif p["bfuse_speedup"] >= 1.05:
+            missed += 1
+        assert c["fuse"] == p["chooser"]                 # what the suite's run decided on the GPU box
+    winners = sum(1 for p in data["pairs"] if p["bfuse_speedup"] >= 1.05)
+    assert fused >= 20 and missed <= winners // 2
+    assert math.exp(log_gain / 48) >= 1.04
+
+
+def test_the_footprint_rule_on_the_headline_pairs_with_and_without_times():
+    """Pairs 2 and 4: the memory-bound side does not fit a CU next to the GEMM in one round, but its workgroups
+    are short (a row each) and end in the GEMM's shadow: block fusion pays.  A batched GEMM whose workgroups
+    live as long as the kernel does not.  Without times, only a side with neither barriers nor LDS is taken
+    for short-lived."""
+    ki = config.KernelInfo
+    gemm2 = ki("gemm_f32_512x768x2304", True, (256, 1, 1), (256, 1, 1), 156, 15.6)
+    ln = ki("layernorm_512x768", False, (512, 1, 1), (64, 1, 1), 46, 4.1)
+    c = config.choose_fusion(gemm2, ln, 73728, 0)
+    assert not c["side_by_side"] and c["bfuse_pays"] and c["fuse"] == "bfuse" and c["predicted_us"] == 15.6
+    softmax = ki("softmax_causal_12x512x512", False, (1536, 1, 1), (256, 1, 1), 15, 5.2)
+    gemm4 = ki("gemm_gelu_f32_512x768x3072", True, (512, 1, 1), (256, 1, 1), 90, 20.8)
+    c = config.choose_fusion(softmax, gemm4, 0, 32768)
+    assert not c["side_by_side"] and c["fuse"] == "bfuse"
+    long_b = ki("bgemm_f32_32x512x512x128", True, (1024, 1, 1), (128, 1, 1), 100, 27.2)
+    c = config.choose_fusion(ki("gemm_f32_512x768x768", True, (256, 1, 1), (256, 1, 1), 53, 7.0), long_b, 36864, 16384)
+    assert c["fuse"] == "none" and c["predicted_us"] >= c["serial_us"]
+    # no times: the LayerNorm (no barriers, no LDS) is taken for short-lived, the batched GEMM is not
+    untimed = lambda k: ki(k.KernelName, k.HasBarriers, k.GridDim, k.BlockDim, k.Reg)
+    assert config.choose_fusion(untimed(gemm2), untimed(ln), 73728, 0)["fuse"] == "bfuse"
+    assert config.choose_fusion(ki("g", True, (256, 1, 1), (256, 1, 1), 53), untimed(long_b), 36864, 16384)["fuse"] == "none"
+    # the bf16 gate projection's 135 KB leave room for nothing beside it: block fusion never pays, thread-level
+    # fusion does when the grids match (pair 5)
+    gate = ki("gemm_bf16_512x4096x14336", True, (256, 1, 1), (640, 1, 1), 116, 46.0)
+    norm = ki("rmsnorm_rope_bf16_512x4096_w2", False, (256, 1, 1), (128, 1, 1), 60, 4.5)
+    c = config.choose_fusion(gate, norm, 135168, 0)
+    assert c["fuse"] == "hfuse" and not c["bfuse_pays"]
+    assert tuner.static_plan.__defaults__[1] == ("hfuse", "bfuse")      # "none" is an answer only where it is asked for

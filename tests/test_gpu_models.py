@@ -162,3 +162,14 @@ def test_pair_matrix_of_the_model_operators(tmp_path):
           f"best {max(x['bfuse_speedup'] for x in rows):.2f}x, worst {min(x['bfuse_speedup'] for x in rows):.2f}x", flush=True)
     assert g > 0
     expect(0.8 < g < 2.0, f"geomean speed-up of block fusion over the 48 pairs {g:.3f}x")
+    # thread-level fusion where the grids allow it: the four one-tile-per-CU dense layers with the two convolutions
+    assert sum(1 for x in rows if "hfuse_ns" in x) == 8
+    # the chooser decided every pair before its fused kernels ran: a fused form it picked is one the library holds,
+    # and a pair left unfused counts at its serial time
+    assert all("chooser" in x and x["chooser"]["kind"] in ("bfuse", "hfuse", "none") and not x["chooser"]["not_built"] for x in rows)
+    fused = [x for x in rows if x["chooser"]["kind"] != "none"]
+    assert all(x["chooser_ns"] == x["serial_ns"] for x in rows if x["chooser"]["kind"] == "none") and len(fused) >= 12
+    gc = suite.geomean([x["chooser_speedup"] for x in rows])
+    worst = min(x["chooser_speedup"] for x in rows)
+    print(f"[models] the chooser's forms: geomean {gc:.3f}x, {len(fused)} of 48 pairs fused, worst {worst:.2f}x", flush=True)
+    expect(worst >= 0.98 and gc >= 1.04, f"chooser over the 48 pairs: geomean {gc:.3f}x, worst pair {worst:.2f}x")
