@@ -49,3 +49,11 @@ BFUSE_KERNEL(gemm_bf16_512x256x14336, GemmGateK256, ({{512, 256, 1, 1}, 2}), ({{
 // a weight held as [K, N] = [4096, 14336] is brought into the GEMM's [N, K] layout once, when it is loaded
 using WeightToNK = Transpose16<4096, 14336>;
 BFUSE_KERNEL(transpose16_4096x14336, WeightToNK, ({{4096, 14336, 1, 1}, 2}), ({{1, 1, 1, 1}, 2}), ({{14336, 4096, 1, 1}, 2}))
+
+// The headline GEMM with clock stamps (instrumentation; `python -m bfuse_project_amd.profile_pair --clock` reads them):
+// the same code with three pairs of counter reads per workgroup, its output 256 x 8 64-bit words longer.  Alone and
+// with the norm waves fused in.  Not an alternative of the product kernel: its output shape differs.
+using GemmGateClk = GemmBf16NTDma<512, 14336, 4096, 128, 224, 3, 4, 4, 2, 2, 11, true>;
+BFUSE_KERNEL(gemm_bf16_512x4096x14336_clk, GemmGateClk, ({{512, 4096, 1, 1}, 2}), ({{14336, 4096, 1, 1}, 2}),
+             ({{512 * 14336 + 256 * GemmGateClk::STAMP_WORDS * 4, 1, 1, 1}, 2}))
+BFUSE_HFUSE_KERNEL(gemm_bf16_512x4096x14336_clk, GemmGateClk, rmsnorm_rope_bf16_512x4096_w2, NormRope2)

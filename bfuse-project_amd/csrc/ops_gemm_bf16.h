@@ -54,8 +54,17 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 // consecutive steps live in two register sets, so the rolled loop holds 2 * NSTG_ steps.  Measured
 // on MI355X on the 512 x 4096 x 14336 instance, both forms in one run: 46.8 against 48.2 us, and
 // 47.8 against 49.4-49.8 us with the norm waves fused in.
-template <int M_, int N_, int K_, int BM_, int BN_, int NSTG_ = 3, int PD_ = 4, int WGM_ = 2, int WGN_ = 2, int PW_ = 0, int EARLY_ = 0>
+// CLK_ (instrumentation, off in every product kernel): wave 0 of each workgroup reads the shader-clock
+// counter and the 100 MHz wall clock before its K loop, after it, and when its last store has been
+// acknowledged, and writes them with the XCD it ran on behind the output matrix (STAMP_WORDS 64-bit words per
+// workgroup at byte offset M * N * 2 of O; the kernel is then registered with an output that much larger).
+// The counters are scalar memory reads; each is waited for at once, so none is in flight when the
+// hand-counted LDS waits of the loop run.
+template <int M_, int N_, int K_, int BM_, int BN_, int NSTG_ = 3, int PD_ = 4, int WGM_ = 2, int WGN_ = 2, int PW_ = 0, int EARLY_ = 0,
+          bool CLK_ = false>
 struct GemmBf16NTDma {
+    static constexpr bool CLK = CLK_;
+    static constexpr int STAMP_WORDS = 8;   // clock x 3, wall x 3, XCC_ID, HW_ID
     static constexpr int M = M_, N = N_, K = K_, BM = BM_, BN = BN_, NSTG = NSTG_;
     static constexpr int BK = 64;
     static constexpr int WGM = WGM_, WGN = WGN_, NCOMP = WGM_ * WGN_, PW = PW_;
@@ -415,6 +424,9 @@ struct GemmBf16NTDma {
             }
         }
 
+        unsigned long long stamp_c[3] = {0, 0, 0}, stamp_w[3] = {0, 0, 0};
+        if constexpr (CLK_) read_clocks(stamp_c[0], stamp_w[0]);
+
         // K-steps are taken NSTG at a time so that the LDS stage of each is a compile-time constant;
         // the loop stays rolled whatever K is: operand registers with reads in flight must never be
         // spilled (the compiler takes an asm output for written when the asm is issued), and a
@@ -440,6 +452,7 @@ struct GemmBf16NTDma {
                 if constexpr (NSTG > 3) k_step<3, PW == 0>(kt0 + 3, acc, ad, src, lds, full, sync);
             }
         }
+        if constexpr (CLK_) read_clocks(stamp_c[1], stamp_w[1]);
         sync();  // all waves are done reading the last stage before the tile buffer overwrites it
 
         unsigned short* ct = reinterpret_cast<unsigned short*>(sm.t);
@@ -467,6 +480,30 @@ struct GemmBf16NTDma {
                     *reinterpret_cast<const u32x4*>(ct + row * CPITCH + col);
             }
         }
+        if constexpr (CLK_) {
+            wait_vm<0>();   // this wave's stores have been acknowledged
+            read_clocks(stamp_c[2], stamp_w[2]);
+            if (tid == 0) {
+                unsigned long long* st = reinterpret_cast<unsigned long long*>(C + (size_t)M * N) + (size_t)vblock * STAMP_WORDS;
+#pragma unroll
+                for (int i = 0; i < 3; ++i) {
+                    st[i] = stamp_c[i];
+                    st[3 + i] = stamp_w[i];
+                }
+                st[6] = __builtin_amdgcn_s_getreg((3 << 11) | 20);    // HW_REG_XCC_ID, bits 3:0
+                st[7] = __builtin_amdgcn_s_getreg((31 << 11) | 4);    // HW_REG_HW_ID
+            }
+        }
+    }
+
+    // shader-clock counter and 100 MHz wall clock, both landed before anything else is issued
+    __device__ static __forceinline__ void read_clocks(unsigned long long& c, unsigned long long& w)
+    {
+#if defined(__HIP_DEVICE_COMPILE__)
+        c = clock64();
+        w = wall_clock64();
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(c), "+s"(w));
+#endif
     }
 };
 

@@ -125,3 +125,30 @@ def test_shutdown_releases_everything_and_the_library_can_be_initialized_again()
         op2.launch("kernel1")
         y = op2.download(0)
     assert np.array_equal(y.ravel(), np.maximum(x + b, 0.0))
+
+
+def test_clock_stamped_gemm_computes_what_the_product_kernel_computes():
+    """The instrumented instance of pair 5's GEMM (clock stamps behind its output matrix) is the product kernel
+    plus counter reads: the matrix must be byte-identical, alone and with the norm waves fused in, and the stamps
+    ordered (loop start < loop end < last store acknowledged) on eight XCDs; the table of
+    `python -m bfuse_project_amd.profile_pair --clock` comes out of them."""
+    import numpy as np
+    import bfuse_project_amd as bf
+    from bfuse_project_amd.profile_pair import clock_table
+    from bfuse_project_amd.workloads import PAIRS
+    print("clock-stamped GEMM", flush=True)
+    I1, F1, I2, F2 = PAIRS[5].inputs()
+    with bf.Operation("gemm_bf16_512x4096x14336", "rmsnorm_rope_bf16_512x4096_w2") as op:
+        want = op.run_kernel(0, I1, F1)
+        want2 = op.run_kernel(1, I2, F2)
+    with bf.Operation("gemm_bf16_512x4096x14336_clk", "rmsnorm_rope_bf16_512x4096_w2") as op:
+        got = op.run_kernel(0, I1, F1)
+        q1, q2 = op.run_fuse(op.fused("hfuse"), I1, F1, I2, F2)
+    n = 512 * 14336
+    assert np.array_equal(got.ravel()[:n], want.ravel()) and np.array_equal(q1.ravel()[:n], want.ravel()) and np.array_equal(q2, want2)
+    st = got.ravel().view(np.uint8)[n * 2:].view(np.uint64).reshape(256, 8).astype(np.int64)
+    assert np.all(st[:, 0] < st[:, 1]) and np.all(st[:, 1] < st[:, 2]) and np.all(st[:, 3] <= st[:, 4]) and np.all(st[:, 4] <= st[:, 5])
+    assert sorted(set((st[:, 6] & 15).tolist())) == list(range(8))
+    table = clock_table(20)
+    print(table, flush=True)
+    assert "shader clocks per K-stage" in table and table.count("| 7 |") == 2
