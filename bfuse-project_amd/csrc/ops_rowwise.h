@@ -152,7 +152,17 @@ struct SoftmaxCausal {
     using Smem = NoSmem;
 
     // rows row0 + b*stride, b = 0..RB-1; every row is reduced on its own, in the same order
-    // whatever RB is
+    // whatever RB is.
+    //
+    // The query position i of a row is the same for every lane of the wave, so what the causal mask does
+    // to each 256-column block (one f32x4 per lane) is decided by scalar branches: a block left of the
+    // diagonal is visible whole (no per-element test), the block on the diagonal is masked per element,
+    // a block right of it is hidden whole -- it is neither loaded nor run through max / exp / sum, its
+    // probabilities are written as zeros.  Under fusion every vector instruction of this side takes an
+    // issue slot on a SIMD whose matrix core the partner's GEMM keeps busy (measured on pair 4: the
+    // softmax's arithmetic costs the fused kernel 0.8 us, its loads and stores 0.6), so the row's
+    // instruction count is what is minimised: exp(x - m) is one fused multiply-add and one v_exp_f32
+    // per element, the row's reciprocal one v_rcp_f32.
     __device__ static __forceinline__ void rows(int row0, int stride, int lane, const void* I, void* O)
     {
         const float ninf = -__builtin_inff();
@@ -164,38 +174,47 @@ struct SoftmaxCausal {
             const f32x4* __restrict__ x = static_cast<const f32x4*>(I) + (size_t)row * (S / 4);
 #pragma unroll
             for (int c = 0; c < VEC; ++c) {
-                const int col = (c * 64 + lane) * 4;
-                v[b][c] = f32x4{ninf, ninf, ninf, ninf};
-                if (col <= i) {
-                    const f32x4 t = x[c * 64 + lane];
+                if (256 * c + 255 <= i) {                 // visible whole (scalar branch)
+                    v[b][c] = x[c * 64 + lane];
+                } else if (256 * c <= i) {                // on the diagonal
+                    const int col = (c * 64 + lane) * 4;
+                    v[b][c] = f32x4{ninf, ninf, ninf, ninf};
+                    if (col <= i) {
+                        const f32x4 t = x[c * 64 + lane];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) v[b][c][e] = (col + e <= i) ? t[e] : ninf;
+                        for (int e = 0; e < 4; ++e) v[b][c][e] = (col + e <= i) ? t[e] : ninf;
+                    }
                 }
             }
         }
 #pragma unroll
         for (int b = 0; b < RB; ++b) {
             const int row = row0 + b * stride;
+            const int i = row % S;
             f32x4* __restrict__ y = static_cast<f32x4*>(O) + (size_t)row * (S / 4);
             float m = ninf;
 #pragma unroll
             for (int c = 0; c < VEC; ++c)
-                m = fmaxf(m, fmaxf(fmaxf(v[b][c][0], v[b][c][1]), fmaxf(v[b][c][2], v[b][c][3])));
+                if (256 * c <= i) m = fmaxf(fmaxf(m, fmaxf(v[b][c][0], v[b][c][1])), fmaxf(v[b][c][2], v[b][c][3]));
             m = wave_max(m);
+            const float mneg = -m * 1.4426950408889634f;
             float s = 0.f;
 #pragma unroll
             for (int c = 0; c < VEC; ++c) {
+                if (256 * c <= i) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e)   // exp(x - m) = 2^((x - m) log2 e): one v_exp_f32; masked columns give 2^-inf == 0
-                    v[b][c][e] = __builtin_amdgcn_exp2f((v[b][c][e] - m) * 1.4426950408889634f);
-                s += (v[b][c][0] + v[b][c][1]) + (v[b][c][2] + v[b][c][3]);
+                    for (int e = 0; e < 4; ++e)   // exp(x - m) = 2^(x log2 e - m log2 e): one fma, one v_exp_f32; masked columns give 2^-inf == 0
+                        v[b][c][e] = __builtin_amdgcn_exp2f(__builtin_fmaf(v[b][c][e], 1.4426950408889634f, mneg));
+                    s += (v[b][c][0] + v[b][c][1]) + (v[b][c][2] + v[b][c][3]);
+                }
             }
             s = wave_sum(s);
-            // one division per row, one multiplication per element: under fusion these instructions
-            // compete for issue slots with the other side's MFMAs (an IEEE division is ~10 of them)
-            const float rs = 1.0f / s;
+            const float rs = __builtin_amdgcn_rcpf(s);   // s >= 1 (the row's maximum contributes 2^0)
 #pragma unroll
-            for (int c = 0; c < VEC; ++c) y[c * 64 + lane] = v[b][c] * rs;
+            for (int c = 0; c < VEC; ++c) {
+                if (256 * c <= i) y[c * 64 + lane] = v[b][c] * rs;
+                else y[c * 64 + lane] = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
         }
     }
 
