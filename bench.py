@@ -220,7 +220,7 @@ def best_unfused(k1, k2, inputs, R, BW, b_ser, b_k1, b_k2):
 def measure(number, K, W, spec, ceilings, power_check=True):
     import bfuse_project_amd as bf
     from bfuse_project_amd import tuner
-    from bfuse_project_amd.workloads import PAIRS, MEASURED_TRAFFIC, TRAFFIC_SOURCE, CONFIG_KINDS, BESIDE, FLOORS
+    from bfuse_project_amd.workloads import PAIRS, measured_traffic, TRAFFIC_SOURCE, CONFIG_KINDS, BESIDE, FLOORS
 
     pair = PAIRS[number]
     k1, k2, kind, suffix, note = pick_fusion(number, spec)
@@ -370,7 +370,7 @@ def measure(number, K, W, spec, ceilings, power_check=True):
         "roofline": {"bound": pair.bound, "achieved": round(achieved, 2), "peak": pair.peak, "unit": unit,
                      "frac": round(achieved / pair.peak, 4),
                      "measured_peak": measured_peak, "frac_of_measured_peak": round(achieved / measured_peak, 4),
-                     "traffic": MEASURED_TRAFFIC.get(fused.name),
+                     "traffic": measured_traffic(fused.name),
                      "traffic_source": TRAFFIC_SOURCE.get(fused.name),
                      "kernel": fused.name, "avg_us": round(fused_us, 3),
                      "algorithmic": {"flops": pair.flops, "bytes": pair.bytes1 + pair.bytes2}},

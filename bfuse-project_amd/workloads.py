@@ -196,17 +196,10 @@ RT_SIDES = {
 
 # Bytes per launch that leave the eight L2s towards memory, for each headline fused kernel: measured
 # with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by what the same counters read for a 64 MiB
-# copy kernel (the derivation and commands are in the profile summaries shipped with the repository).
-# An operand that workgroups on all eight XCDs share is counted once per XCD.
-MEASURED_TRAFFIC = {
-    "gemm_f32_512x512x512_bias_relu_1048576_fused_hfuse": 20_020_000,
-    "gemm_f32_512x768x2304_layernorm_512x768_fused_bfuse_r": 27_740_000,
-    "conv3x3_f32_64x56x56_64_maxpool3x3s2_f32_64x112x112_fused_bfuse_c256": 7_670_000,
-    "softmax_causal_12x512x512_gemm_gelu_f32_512x768x3072_fused_bfuse_c256": 47_730_000,
-    "gemm_bf16_512x4096x14336_rmsnorm_rope_bf16_512x4096_w2_fused_hfuse": 175_670_000,
-}
-
-# the profile summary each figure above was taken from
+# copy kernel.  The figures live in the profile summaries shipped with the repository (derivation and
+# commands are there); `measured_traffic` reads the fused kernel's row out of its summary, so the
+# benchmark line cannot quote a figure the summary does not hold.  An operand that workgroups on all
+# eight XCDs share is counted once per XCD.
 TRAFFIC_SOURCE = {
     "gemm_f32_512x512x512_bias_relu_1048576_fused_hfuse": "profiles/pair1_gemm_f32_bias_relu_hfuse.md",
     "gemm_f32_512x768x2304_layernorm_512x768_fused_bfuse_r": "profiles/pair2_gemm_f32_layernorm_bfuse.md",
@@ -214,6 +207,39 @@ TRAFFIC_SOURCE = {
     "softmax_causal_12x512x512_gemm_gelu_f32_512x768x3072_fused_bfuse_c256": "profiles/pair4_softmax_gemm_gelu_bfuse.md",
     "gemm_bf16_512x4096x14336_rmsnorm_rope_bf16_512x4096_w2_fused_hfuse": "profiles/pair5_gemm_bf16_rmsnorm_rope_hfuse.md",
 }
+
+
+def measured_traffic(kernel: str, root: str = None):
+    """Bytes per launch of `kernel` from the traffic table of its profile summary (the row
+    "| `kernel` | FETCH raw | WRITE raw | read MB | write MB | total MB |"), or None if the kernel has no
+    summary.  Raises if the summary exists but holds no row for the kernel: the summary then describes another
+    build."""
+    import os
+    src = TRAFFIC_SOURCE.get(kernel)
+    if src is None:
+        return None
+    root = root or os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    with open(os.path.join(root, src)) as f:
+        for line in f:
+            cells = [c.strip() for c in line.split("|")]
+            if len(cells) >= 8 and cells[1] == f"`{kernel}`":
+                return int(round(float(cells[6]) * 1e6, -4))
+    raise LookupError(f"{src} has no traffic row for {kernel}")
+
+
+def check_traffic_sources(root: str = None) -> dict:
+    """Every headline fused kernel is registered, has a profile summary, and the summary has its row.
+    Part of the build check (__graft_entry__.build) and of the host tests."""
+    from .operation import kernel_info
+    out = {}
+    for n, (k1, k2, kind, suffix) in HEADLINE.items():
+        name = f"{k1}_{k2}_fused_{kind}{suffix}"
+        kernel_info(name)                         # raises for a kernel the library does not hold
+        if name not in TRAFFIC_SOURCE:
+            raise LookupError(f"pair {n}: no profile summary is named for {name}")
+        out[name] = measured_traffic(name, root)
+    return out
+
 
 def standalone_alternatives(name: str) -> List[str]:
     """Every standalone kernel of the registry that computes what `name` computes: the same operator at the

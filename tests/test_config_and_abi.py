@@ -168,3 +168,17 @@ def test_choose_fusion_uses_footprints():
     assert not both["hfuse_ok"]                                        # two barrier-bearing sides -> block fusion
     big = config.choose_fusion(bf.KernelInfo("g", True, (256, 1, 1), (256, 1, 1), 300), ln, 98304, 0)
     assert big["wg_per_cu"][0] == 1                                    # > 256 VGPRs: nothing fits next to it
+
+
+def test_traffic_figures_come_out_of_the_profile_summaries_of_the_registered_kernels():
+    """`roofline.traffic` of the benchmark line is read from the traffic table of the fused kernel's profile
+    summary: every headline kernel is registered, has a summary, and the summary has a row for it with a figure
+    between the pair's algorithmic bytes and three times that."""
+    from bfuse_project_amd.workloads import HEADLINE, PAIRS, check_traffic_sources, measured_traffic
+    got = check_traffic_sources()
+    assert len(got) == 5
+    for n, (k1, k2, kind, suffix) in HEADLINE.items():
+        t = got[f"{k1}_{k2}_fused_{kind}{suffix}"]
+        alg = PAIRS[n].bytes1 + PAIRS[n].bytes2
+        assert alg <= t <= 3 * alg, (n, t, alg)
+    assert measured_traffic("bias_relu_4096") is None
