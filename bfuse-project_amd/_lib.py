@@ -63,6 +63,7 @@ EXPORTS = [
     "bfuse_set_elem_bytes", "initialize_kernel1", "initialize_kernel2", "finalize_kernel1", "finalize_kernel2",
     "run_kernel1", "run_kernel2", "run_parallel", "run_fuse",
     "bfuse_upload", "bfuse_zero_output", "bfuse_download", "bfuse_synchronize", "bfuse_launch",
+    "bfuse_upload_part", "bfuse_download_part", "bfuse_checksum_output",
     "bfuse_time", "bfuse_time_batched", "bfuse_module_load", "bfuse_module_unload", "bfuse_module_launch",
     "bfuse_initialize_side", "bfuse_finalize_side", "bfuse_launch_list", "bfuse_time_list",
     "bfuse_fill_uniform", "bfuse_fill_normal", "bfuse_f32_to_bf16", "bfuse_bf16_to_f32", "bfuse_check_matrix",
@@ -112,6 +113,9 @@ def lib():
         l.run_fuse.argtypes = [vp] * 6 + [ip] * 6 + [vp, up, up, C.c_size_t, C.c_size_t]
         l.bfuse_upload.argtypes = [C.c_int, vp, vp]
         l.bfuse_download.argtypes = [C.c_int, vp]
+        l.bfuse_upload_part.argtypes = [C.c_int, C.c_int, C.c_size_t, vp, C.c_size_t]
+        l.bfuse_download_part.argtypes = [C.c_int, C.c_size_t, vp, C.c_size_t]
+        l.bfuse_checksum_output.argtypes = [C.c_int, C.c_size_t, vp]
         l.bfuse_launch.argtypes = [C.c_int, vp, up, up, vp, up, up]
         fp = C.POINTER(C.c_float)
         l.bfuse_time.argtypes = [C.c_int, vp, up, up, vp, up, up, C.c_int, C.c_int, fp, fp, fp]

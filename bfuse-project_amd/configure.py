@@ -78,10 +78,11 @@ def candidate_names(kernel_id: str, args, dtype: Optional[str]) -> List[str]:
         return [f"gemm_{t}_{b}x{i}x{o}" for t in types]
     if op == "conv2d":
         n, h, w, co, ci, kh, kw, stride, pad = args
-        if n != 1:
-            return []
         names = []
         for t in types:
+            if n != 1:                                               # a batch is part of the name
+                names.append(f"conv{kh}x{kw}s{stride}p{pad}_{t}_{n}x{ci}x{h}x{w}_{co}")
+                continue
             if (kh, kw, stride, pad) == (3, 3, 1, 1):
                 names.append(f"conv3x3_{t}_{ci}x{h}x{w}_{co}")       # the kernel tuned for this case, where instantiated
             names.append(f"conv{kh}x{kw}s{stride}p{pad}_{t}_{ci}x{h}x{w}_{co}")
@@ -136,10 +137,11 @@ def instantiation_hint(kernel_id: str, args) -> str:
                 f"({{{{{b}, {i}, 1, 1}}, 4}}), ({{{{{i}, {o}, 1, 1}}, 4}}), ({{{{{b}, {o}, 1, 1}}, 4}}))  in csrc/kernels_*.hip")
     if op == "conv2d":
         n, h, w, co, ci, kh, kw, stride, pad = args
-        if n != 1:
-            return "the library's convolutions are batch 1 (csrc/ops_conv_general.h)"
-        return (f"using Conv = ConvF32Lds<{ci}, {co}, {h}, {w}, {kh}, {kw}, {stride}, {pad}, BM, PB, KS>;  "
-                f"BFUSE_KERNEL(conv{kh}x{kw}s{stride}p{pad}_f32_{ci}x{h}x{w}_{co}, Conv, ...)  in csrc/kernels_*.hip")
+        if ci % 16 != 0 and ci > 4:
+            return "the library's convolutions take input channels in groups of 16, or at most 4 (csrc/ops_conv_general.h)"
+        batch = f"{n}x" if n != 1 else ""
+        return (f"using Conv = ConvF32Auto<{ci}, {co}, {h}, {w}, {kh}, {kw}, {stride}, {pad}, {n}>;  "
+                f"BFUSE_KERNEL(conv{kh}x{kw}s{stride}p{pad}_f32_{batch}{ci}x{h}x{w}_{co}, Conv, ...)  in csrc/kernels_*.hip")
     b, m, k, n = args
     return (f"using Bgemm = GemmF32<{m}, {n}, {k}, BM, BN, KS, kEpiNone, 2, 1, true, {b}>;  BFUSE_KERNEL(bgemm_f32_{b}x{m}x{k}x{n}, Bgemm, "
             f"({{{{{b}, {m}, {k}, 1}}, 4}}), ({{{{{b}, {n}, {k}, 1}}, 4}}), ({{{{{b}, {m}, {n}, 1}}, 4}}))  in csrc/kernels_*.hip")

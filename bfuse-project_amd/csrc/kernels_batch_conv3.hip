@@ -1,0 +1,26 @@
+// Batch-1024 convolutions of the reference's example configurations (test-utils/examples/benchmark.yaml,
+// inception_v3.yaml; argument lists N, H, W, CO, CI, KH, KW, stride, padding) on the general convolution with the
+// library's default tiling.  Names: conv<KH>x<KW>s<stride>p<padding>_f32_<N>x<CI>x<H>x<W>_<CO>.  Part 3 of 4.
+#include "fuse.h"
+#include "ops_conv_general.h"
+
+using namespace bfuse;
+
+BFUSE_MODULE_PROLOGUE()
+
+#define CONV_BATCH(N, CI, H, W, CO, KH, KW, S, P)                                                                 \
+    using Conv_##N##_##CI##_##H##_##W##_##CO##_##KH##_##KW##_##S##_##P = ConvF32Auto<CI, CO, H, W, KH, KW, S, P, N>; \
+    BFUSE_KERNEL(conv##KH##x##KW##s##S##p##P##_f32_##N##x##CI##x##H##x##W##_##CO,                                    \
+                 Conv_##N##_##CI##_##H##_##W##_##CO##_##KH##_##KW##_##S##_##P, ({{N, CI, H, W}, 4}), ({{CO, CI, KH, KW}, 4}), \
+                 ({{N, CO, (H - KH + 2 * P) / S + 1, (W - KW + 2 * P) / S + 1}, 4}))
+
+CONV_BATCH(1024, 64, 56, 56, 64, 1, 1, 1, 0)
+CONV_BATCH(1024, 128, 28, 28, 256, 3, 3, 2, 1)
+CONV_BATCH(1024, 512, 7, 7, 512, 3, 3, 1, 1)
+CONV_BATCH(1024, 288, 35, 35, 64, 1, 1, 1, 0)
+CONV_BATCH(1024, 768, 17, 17, 192, 1, 1, 1, 0)
+CONV_BATCH(1024, 3, 299, 299, 32, 3, 3, 2, 0)
+CONV_BATCH(1024, 80, 73, 73, 192, 3, 3, 1, 0)
+CONV_BATCH(1024, 64, 35, 35, 96, 3, 3, 1, 1)
+CONV_BATCH(1024, 1280, 8, 8, 384, 1, 1, 1, 0)
+CONV_BATCH(1024, 2048, 8, 8, 320, 1, 1, 1, 0)

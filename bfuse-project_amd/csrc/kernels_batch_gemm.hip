@@ -1,0 +1,39 @@
+// The dense and bgemm operators of the reference's test-utils/examples/benchmark.yaml: the layers of llm.yaml at
+// 1024 rows (dense: batch, in, out) and at 1024 independent products (bgemm: batch, M, K, N), fp32, with the
+// tilings of their 512-row / 16-product counterparts (model_ops.h) -- twice, or 64 times, the workgroups.
+#include "fuse.h"
+#include "ops_gemm_f32.h"
+#include "ops_gemm_f32_dma.h"
+
+using namespace bfuse;
+
+BFUSE_MODULE_PROLOGUE()
+
+#define DENSE_F32(M, K, N, ...)                                                                                  \
+    using Dense_##M##x##K##x##N = GemmF32Dma<M, N, K, __VA_ARGS__>;                                               \
+    BFUSE_KERNEL(gemm_f32_##M##x##K##x##N, Dense_##M##x##K##x##N, ({{M, K, 1, 1}, 4}), ({{K, N, 1, 1}, 4}), ({{M, N, 1, 1}, 4}))
+DENSE_F32(1024, 768, 768, 32, 48, 4)
+DENSE_F32(1024, 768, 3072, 32, 96, 4, kEpiNone, 2)
+DENSE_F32(1024, 3072, 768, 32, 48, 4)
+DENSE_F32(1024, 768, 2304, 32, 144, 4)
+DENSE_F32(1024, 4096, 4096, 64, 128, 4)
+DENSE_F32(1024, 4096, 1024, 32, 64, 4)
+DENSE_F32(1024, 4096, 14336, 64, 128, 4)
+DENSE_F32(1024, 14336, 4096, 64, 128, 4)
+
+// C[b] = A[b] . B[b]^T, A [b, M, K], B [b, N, K]: <M, N, K, BM, BN, waves over K>
+#define BGEMM_F32(B, M, K, N, BM, BN, KS)                                                                        \
+    using Bgemm_##B##x##M##x##K##x##N = GemmF32<M, N, K, BM, BN, KS, kEpiNone, 2, 1, true, B>;                    \
+    BFUSE_KERNEL(bgemm_f32_##B##x##M##x##K##x##N, Bgemm_##B##x##M##x##K##x##N, ({{B, M, K, 1}, 4}), ({{B, N, K, 1}, 4}), ({{B, M, N, 1}, 4}))
+BGEMM_F32(1024, 512, 64, 512, 64, 64, 1)
+BGEMM_F32(1024, 512, 512, 64, 32, 64, 2)
+BGEMM_F32(1024, 512, 128, 512, 64, 64, 1)
+BGEMM_F32(1024, 512, 512, 128, 32, 64, 2)
+BGEMM_F32(1024, 256, 64, 256, 64, 64, 1)
+BGEMM_F32(1024, 256, 256, 64, 16, 64, 2)
+BGEMM_F32(1024, 256, 80, 256, 64, 64, 1)
+BGEMM_F32(1024, 256, 256, 80, 16, 80, 2)
+BGEMM_F32(1024, 208, 64, 208, 16, 208, 1)
+BGEMM_F32(1024, 208, 208, 64, 16, 64, 1)
+BGEMM_F32(1024, 208, 80, 208, 16, 208, 1)
+BGEMM_F32(1024, 208, 208, 80, 16, 80, 1)

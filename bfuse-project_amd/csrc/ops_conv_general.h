@@ -1,4 +1,4 @@
-// Convolution of any filter size, stride and padding (NCHW data, OIHW weights, batch 1, dilation 1)
+// Convolution of any filter size, stride, padding and batch (NCHW data, OIHW weights, dilation 1)
 // as an implicit GEMM on the matrix cores with the image patch staged in LDS: the general form of
 // Conv3x3F32Lds (ops_conv.h), which stays the tuned kernel for 3x3 / stride 1 / padding 1 on images
 // whose rows are whole 16-byte chunks.
@@ -22,9 +22,12 @@
 // [channel quad][row][column][4 channels].  The B operand of tap (kh, kw) for output pixel (oy, ox)
 // then sits at position ((oy-oy_lo)*S + kh)*WP + ox*S + kw: a per-lane base plus a compile-time
 // offset per tap, for any stride; padding and rows outside the image read as zero, as a border test
-// would give.  Image rows that are not whole 16-byte chunks (W = 14, 7) are staged with 8- or 4-byte
-// loads.  A last pixel block that runs past the image (14x14 and 7x7 outputs are not multiples of 16
+// would give.  Image rows that are not whole 16-byte chunks (W = 14, 7, 35, 299 ...) are staged from aligned
+// 16-byte loads over the contiguous span of rows.  A last pixel block that runs past the image (14x14 and 7x7 outputs are not multiples of 16
 // pixels) computes on the last pixel again and is not stored.
+//
+// A batch of NIMG images is NIMG times the workgroups of one image, image after image: every image is tiled
+// alike, so what holds for one (placement of the tiles over the XCDs, the staged patch) holds for all.
 #pragma once
 #include <hip/hip_runtime.h>
 
@@ -36,9 +39,9 @@ namespace bfuse {
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 
-template <int CI_, int CO_, int H_, int W_, int KH_, int KW_, int S_, int P_, int BM_, int PB_, int KS_>
+template <int CI_, int CO_, int H_, int W_, int KH_, int KW_, int S_, int P_, int BM_, int PB_, int KS_, int NIMG_ = 1>
 struct ConvF32Lds {
-    static constexpr int CI = CI_, CO = CO_, H = H_, W = W_, KH = KH_, KW = KW_, S = S_, P = P_, BM = BM_, PB = PB_, KS = KS_;
+    static constexpr int CI = CI_, CO = CO_, H = H_, W = W_, KH = KH_, KW = KW_, S = S_, P = P_, BM = BM_, PB = PB_, KS = KS_, NIMG = NIMG_;
     static constexpr int OH = (H - KH + 2 * P) / S + 1, OW = (W - KW + 2 * P) / S + 1;
     static constexpr int HW = H * W, OHW = OH * OW, T = KH * KW;
     static constexpr int CG = CI >= 16 ? 16 : 4;        // channels per group
@@ -67,7 +70,9 @@ struct ConvF32Lds {
     static_assert(S >= 1 && OH >= 1 && OW >= 1, "shape");
 
     static constexpr int NCT = CO / BM;
-    static constexpr Dims3 GRID{NPT * NCT, 1, 1};
+    static constexpr int WG_PER_IMAGE = NPT * NCT;
+    static_assert(NIMG >= 1 && (long long)WG_PER_IMAGE * NIMG < (1LL << 31), "grid size");
+    static constexpr Dims3 GRID{WG_PER_IMAGE * NIMG, 1, 1};
     static constexpr Dims3 BLOCK{64 * KS, 1, 1};
     static constexpr int THREADS = 64 * KS;
     static constexpr bool HAS_BARRIERS = KS > 1;
@@ -114,6 +119,12 @@ struct ConvF32Lds {
         const float* __restrict__ X = static_cast<const float*>(I);
         const float* __restrict__ Wt = static_cast<const float*>(F);
         float* __restrict__ Y = static_cast<float*>(O);
+        if constexpr (NIMG > 1) {
+            const int img = vblock / WG_PER_IMAGE;
+            vblock -= img * WG_PER_IMAGE;
+            X += (size_t)img * CI * HW;
+            Y += (size_t)img * CO * OHW;
+        }
         int pt, ct;
         tile_of(vblock, pt, ct);
         const int p0 = pt * TP, co0 = ct * BM;
@@ -170,38 +181,80 @@ struct ConvF32Lds {
             const int cl = lane / LPC, cu = lane % LPC;
             // in batches of JB loads, so that a large patch (7x7 filters on 224-wide rows) does not need a
             // register per element
-            constexpr int JB = NLD < 64 / VW ? NLD : 64 / VW;
+            if constexpr (VW == 4 || W < 4) {
+                constexpr int JB = NLD < 16 ? NLD : 16;
+#pragma unroll 1
+                for (int j0 = 0; j0 < NLD; j0 += JB) {
+                    float v[JB][VW];
 #pragma unroll
-            for (int j0 = 0; j0 < NLD; j0 += JB) {
-                float v[JB][VW];
+                    for (int jj = 0; jj < JB; ++jj) {
+                        const int u = (j0 + jj) * LPC + cu;
+                        const int r = (u * VW) / W, x = (u * VW) % W;
+                        const int iy = iy_lo + r;
+                        const bool ok = j0 + jj < NLD && u < NU && iy >= 0 && iy < H && ci0 + cl < CI;
+                        const float* src = X + (size_t)(ci0 + cl) * HW + iy * W + x;
+                        if constexpr (VW == 4) {
+                            const f32x4 q = ok ? *reinterpret_cast<const f32x4*>(src) : f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int jj = 0; jj < JB; ++jj) {
-                    const int u = (j0 + jj) * LPC + cu;
-                    const int r = (u * VW) / W, x = (u * VW) % W;
-                    const int iy = iy_lo + r;
-                    const bool ok = j0 + jj < NLD && u < NU && iy >= 0 && iy < H && ci0 + cl < CI;
-                    const float* src = X + (size_t)(ci0 + cl) * HW + iy * W + x;
-                    if constexpr (VW == 4) {
-                        const f32x4 q = ok ? *reinterpret_cast<const f32x4*>(src) : f32x4{0.f, 0.f, 0.f, 0.f};
+                            for (int e = 0; e < 4; ++e) v[jj][e] = q[e];
+                        } else if constexpr (VW == 2) {
+                            const f32x2 q = ok ? *reinterpret_cast<const f32x2*>(src) : f32x2{0.f, 0.f};
+                            v[jj][0] = q[0];
+                            v[jj][1] = q[1];
+                        } else {
+                            v[jj][0] = ok ? *src : 0.f;
+                        }
+                    }
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) v[jj][e] = q[e];
-                    } else if constexpr (VW == 2) {
-                        const f32x2 q = ok ? *reinterpret_cast<const f32x2*>(src) : f32x2{0.f, 0.f};
-                        v[jj][0] = q[0];
-                        v[jj][1] = q[1];
-                    } else {
-                        v[jj][0] = ok ? *src : 0.f;
+                    for (int jj = 0; jj < JB; ++jj) {
+                        const int u = (j0 + jj) * LPC + cu;
+                        const int r = (u * VW) / W, x = (u * VW) % W;
+                        const int iy = iy_lo + r;
+                        if (j0 + jj < NLD && u < NU && iy >= 0 && iy < H && ci0 + cl < CI) {
+                            float* dst = reinterpret_cast<float*>(tile + (cl / 4) * PLANE + (r * WP + P + x) * 16) + cl % 4;
+#pragma unroll
+                            for (int e = 0; e < VW; ++e) dst[4 * e] = v[jj][e];
+                        }
                     }
                 }
+            } else {
+                // Image rows that do not start on 16-byte boundaries (odd widths; any width when the image itself
+                // starts off one): the rows of a channel that lie inside the image are one contiguous span, which
+                // is fetched with ALIGNED 16-byte loads from the boundary below its start; each of a vector's
+                // four floats then finds its own (row, column), and those before and behind the span are dropped.
+                const int r_lo = iy_lo < 0 ? -iy_lo : 0;
+                const int r_hi = H - iy_lo < R ? H - iy_lo : R;
+                const int len = (r_hi - r_lo) * W;
+                const float* span = X + (size_t)(ci0 + cl) * HW + (iy_lo + r_lo) * W;
+                const int mis = (int)((reinterpret_cast<size_t>(span) >> 2) & 3);
+                const f32x4* vec = reinterpret_cast<const f32x4*>(span - mis);
+                const bool chan = ci0 + cl < CI;
+                constexpr int NV = (R * W + 3) / 4 + 1;          // aligned vectors that can overlap a span
+                constexpr int NLA = (NV + LPC - 1) / LPC;
+                constexpr int JA = NLA < 16 ? NLA : 16;
+#pragma unroll 1
+                for (int j0 = 0; j0 < NLA; j0 += JA) {
+                    f32x4 v[JA];
 #pragma unroll
-                for (int jj = 0; jj < JB; ++jj) {
-                    const int u = (j0 + jj) * LPC + cu;
-                    const int r = (u * VW) / W, x = (u * VW) % W;
-                    const int iy = iy_lo + r;
-                    if (j0 + jj < NLD && u < NU && iy >= 0 && iy < H && ci0 + cl < CI) {
-                        float* dst = reinterpret_cast<float*>(tile + (cl / 4) * PLANE + (r * WP + P + x) * 16) + cl % 4;
+                    for (int jj = 0; jj < JA; ++jj) {
+                        const int u = (j0 + jj) * LPC + cu;
+                        const int i0 = 4 * u - mis;              // span index of the vector's first float
+                        v[jj] = (chan && i0 + 3 >= 0 && i0 < len) ? vec[u] : f32x4{0.f, 0.f, 0.f, 0.f};
+                    }
 #pragma unroll
-                        for (int e = 0; e < VW; ++e) dst[4 * e] = v[jj][e];
+                    for (int jj = 0; jj < JA; ++jj) {
+                        const int u = (j0 + jj) * LPC + cu;
+                        const int i0 = 4 * u - mis;
+                        int r = (i0 + W) / W - 1 + r_lo, x = (i0 + W) % W;   // i0 >= -3 and W >= 4
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            if (chan && i0 + e >= 0 && i0 + e < len)
+                                reinterpret_cast<float*>(tile + (cl / 4) * PLANE + (r * WP + P + x) * 16)[cl % 4] = v[jj][e];
+                            if (++x == W) {
+                                x = 0;
+                                ++r;
+                            }
+                        }
                     }
                 }
             }
@@ -274,6 +327,37 @@ struct ConvF32Lds {
         }
     }
 };
+
+// The tiling the library gives a convolution it has no hand-picked one for: as many output channels per
+// workgroup as keep the filter fragments of a wave within ~72 registers (the staged patch is shared by all
+// of them), 64 pixels (or the whole image when it has fewer), and as many waves over the channel groups as
+// leave room for two workgroups' patches in a CU's LDS.
+template <int CI, int CO, int H, int W, int KH, int KW, int S, int P, int NIMG>
+struct ConvTiling {
+    static constexpr int T = KH * KW;
+    static constexpr int OHW = ((H - KH + 2 * P) / S + 1) * ((W - KW + 2 * P) / S + 1);
+    static constexpr int pick_bm()
+    {
+        if (CI < 16) return 16;
+        if (CO % 64 == 0 && 4 * T <= 18) return 64;
+        if (CO % 48 == 0 && 3 * T <= 18) return 48;
+        if (CO % 32 == 0 && 2 * T <= 18) return 32;
+        return 16;
+    }
+    static constexpr int BM = pick_bm();
+    static constexpr int PB = OHW >= 64 ? 4 : (OHW + 15) / 16;
+    static constexpr int NGROUP = CI >= 16 ? CI / 16 : 1;
+    static constexpr int TILE = ConvF32Lds<CI, CO, H, W, KH, KW, S, P, BM, PB, 1, NIMG>::TILE_BYTES;
+    static constexpr int pick_ks()
+    {
+        if (NGROUP % 4 == 0 && 4 * TILE <= 80 * 1024) return 4;
+        if (NGROUP % 2 == 0 && 2 * TILE <= 80 * 1024) return 2;
+        return 1;
+    }
+    using type = ConvF32Lds<CI, CO, H, W, KH, KW, S, P, BM, PB, pick_ks(), NIMG>;
+};
+template <int CI, int CO, int H, int W, int KH, int KW, int S, int P, int NIMG = 1>
+using ConvF32Auto = typename ConvTiling<CI, CO, H, W, KH, KW, S, P, NIMG>::type;
 
 // An operator with its first two operands exchanged: a 1x1 / stride 1 convolution is the product
 // Wt[CO, CI] . X[CI, H*W], i.e. a GEMM whose first operand is the convolution's SECOND (the weights).

@@ -894,6 +894,79 @@ int bfuse_download(int side, void* O)
     return rc;
 }
 
+int bfuse_upload_part(int side, int tensor, size_t offset, const void* src, size_t bytes)
+{
+    if (side < 1 || side > kMaxKernels) return fail(BFUSE_ERR_ARG, "side must be 1 .. %d", kMaxKernels);
+    Side& s = g.side[side - 1];
+    if (!s.live) return fail(BFUSE_ERR_STATE, "kernel%d is not initialized", side);
+    if (tensor != 0 && tensor != 1) return fail(BFUSE_ERR_ARG, "tensor must be 0 (I) or 1 (F)");
+    if (!src) return fail(BFUSE_ERR_ARG, "null host buffer");
+    if (offset > s.bytes[tensor] || bytes > s.bytes[tensor] - offset)
+        return fail(BFUSE_ERR_ARG, "bytes %zu .. %zu are outside the tensor's %zu", offset, offset + bytes, s.bytes[tensor]);
+    if (bytes) HIP_TRY(hipMemcpy(static_cast<char*>(s.buf[tensor]) + offset, src, bytes, hipMemcpyHostToDevice));
+    return BFUSE_OK;
+}
+
+int bfuse_download_part(int side, size_t offset, void* dst, size_t bytes)
+{
+    if (side < 1 || side > kMaxKernels) return fail(BFUSE_ERR_ARG, "side must be 1 .. %d", kMaxKernels);
+    Side& s = g.side[side - 1];
+    if (!s.live) return fail(BFUSE_ERR_STATE, "kernel%d is not initialized", side);
+    if (!dst) return fail(BFUSE_ERR_ARG, "null host buffer");
+    if (offset > s.bytes[2] || bytes > s.bytes[2] - offset)
+        return fail(BFUSE_ERR_ARG, "bytes %zu .. %zu are outside the output's %zu", offset, offset + bytes, s.bytes[2]);
+    const int rc = sync_and_check();
+    if (rc && rc != BFUSE_ERR_SYNC) return rc;
+    if (bytes) HIP_TRY(hipMemcpy(dst, static_cast<const char*>(s.buf[2]) + offset, bytes, hipMemcpyDeviceToHost));
+    return rc;
+}
+
+// Two order-independent sums (mod 2^64) over the 32-bit words of each chunk: the words themselves, and the
+// words weighted by their position in the chunk.  grid = (parts, chunks).
+__global__ void checksum_kernel(const unsigned* __restrict__ p, size_t words_per_chunk, unsigned long long* __restrict__ sums)
+{
+    const unsigned* __restrict__ q = p + (size_t)blockIdx.y * words_per_chunk;
+    unsigned long long a = 0, b = 0;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < words_per_chunk; i += (size_t)gridDim.x * blockDim.x) {
+        const unsigned w = q[i];
+        a += w;
+        b += (unsigned long long)w * (unsigned long long)(i % 65521u + 1u);
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        a += __shfl_down(a, off, 64);
+        b += __shfl_down(b, off, 64);
+    }
+    if ((threadIdx.x & 63) == 0) {
+        atomicAdd(&sums[2 * (size_t)blockIdx.y], a);
+        atomicAdd(&sums[2 * (size_t)blockIdx.y + 1], b);
+    }
+}
+
+int bfuse_checksum_output(int side, size_t chunk_bytes, unsigned long long* sums)
+{
+    if (side < 1 || side > kMaxKernels) return fail(BFUSE_ERR_ARG, "side must be 1 .. %d", kMaxKernels);
+    Side& s = g.side[side - 1];
+    if (!s.live) return fail(BFUSE_ERR_STATE, "kernel%d is not initialized", side);
+    if (!sums) return fail(BFUSE_ERR_ARG, "null result buffer");
+    if (chunk_bytes == 0 || chunk_bytes % 4 != 0 || s.bytes[2] % chunk_bytes != 0)
+        return fail(BFUSE_ERR_ARG, "the chunk size %zu must be a multiple of 4 that divides the output's %zu bytes", chunk_bytes, s.bytes[2]);
+    const size_t chunks = s.bytes[2] / chunk_bytes, words = chunk_bytes / 4;
+    if (chunks > 65535) return fail(BFUSE_ERR_ARG, "%zu chunks: at most 65535", chunks);
+    const int rc = sync_and_check();
+    if (rc && rc != BFUSE_ERR_SYNC) return rc;
+    DevBuf d;
+    HIP_TRY(hipMalloc(&d.p, chunks * 2 * sizeof(unsigned long long)));
+    HIP_TRY(hipMemset(d.p, 0, chunks * 2 * sizeof(unsigned long long)));
+    size_t parts = (words + 256 * 16 - 1) / (256 * 16);   // ~16 words per thread
+    if (parts > 64) parts = 64;
+    if (parts < 1) parts = 1;
+    hipLaunchKernelGGL(checksum_kernel, dim3((unsigned)parts, (unsigned)chunks), dim3(256), 0, nullptr,
+                       static_cast<const unsigned*>(s.buf[2]), words, d.as<unsigned long long>());
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipMemcpy(sums, d.p, chunks * 2 * sizeof(unsigned long long), hipMemcpyDeviceToHost));
+    return rc;
+}
+
 int bfuse_synchronize(void)
 {
     if (!g.inited) return fail(BFUSE_ERR_STATE, "bfuse_init has not been called");

@@ -170,6 +170,29 @@ class Operation:
         _lib.check(self.l.bfuse_download(side + 1, O.ctypes.data))
         return O
 
+    def upload_part(self, side: int, tensor: int, offset: int, arr):
+        """Writes `arr` into tensor 0 (I) or 1 (F) of the side, starting at element `offset`."""
+        k = self.k[side]
+        a = np.ascontiguousarray(arr, dtype=_DT[k.elem_bytes[tensor]])
+        _lib.check(self.l.bfuse_upload_part(side + 1, tensor, offset * a.itemsize, a.ctypes.data, a.nbytes))
+
+    def download_part(self, side: int, offset: int, count: int) -> np.ndarray:
+        """`count` elements of the side's output, starting at element `offset`."""
+        O = np.empty(count, _DT[self.k[side].elem_bytes[2]])
+        _lib.check(self.l.bfuse_download_part(side + 1, offset * O.itemsize, O.ctypes.data, O.nbytes))
+        return O
+
+    def checksum_output(self, side: int, chunk_elems: int) -> np.ndarray:
+        """Device-side checksums of the side's output in chunks of `chunk_elems` elements: an array
+        [chunks, 2] of uint64 that `checksum_of` reproduces on the host for expected contents."""
+        k = self.k[side]
+        total = int(np.prod(k.shapes[2]))
+        if chunk_elems < 1 or total % chunk_elems:
+            raise ValueError(f"{k.name}: chunks of {chunk_elems} elements do not divide the output's {total}")
+        sums = np.zeros((total // chunk_elems, 2), np.uint64)
+        _lib.check(self.l.bfuse_checksum_output(side + 1, chunk_elems * k.elem_bytes[2], sums.ctypes.data))
+        return sums
+
     def _mode_args(self, mode: str, fused: Optional[KernelHandle]):
         a, b = self.k
         if mode == "kernel1":
@@ -384,6 +407,14 @@ def bf16_to_f32(x: np.ndarray) -> np.ndarray:
     out = np.empty(x.shape, np.float32)
     _lib.lib().bfuse_bf16_to_f32(x.size, x.ctypes.data, out.ctypes.data)
     return out
+
+
+def checksum_of(chunk: np.ndarray) -> np.ndarray:
+    """What Operation.checksum_output reports for a chunk with these contents (a whole number of 32-bit words)."""
+    w = np.ascontiguousarray(chunk).ravel().view(np.uint32).astype(np.uint64)
+    pos = (np.arange(w.size, dtype=np.uint64) % np.uint64(65521)) + np.uint64(1)
+    with np.errstate(over="ignore"):
+        return np.array([w.sum(dtype=np.uint64), (w * pos).sum(dtype=np.uint64)], np.uint64)
 
 
 def check_matrix(o: np.ndarray, o_ans: np.ndarray, eps: float = 1e-3) -> int:

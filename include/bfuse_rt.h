@@ -208,6 +208,18 @@ int bfuse_zero_output(int side);
 int bfuse_download(int side, void* O);
 int bfuse_synchronize(void);
 
+/* The same for a part of a tensor: operands and results of several GB (the reference's benchmark.yaml runs every
+ * operator at batch 1024) need not pass through one host array.  `tensor`: 0 = I, 1 = F; offsets and sizes in
+ * bytes.  No counterpart in the reference, whose harness copies whole tensors (operation_cu.py:74-118). */
+int bfuse_upload_part(int side, int tensor, size_t offset, const void* src, size_t bytes);
+int bfuse_download_part(int side, size_t offset, void* dst, size_t bytes);
+/* Checksums of the side's output, computed on the device: the output is cut into chunks of `chunk_bytes`
+ * (a multiple of 4 that divides it; at most 65535 chunks) and sums[2c], sums[2c+1] receive, mod 2^64, the sum
+ * of chunk c's 32-bit words w[i] and the sum of w[i] * (i mod 65521 + 1).  Two runs wrote the same bytes iff
+ * (up to collisions) their sums agree -- the comparison the reference makes on the host with check_matrix
+ * (operation_cu.py:29-45), for outputs too large to copy back. */
+int bfuse_checksum_output(int side, size_t chunk_bytes, unsigned long long* sums);
+
 enum {
     BFUSE_MODE_KERNEL1 = 0,   /* the reference CLI's T = 0..4 (main_cc.py:22-36) */
     BFUSE_MODE_KERNEL2 = 1,

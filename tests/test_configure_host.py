@@ -119,10 +119,11 @@ def test_a_kernel_registered_for_other_shapes_than_the_ids_is_refused():
 
 
 @pytest.mark.skipif(not os.path.isdir(REF_EXAMPLES), reason="the reference's example configs are not on this machine")
-@pytest.mark.parametrize("name,count", [("llm.yaml", 26), ("resnet-18.yaml", 12)])
+@pytest.mark.parametrize("name,count", [("llm.yaml", 26), ("resnet-18.yaml", 12), ("benchmark.yaml", 84), ("inception_v3.yaml", 60)])
 def test_the_references_own_example_configs_resolve_completely(tmp_path, name, count):
-    """The reference's examples (read in place) ship with empty fusion sets: every id goes into both sets, as its
-    benchmark.yaml does, and EVERY id resolves without --skip-missing -- in fp32, the reference's arithmetic."""
+    """The reference's examples (read in place): every id goes into both fusion sets (llm.yaml and resnet-18.yaml
+    ship with empty sets; benchmark.yaml and inception_v3.yaml, every operator at batch 1024, name one copy of
+    each id per set), and EVERY id resolves without --skip-missing -- in fp32, the reference's arithmetic."""
     with open(os.path.join(REF_EXAMPLES, name)) as f:
         doc = yaml.safe_load(f)
     ids = list(doc["KernelInfo"])

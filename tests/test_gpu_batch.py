@@ -1,0 +1,200 @@
+"""The operators of the reference's test-utils/examples/benchmark.yaml and inception_v3.yaml: every operator at
+batch 1024 (convolutions of 1024 images, 1024 independent batched products, dense layers of 1024 rows).
+
+Operands and results of these run to several GB, so nothing passes through one host array: the batch is made of
+12 variants -- three random base items, each scaled by 2^-1, 1, 2 and 4 -- dealt over the 1024 positions, and
+
+  * the three unscaled base results are compared with the CPU oracle (1e-5 of max(|ref|, rms));
+  * the nine scaled variants must equal their base result times the same power of two, bit for bit
+    (convolution and matrix product are linear, and scaling by a power of two is exact);
+  * every one of the 1024 results is compared, through a checksum computed on the device, with the variant
+    that belongs at its position -- a result written to the wrong place, read from the wrong item or left
+    out changes a checksum;
+  * selector operands make every output element of the first three items one operand element exactly.
+"""
+import numpy as np
+import pytest
+
+import bfuse_project_amd as bf
+from bfuse_project_amd.operation import checksum_of, fill_normal
+from oracle import oracle as orf
+from tests import oracle_cases
+
+pytestmark = pytest.mark.gpu
+
+PARTNER = "layernorm_512x768"     # an Operation holds two sides; the second is not launched here
+N = 1024
+EXPS = (-1, 0, 1, 2)
+NBASE = 3
+NVAR = NBASE * len(EXPS)
+
+
+def variant_of(b):
+    """Variant (base = j % 3, exponent = EXPS[j // 3]) of batch position b: the first 12 positions are the 12
+    variants in order, the rest follow a fixed scramble."""
+    return b if b < NVAR else (b * 7 + b // NVAR) % NVAR
+
+
+def _scales():
+    return [np.float32(2.0 ** EXPS[j // NBASE]) for j in range(NVAR)]
+
+
+def _check_batch(op, item, heads, name, flops_per_item):
+    """heads: the first NVAR results, [NVAR, item].  Linearity among them, then every position by checksum."""
+    sc = _scales()
+    unit = [NBASE * EXPS.index(0) + v for v in range(NBASE)]
+    for j in range(NVAR):
+        assert heads[j].tobytes() == (heads[unit[j % NBASE]] * sc[j]).tobytes(), f"variant {j}: not its base result times {sc[j]}"
+    want = np.stack([checksum_of(heads[j]) for j in range(NVAR)])
+    got = op.checksum_output(0, item)
+    bad = [b for b in range(N) if not np.array_equal(got[b], want[variant_of(b)])]
+    assert not bad, f"{len(bad)} of {N} results differ from the variant at their position, first {bad[:8]}"
+    t = float(np.mean(op.time("kernel1", warmup=1, reps=3)[0]))
+    print(f"[batch] {name}: {t / 1e3:.2f} ms ({flops_per_item * N / t * 1e-6:.1f} TFLOP/s)", flush=True)
+
+
+# ---- convolutions: N, H, W, CO, CI, KH, KW, stride, padding (scripts/configure_kernels.py:28-38) -----------
+CONVS = [
+    (224, 224, 64, 3, 7, 7, 2, 3), (56, 56, 64, 64, 3, 3, 1, 1), (56, 56, 64, 64, 1, 1, 1, 0), (56, 56, 128, 64, 3, 3, 2, 1),
+    (28, 28, 128, 128, 3, 3, 1, 1), (56, 56, 128, 64, 1, 1, 2, 0), (28, 28, 256, 128, 3, 3, 2, 1), (14, 14, 256, 256, 3, 3, 1, 1),
+    (28, 28, 256, 128, 1, 1, 2, 0), (14, 14, 512, 256, 3, 3, 2, 1), (7, 7, 512, 512, 3, 3, 1, 1), (14, 14, 512, 256, 1, 1, 2, 0),
+    (35, 35, 64, 256, 1, 1, 1, 0), (35, 35, 48, 256, 1, 1, 1, 0), (35, 35, 64, 288, 1, 1, 1, 0), (35, 35, 48, 288, 1, 1, 1, 0),
+    (35, 35, 384, 288, 3, 3, 2, 0), (35, 35, 96, 96, 3, 3, 2, 0), (17, 17, 192, 768, 1, 1, 1, 0), (17, 17, 128, 768, 1, 1, 1, 0),
+    (17, 17, 160, 768, 1, 1, 1, 0), (17, 17, 320, 192, 3, 3, 2, 0),
+    (299, 299, 32, 3, 3, 3, 2, 0), (149, 149, 32, 32, 3, 3, 1, 0), (147, 147, 64, 32, 3, 3, 1, 1), (73, 73, 80, 64, 1, 1, 1, 0),
+    (73, 73, 192, 80, 3, 3, 1, 0), (35, 35, 64, 192, 1, 1, 1, 0), (35, 35, 48, 192, 1, 1, 1, 0), (35, 35, 64, 48, 5, 5, 1, 2),
+    (35, 35, 96, 64, 3, 3, 1, 1), (35, 35, 96, 96, 3, 3, 1, 1), (35, 35, 32, 192, 1, 1, 1, 0), (8, 8, 320, 1280, 1, 1, 1, 0),
+    (8, 8, 384, 1280, 1, 1, 1, 0), (8, 8, 448, 1280, 1, 1, 1, 0), (8, 8, 384, 448, 3, 3, 1, 1), (8, 8, 192, 1280, 1, 1, 1, 0),
+    (8, 8, 320, 2048, 1, 1, 1, 0), (8, 8, 384, 2048, 1, 1, 1, 0), (8, 8, 448, 2048, 1, 1, 1, 0), (8, 8, 192, 2048, 1, 1, 1, 0)]
+
+
+@pytest.mark.parametrize("h,w,co,ci,kh,kw,s,p", CONVS)
+def test_convolution_of_1024_images(h, w, co, ci, kh, kw, s, p):
+    name = f"conv{kh}x{kw}s{s}p{p}_f32_{N}x{ci}x{h}x{w}_{co}"
+    print(f"[batch] conv2d [{N}, {h}, {w}, {co}, {ci}, {kh}, {kw}, {s}, {p}] -> {name}", flush=True)
+    oh, ow = (h - kh + 2 * p) // s + 1, (w - kw + 2 * p) // s + 1
+    img, item = ci * h * w, co * oh * ow
+    bases = np.maximum(fill_normal(0xBC0 + ci + h + co, NBASE * img, 0.0, 1.0), 0.0).reshape(NBASE, img)
+    wt = fill_normal(0xBC8 + co + kh + ci, co * ci * kh * kw, 0.0, 0.05)
+    sc = _scales()
+    variants = [bases[j % NBASE] * sc[j] for j in range(NVAR)]
+    # selector filters: output channel c copies input channel (5c + 1) mod CI under tap (c mod KH, (2c + 1) mod KW)
+    sel = np.zeros((co, ci, kh, kw), np.float32)
+    cs = np.arange(co)
+    sel[cs, (5 * cs + 1) % ci, cs % kh, (2 * cs + 1) % kw] = 1.0
+    with bf.Operation(name, PARTNER) as op:
+        assert tuple(op.k[0].shapes[0]) == (N, ci, h, w) and tuple(op.k[0].shapes[2]) == (N, co, oh, ow)
+        for b in range(N):
+            op.upload_part(0, 0, b * img, variants[variant_of(b)])
+        op.upload_part(0, 1, 0, sel)
+        op.zero_outputs()
+        op.launch("kernel1")
+        ysel = op.download_part(0, 0, NBASE * item).reshape(NBASE, co, oh, ow)
+        op.upload_part(0, 1, 0, wt)
+        op.zero_outputs()
+        op.launch("kernel1")
+        heads = op.download_part(0, 0, NVAR * item).reshape(NVAR, item)
+        _check_batch(op, item, heads, name, 2.0 * co * ci * kh * kw * oh * ow)
+    for v in range(NBASE):     # position v holds base v scaled by 2^EXPS[0]
+        xp = np.pad(variants[v].reshape(ci, h, w), ((0, 0), (p, p), (p, p)))
+        want_sel = np.stack([xp[(5 * c_ + 1) % ci, c_ % kh:c_ % kh + s * oh:s, (2 * c_ + 1) % kw:(2 * c_ + 1) % kw + s * ow:s] for c_ in range(co)])
+        assert np.array_equal(ysel[v], want_sel), "selector filters: an output element is not the input element it selects"
+    want = orf.conv2d(bases.reshape(NBASE, ci, h, w), wt.reshape(co, ci, kh, kw), s=s, p=p)
+    unit0 = NBASE * EXPS.index(0)
+    st = oracle_cases.rel_stats(heads[unit0:unit0 + NBASE], want, 1e-5)
+    print(f"[parity] {name}: worst |d|/max(|ref|,rms) {st['worst_floor_rel']:.3e}; {st['n_fail']} fail", flush=True)
+    assert st["n_fail"] == 0
+
+
+# ---- batched products: batch, M, K, N; C[b] = A[b] . B[b]^T with B [b, N, K] (configure_kernels.py:14-19) -----
+BGEMMS = [(512, 64, 512), (512, 512, 64), (512, 128, 512), (512, 512, 128), (256, 64, 256), (256, 256, 64), (256, 80, 256),
+          (256, 256, 80), (208, 64, 208), (208, 208, 64), (208, 80, 208), (208, 208, 80)]
+
+
+@pytest.mark.parametrize("m,k,n", BGEMMS)
+def test_1024_batched_products(m, k, n):
+    name = f"bgemm_f32_{N}x{m}x{k}x{n}"
+    print(f"[batch] bgemm [{N}, {m}, {k}, {n}] -> {name}", flush=True)
+    a = fill_normal(0x1BA + k + m, NBASE * m * k, 0.0, 1.0).reshape(NBASE, m * k)
+    w = fill_normal(0x2BA + n + k, NBASE * n * k, 0.0, 0.125).reshape(NBASE, n * k)
+    sc = _scales()
+    a_var = [a[j % NBASE] * sc[j] for j in range(NVAR)]
+    # A[r, :] = one-hot at k = (r + v) mod K  =>  C[r, j] = B[j, (r + v) mod K] exactly
+    sel = np.zeros((NBASE, m, k), np.float32)
+    for v in range(NBASE):
+        sel[v, np.arange(m), (np.arange(m) + v) % k] = 1.0
+    with bf.Operation(name, PARTNER) as op:
+        for b in range(N):
+            j = variant_of(b)
+            op.upload_part(0, 0, b * m * k, a_var[j])
+            op.upload_part(0, 1, b * n * k, w[j % NBASE])
+        op.zero_outputs()
+        op.launch("kernel1")
+        heads = op.download_part(0, 0, NVAR * m * n).reshape(NVAR, m * n)
+        _check_batch(op, m * n, heads, name, 2.0 * m * n * k)
+        op.upload_part(0, 0, 0, sel)
+        op.zero_outputs()
+        op.launch("kernel1")
+        csel = op.download_part(0, 0, NBASE * m * n).reshape(NBASE, m, n)
+    for v in range(NBASE):
+        assert np.array_equal(csel[v], w[v].reshape(n, k)[:, (np.arange(m) + v) % k].T), "selector inputs: an output element is not the B element it selects"
+    want = np.stack([orf.gemm_f32(a[v].reshape(m, k), w[v].reshape(n, k), b_is_nk=True) for v in range(NBASE)])
+    unit0 = NBASE * EXPS.index(0)
+    st = oracle_cases.rel_stats(heads[unit0:unit0 + NBASE], want, 1e-5)
+    print(f"[parity] {name}: worst |d|/max(|ref|,rms) {st['worst_floor_rel']:.3e}; {st['n_fail']} fail", flush=True)
+    assert st["n_fail"] == 0
+
+
+# ---- dense layers of 1024 rows: batch, in, out (configure_kernels.py:21-26), weight from the (out, in) layout ----
+DENSES = [(768, 768), (768, 3072), (3072, 768), (768, 2304), (4096, 4096), (4096, 1024), (4096, 14336), (14336, 4096)]
+
+
+@pytest.mark.parametrize("k,n", DENSES)
+def test_dense_layer_of_1024_rows(k, n):
+    m = N
+    name = f"gemm_f32_{m}x{k}x{n}"
+    print(f"[batch] dense [{m}, {k}, {n}] -> {name} (weight through transpose32_{n}x{k})", flush=True)
+    a = fill_normal(0xA4B + k, m * k, 0.0, 1.0)
+    w_nk = fill_normal(0xB4B + n, n * k, 0.0, 0.02)
+    with bf.Operation(f"transpose32_{n}x{k}", "bias_relu_4096") as op:
+        w_kn = op.run_kernel(0, w_nk, np.zeros(1, np.float32))
+    assert np.array_equal(w_kn.reshape(k, n), w_nk.reshape(n, k).T)
+    with bf.Operation(name, PARTNER) as op:
+        c = op.run_kernel(0, a, w_kn)
+        sel = np.zeros((m, k), np.float32)
+        sel[np.arange(m), (np.arange(m) * 37) % k] = 1.0
+        cs = op.run_kernel(0, sel.ravel(), w_kn)
+        op.upload(0, a, w_kn)
+        t = float(np.mean(op.time("kernel1", warmup=3, reps=10)[0]))
+    W = w_nk.reshape(n, k)
+    assert np.array_equal(cs.reshape(m, n), W[:, (np.arange(m) * 37) % k].T), "selector inputs: an output element is not the weight it selects"
+    rows, cols = np.arange(3, m, 8), np.arange(5, n, 8)
+    want = orf.gemm_f32(np.ascontiguousarray(a.reshape(m, k)[rows]), np.ascontiguousarray(W[cols]), b_is_nk=True)
+    got = np.ascontiguousarray(c.reshape(m, n)[np.ix_(rows, cols)])
+    st = oracle_cases.rel_stats(got, want, 1e-5)
+    print(f"[parity] {name}: sample {len(rows)} x {len(cols)} over K = {k}: worst |d|/max(|ref|,rms) {st['worst_floor_rel']:.3e}; "
+          f"{st['n_fail']} fail; {t:.1f} us ({2.0 * m * n * k / t * 1e-6:.1f} TFLOP/s)", flush=True)
+    assert st["n_fail"] == 0
+
+
+def test_checksums_and_partial_copies_agree_with_whole_copies():
+    """The helpers the tests above rest on, on a small kernel: a partial upload / download moves the bytes it
+    says, and the device's checksums are the ones the host computes from a downloaded output."""
+    m, k, n = 512, 768, 768
+    a, w = fill_normal(1, m * k, 0.0, 1.0), fill_normal(2, k * n, 0.0, 0.05)
+    with bf.Operation(f"gemm_f32_{m}x{k}x{n}", PARTNER) as op:
+        c = op.run_kernel(0, a, w)
+        op.upload(0, np.zeros(m * k, np.float32), w)
+        for r0 in range(0, m, 128):
+            op.upload_part(0, 0, r0 * k, a[r0 * k:(r0 + 128) * k])
+        op.zero_outputs()
+        op.launch("kernel1")
+        assert op.download(0).tobytes() == c.tobytes()
+        assert op.download_part(0, 5 * n + 3, 1000).tobytes() == c.ravel()[5 * n + 3:5 * n + 1003].tobytes()
+        sums = op.checksum_output(0, 64 * n)
+        want = np.stack([checksum_of(c.ravel()[i * 64 * n:(i + 1) * 64 * n]) for i in range(m // 64)])
+        assert np.array_equal(sums, want)
+        with pytest.raises(bf.BfuseError):
+            op.upload_part(0, 0, m * k - 10, a[:11])
+        with pytest.raises(ValueError):
+            op.checksum_output(0, 7)
