@@ -59,7 +59,7 @@ EXPORTS = [
     "bfuse_last_error", "bfuse_init", "bfuse_shutdown", "bfuse_device_info", "bfuse_device_memory",
     "bfuse_plan_threads", "bfuse_plan_blocks", "bfuse_map_block", "bfuse_map_thread", "bfuse_map_blocks_device", "bfuse_map_blocks_device_noalloc", "bfuse_probe_placement", "bfuse_set_plan",
     "bfuse_set_sync_spin_limit",
-    "bfuse_kernel_count", "bfuse_kernel_at", "bfuse_kernel_find",
+    "bfuse_kernel_count", "bfuse_kernel_at", "bfuse_kernel_find", "bfuse_load_kernels", "bfuse_kernel_op_type", "bfuse_kernel_op_lds",
     "bfuse_set_elem_bytes", "initialize_kernel1", "initialize_kernel2", "finalize_kernel1", "finalize_kernel2",
     "run_kernel1", "run_kernel2", "run_parallel", "run_fuse",
     "bfuse_upload", "bfuse_zero_output", "bfuse_download", "bfuse_synchronize", "bfuse_launch",
@@ -105,6 +105,10 @@ def lib():
         l.bfuse_probe_placement.argtypes = [C.c_int, C.c_int, C.c_int, vp, vp, vp, vp, vp]
         l.bfuse_kernel_at.argtypes = [C.c_int, C.POINTER(KernelInfoC)]
         l.bfuse_kernel_find.argtypes = [C.c_char_p, C.POINTER(KernelInfoC)]
+        l.bfuse_load_kernels.argtypes = [C.c_char_p]
+        l.bfuse_kernel_op_type.argtypes = [C.c_char_p]
+        l.bfuse_kernel_op_type.restype = C.c_char_p
+        l.bfuse_kernel_op_lds.argtypes = [C.c_char_p]
         for n in ("initialize_kernel1", "initialize_kernel2"):
             getattr(l, n).argtypes = [ip, ip, ip]
         for n in ("run_kernel1", "run_kernel2"):

@@ -380,7 +380,24 @@ struct KernelEntry {
     unsigned (*read_sync_timeouts)();  // device counter of GroupSync give-ups in this module (read and reset)
     int (*set_spin_limit)(unsigned);   // polls a side barrier of this module makes before it gives up (0 = ok)
     int (*set_plan)(const BlockPlan*); // bfuse_rt: per-kernel hook called when a plan is installed (0 = ok); the plan itself travels as a kernel argument
+    const char* op_type = "";          // single: the operator's C++ type, spelled so that it can be compiled again
+    int smem_bytes = -1;               // single: sizeof(Op::Smem), the LDS the operator's body declares
 };
+
+// The operator type as the compiler spells it, every template argument written out
+// ("bfuse::GemmF32Dma<512, 768, 768, 32, 48, 4, 0, 3>"): what a module of fused kernels built later for a
+// pair of registered kernels names its sides by.
+template <class Op>
+const char* op_type_name()
+{
+    const char* pretty = __PRETTY_FUNCTION__;        // "... [Op = <type>]"
+    static const std::string name = [pretty] {
+        const std::string f = pretty;
+        const size_t a = f.find("Op = "), b = f.rfind(']');
+        return (a == std::string::npos || b == std::string::npos || b < a + 5) ? std::string() : f.substr(a + 5, b - a - 5);
+    }();
+    return name.c_str();
+}
 
 // per-module (translation unit) access to its own copies of the side-barrier device variables
 struct ModuleHooks {
@@ -408,6 +425,8 @@ KernelEntry make_single_entry(const char* name, const void* func, TensorDesc i, 
     e.io[0] = i; e.io[1] = f; e.io[2] = o;
     e.read_sync_timeouts = hooks.read_sync_timeouts;
     e.set_spin_limit = hooks.set_spin_limit;
+    e.op_type = op_type_name<Op>();
+    e.smem_bytes = (int)sizeof(typename Op::Smem);
     return e;
 }
 

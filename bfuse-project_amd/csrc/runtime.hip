@@ -4,9 +4,12 @@
 #include <hip/hip_runtime.h>
 #include <hip/hip_ext.h>
 
+#include <dlfcn.h>
+
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <string>
 #include <map>
@@ -724,8 +727,72 @@ static void fill_info(const KernelEntry& e, bfuse_kernel_info* o)
 // them; bfuse_kernel_find still finds them by name.
 static bool enumerated(const KernelEntry& e) { return e.name.rfind("selftest_", 0) != 0; }
 
+// Modules of fused kernels built after the library (one shared object per suite): loading one runs its
+// registrars, which append to the registry above.  BFUSE_KERNEL_MODULES (paths separated by ':') names modules
+// to load before the first look at the registry, so that every program over this library -- the command-line
+// driver included -- sees them without an option of its own.
+static int load_kernels(const char* path)
+{
+    static std::vector<std::string> loaded;
+    for (const auto& p : loaded)
+        if (p == path) return BFUSE_OK;
+    const size_t before = registry().size();
+    void* h = dlopen(path, RTLD_NOW | RTLD_LOCAL);
+    if (!h) return fail(BFUSE_ERR_ARG, "cannot load kernel module '%s': %s", path, dlerror());
+    if (registry().size() == before) {
+        dlclose(h);
+        return fail(BFUSE_ERR_ARG, "'%s' registered no kernel: not a module built against this library", path);
+    }
+    loaded.emplace_back(path);
+    return BFUSE_OK;
+}
+
+static int load_env_modules()
+{
+    static bool done = false;
+    static int status = BFUSE_OK;
+    if (done) return status;
+    done = true;
+    const char* env = getenv("BFUSE_KERNEL_MODULES");
+    if (!env) return status;
+    std::string all(env);
+    size_t a = 0;
+    while (a <= all.size()) {
+        size_t b = all.find(':', a);
+        if (b == std::string::npos) b = all.size();
+        if (b > a && (status = load_kernels(all.substr(a, b - a).c_str()))) return status;
+        a = b + 1;
+    }
+    return status;
+}
+
+int bfuse_load_kernels(const char* shared_object_path)
+{
+    if (!shared_object_path || !*shared_object_path) return fail(BFUSE_ERR_ARG, "null module path");
+    int rc = load_env_modules();
+    if (rc) return rc;
+    return load_kernels(shared_object_path);
+}
+
+const char* bfuse_kernel_op_type(const char* name)
+{
+    if (!name || load_env_modules()) return nullptr;
+    for (const auto& e : registry())
+        if (e.name == name) return e.kind == kSingle ? e.op_type : nullptr;
+    return nullptr;
+}
+
+int bfuse_kernel_op_lds(const char* name)
+{
+    if (!name || load_env_modules()) return -1;
+    for (const auto& e : registry())
+        if (e.name == name) return e.kind == kSingle ? e.smem_bytes : -1;
+    return -1;
+}
+
 int bfuse_kernel_count(void)
 {
+    if (load_env_modules()) return 0;
     int n = 0;
     for (const auto& e : registry()) n += enumerated(e);
     return n;
@@ -734,6 +801,7 @@ int bfuse_kernel_count(void)
 int bfuse_kernel_at(int index, bfuse_kernel_info* out)
 {
     if (index < 0 || !out) return fail(BFUSE_ERR_ARG, "index out of range");
+    if (int rc = load_env_modules()) return rc;
     for (const auto& e : registry())
         if (enumerated(e) && index-- == 0) {
             fill_info(e, out);
@@ -745,6 +813,7 @@ int bfuse_kernel_at(int index, bfuse_kernel_info* out)
 int bfuse_kernel_find(const char* name, bfuse_kernel_info* out)
 {
     if (!name || !out) return fail(BFUSE_ERR_ARG, "null argument");
+    if (int rc = load_env_modules()) return rc;
     for (const auto& e : registry())
         if (e.name == name) {
             fill_info(e, out);

@@ -3,6 +3,7 @@ operation_cu.py:123-256): initialize / run_kernel1 / run_kernel2 / run_parallel 
 finalize over numpy buffers, plus the device-resident launch and GPU-side timing entry points.
 """
 import ctypes as C
+import os
 from dataclasses import dataclass, replace
 from typing import List, Optional, Sequence
 
@@ -407,6 +408,11 @@ def bf16_to_f32(x: np.ndarray) -> np.ndarray:
     out = np.empty(x.shape, np.float32)
     _lib.lib().bfuse_bf16_to_f32(x.size, x.ctypes.data, out.ctypes.data)
     return out
+
+
+def load_kernels(path: str) -> None:
+    """Adds the fused kernels of a module built by build_pairs to the registry (found by name from then on)."""
+    _lib.check(_lib.lib().bfuse_load_kernels(os.fspath(path).encode()))
 
 
 def checksum_of(chunk: np.ndarray) -> np.ndarray:

@@ -1,11 +1,12 @@
 """One command from a user config to the speed-up table: the reference's scripts/quick_start.py
 (`quick_start.py example -o file`, its six steps :27-160).
 
-    python -m bfuse_project_amd.quick_start example.yaml -o OUT [--dtype f32|bf16] [--skip-missing]
+    python -m bfuse_project_amd.quick_start example.yaml -o OUT [--dtype f32|bf16] [--skip-missing] [--build-pairs]
 
   reference step                                   here
   [1/6] configure test-suite (TVM kernels)         [1/3] `configure`: ids resolved against the registry
-  [2/6] generate fused kernels (hfuse, bfuse)      -- the fused kernels are in the library (OUT/config/fused.yaml lists them)
+  [2/6] generate fused kernels (hfuse, bfuse)      -- the fused kernels are in the library (OUT/config/fused.yaml lists them);
+                                                   --build-pairs: `build_pairs` writes and compiles the pairs it lacks
   [3/6] generate benchmark, [4/6] make             -- the harness is the library; nothing is generated or compiled
   [5/6] profile the benchmark                      [2/3] `suite`: every pair in every mode, validated, traces under OUT/exec
   [6/6] draw profile results                       [3/3] speed-up table: OUT/summary.md, OUT/summary.json
@@ -22,8 +23,9 @@ def main(argv=None) -> int:
     ap.add_argument("-o", dest="file", default="test-suite", help="output directory of the generated test-suite")
     ap.add_argument("--dtype", choices=("f32", "bf16"), default=None)
     ap.add_argument("--skip-missing", action="store_true", help="drop operator ids the library has no kernel for")
+    ap.add_argument("--build-pairs", action="store_true", help="build the fused kernels the library lacks for this suite's pairs (hipcc)")
     args = ap.parse_args(argv)
-    from . import configure, suite
+    from . import build_pairs, configure, suite
 
     print("[1/3] ========================= Configure test-suite =========================", flush=True)
     if not os.path.exists(args.example):
@@ -42,6 +44,10 @@ def main(argv=None) -> int:
     print("[2/3] ========================= Profile the benchmark =========================", flush=True)
     info = suite.load_info(os.path.join(args.file, "config", "info.yaml"))
     try:
+        if args.build_pairs:
+            built = build_pairs.build(args.file)
+            print(f"  built {len(built['kernels'])} fused kernels", flush=True)
+        build_pairs.load_suite_modules(args.file)
         rows = suite.run_suite(info, args.file, validate=True)
     except Exception as e:   # a failed validation or a device error ends the run, as the reference's check=True does
         print(f"Error occurs while profiling the benchmark: {e}", file=sys.stderr)

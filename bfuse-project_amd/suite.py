@@ -47,6 +47,11 @@ def load_info(path: str) -> dict:
     return info
 
 
+def suite_dir_of(info_path: str) -> str:
+    """The suite directory of `<suite>/config/info.yaml` (where configure wrote it)."""
+    return os.path.dirname(os.path.dirname(os.path.abspath(info_path)))
+
+
 def set_names(info: dict) -> Tuple[List[str], List[str]]:
     return list(info["FusionSet"][0]["Set"]), list(info["FusionSet"][1]["Set"])
 
@@ -413,9 +418,18 @@ def main(argv=None) -> int:
         print(f"error: {e}", file=sys.stderr)
         return 1
     exec_dir = os.path.join(args.out, "exec")
+    # fused kernels built for this suite after the library (build_pairs): this process loads them, the
+    # driver's processes find them through the environment
+    from . import build_pairs
+    try:
+        modules = build_pairs.load_suite_modules(suite_dir_of(args.file))
+    except Exception as e:
+        print(f"error: {e}", file=sys.stderr)
+        return 1
     if args.commands:
+        prefix = f"BFUSE_KERNEL_MODULES={':'.join(modules)} " if modules else ""
         for c in exec_commands(info, args.benchmark, exec_dir, args.triangular, args.file):
-            print(" ".join(c))
+            print(prefix + " ".join(c))
         return 0
     rows = analyze(info, exec_dir, args.triangular) if args.analyze else run_suite(info, args.out, not args.no_validate, args.triangular)
     os.makedirs(args.out, exist_ok=True)

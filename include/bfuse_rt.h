@@ -159,6 +159,22 @@ int bfuse_kernel_count(void);
 int bfuse_kernel_at(int index, bfuse_kernel_info* out);
 int bfuse_kernel_find(const char* name, bfuse_kernel_info* out);
 
+/* Fused kernels built after the library.  The reference generates and compiles the fused kernels of a suite
+ * when the suite is configured (scripts/configure_kernels.py:229-320 runs the fuser over every pair of the
+ * user's config; CMakeLists_txt.py compiles the result into the suite's binary).  Here
+ * `python -m bfuse_project_amd.build_pairs <suite dir>` writes the pairs of a configured suite that the library
+ * holds no fused kernel for as instantiations over the registered operators' own types and compiles them into
+ * one shared object per suite; bfuse_load_kernels adds its kernels to the registry (by name, like the built-in
+ * ones).  Modules named in the environment variable BFUSE_KERNEL_MODULES (paths separated by ':') are loaded
+ * before the first look at the registry, whatever the program.
+ * bfuse_kernel_op_type: the C++ type of a standalone kernel's operator, spelled with every template argument
+ * (NULL for unknown names and fused kernels) -- what such a module names its sides by.
+ * bfuse_kernel_op_lds: the bytes of LDS that operator's body declares (-1 likewise), known without a device:
+ * whether two operators fit one workgroup is decided from it before anything is compiled. */
+int bfuse_load_kernels(const char* shared_object_path);
+const char* bfuse_kernel_op_type(const char* name);
+int bfuse_kernel_op_lds(const char* name);
+
 /* ------------------------------------------------------------------------------------------
  * Harness functions -- test-utils/test-suite-files/operation_h.py:9-27.  Same names and
  * argument meaning.  Differences: data pointers are void* (bf16 sides), an int status is
