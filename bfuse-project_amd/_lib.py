@@ -46,7 +46,7 @@ class KernelInfoC(C.Structure):
                 ("regs", C.c_int), ("lds_bytes", C.c_int), ("shape", (C.c_int * 4) * 3),
                 ("elem_bytes", C.c_int * 3), ("side", (C.c_char * 64) * 2),
                 ("pattern", C.c_int), ("p0", C.c_int), ("p1", C.c_int),
-                ("n_sides", C.c_int), ("side_more", (C.c_char * 64) * (MAXK - 2))]
+                ("n_sides", C.c_int), ("side_more", (C.c_char * 64) * (MAXK - 2)), ("matrix_cores", C.c_int)]
 
 
 class LaunchDescC(C.Structure):
@@ -63,7 +63,7 @@ EXPORTS = [
     "bfuse_set_elem_bytes", "initialize_kernel1", "initialize_kernel2", "finalize_kernel1", "finalize_kernel2",
     "run_kernel1", "run_kernel2", "run_parallel", "run_fuse",
     "bfuse_upload", "bfuse_zero_output", "bfuse_download", "bfuse_synchronize", "bfuse_launch",
-    "bfuse_upload_part", "bfuse_download_part", "bfuse_checksum_output",
+    "bfuse_upload_part", "bfuse_download_part", "bfuse_checksum_output", "bfuse_fill_uniform_device",
     "bfuse_time", "bfuse_time_batched", "bfuse_module_load", "bfuse_module_unload", "bfuse_module_launch",
     "bfuse_initialize_side", "bfuse_finalize_side", "bfuse_launch_list", "bfuse_time_list",
     "bfuse_fill_uniform", "bfuse_fill_normal", "bfuse_f32_to_bf16", "bfuse_bf16_to_f32", "bfuse_check_matrix",
@@ -120,6 +120,7 @@ def lib():
         l.bfuse_upload_part.argtypes = [C.c_int, C.c_int, C.c_size_t, vp, C.c_size_t]
         l.bfuse_download_part.argtypes = [C.c_int, C.c_size_t, vp, C.c_size_t]
         l.bfuse_checksum_output.argtypes = [C.c_int, C.c_size_t, vp]
+        l.bfuse_fill_uniform_device.argtypes = [C.c_int, C.c_int, C.c_ulonglong, C.c_float, C.c_float]
         l.bfuse_launch.argtypes = [C.c_int, vp, up, up, vp, up, up]
         fp = C.POINTER(C.c_float)
         l.bfuse_time.argtypes = [C.c_int, vp, up, up, vp, up, up, C.c_int, C.c_int, fp, fp, fp]

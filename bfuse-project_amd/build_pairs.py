@@ -13,7 +13,7 @@ into `<suite>/hip/pairs_<n>.hip` -- the operator types exactly as the library sp
 checks (csrc/Makefile, target `module`).  `<suite>/config/modules.yaml` then names the module; `suite`,
 `quick_start` and `benchmark` (through BFUSE_KERNEL_MODULES) load it and find the new kernels by name.
 
-    python -m bfuse_project_amd.build_pairs SUITE [--forms both|bfuse|hfuse] [--chunk N] [--only K1+K2 ...] [-j J]
+    python -m bfuse_project_amd.build_pairs SUITE [--forms both|bfuse|hfuse] [--chunk N] [--triangular] [--only K1+K2 ...] [-j J]
 
 Thread-level fusion is written only where it can work: both workgroups fit one (at most 1024 threads and
 160 KB of LDS together) and at most one side synchronises (config.choose_fusion's rule).
@@ -95,11 +95,76 @@ def source_text(kernels: Sequence[dict], chunk: int = 256, types=op_type) -> str
     return "\n".join(lines) + "\n"
 
 
-def suite_pairs(suite: str) -> List[Tuple[str, str]]:
+def spilling_kernels(res_text: str) -> List[str]:
+    """Kernels a compilation's resource remarks report scratch memory or register spills for."""
+    out, name = [], None
+    for line in res_text.splitlines():
+        if "Function Name:" in line:
+            name = line.split("Function Name:", 1)[1].split()[0]
+        elif name and any(f"{what}: " in line and int(line.split(f"{what}: ", 1)[1].split()[0]) > 0
+                          for what in ("ScratchSize [bytes/lane]", "VGPRs Spill", "SGPRs Spill")):
+            if name not in out:
+                out.append(name)
+    return out
+
+
+def _unit_kernel(line: str) -> Optional[str]:
+    """The fused kernel a line of a written translation unit defines (or records as not built)."""
+    if line.startswith("BFUSE_BFUSE_KERNEL("):
+        a = [x.strip() for x in line[len("BFUSE_BFUSE_KERNEL("):-1].split(",")]
+        return f"{a[0]}_{a[2]}_fused_bfuse{a[4]}"
+    if line.startswith("BFUSE_HFUSE_KERNEL("):
+        a = [x.strip() for x in line[len("BFUSE_HFUSE_KERNEL("):-1].split(",")]
+        return f"{a[0]}_{a[2]}_fused_hfuse"
+    if line.startswith("// not built"):
+        return line.rsplit(": ", 1)[1].strip()
+    return None
+
+
+def written(hip_dir: str) -> List[str]:
+    """Fused kernels the translation units of a suite already hold (built, to be built, or found not to fit)."""
+    out = []
+    if os.path.isdir(hip_dir):
+        for f in sorted(os.listdir(hip_dir)):
+            if f.startswith("pairs_") and f.endswith(".hip"):
+                with open(os.path.join(hip_dir, f)) as fh:
+                    out += [n for n in map(_unit_kernel, fh.read().splitlines()) if n]
+    return out
+
+
+def drop_spilling(hip_dir: str) -> List[str]:
+    """Removes, from every pairs_*.hip whose last compilation reported spills, the kernels that spilled."""
+    dropped = []
+    for f in sorted(os.listdir(hip_dir)):
+        if not (f.startswith("pairs_") and f.endswith(".res")):
+            continue
+        with open(os.path.join(hip_dir, f)) as fh:
+            bad = spilling_kernels(fh.read())
+        if not bad:
+            continue
+        src = os.path.join(hip_dir, f[:-4] + ".hip")
+        with open(src) as fh:
+            lines = fh.read().splitlines()
+        keep = []
+        for line in lines:
+            name = None if line.startswith("//") else _unit_kernel(line)
+            if name in bad:
+                dropped.append(name)
+                keep.append(f"// not built (does not fit the register file in this form): {name}")
+            else:
+                keep.append(line)
+        with open(src, "w") as fh:
+            fh.write("\n".join(keep) + "\n")
+    return dropped
+
+
+def suite_pairs(suite: str, triangular: bool = False) -> List[Tuple[str, str]]:
+    """The suite's pairs of registry names; `triangular`: the upper triangle the reference profiles when its two
+    sets list the same operators (scripts/profile_test_suite.py:13-47)."""
     with open(os.path.join(suite, "config", "info.yaml")) as f:
         info = yaml.safe_load(f)
     s0, s1 = (s["Set"] for s in info["FusionSet"])
-    return [(a, b) for a in s0 for b in s1]
+    return [(s0[i], s1[j]) for i in range(len(s0)) for j in range(i if triangular else 0, len(s1))]
 
 
 def module_paths(suite: str) -> List[str]:
@@ -122,21 +187,22 @@ def load_suite_modules(suite: str) -> List[str]:
 
 
 def build(suite: str, forms: str = "both", chunk: int = 256, only: Optional[Sequence[str]] = None, per_file: int = 2,
-          jobs: int = 8, compile_: bool = True) -> dict:
+          jobs: int = 8, compile_: bool = True, triangular: bool = False) -> dict:
     """Writes <suite>/hip/pairs_*.hip for the suite's pairs that lack a fused kernel and builds the module.
     Returns {"kernels": [...], "files": [...], "module": path or None}."""
     from .operation import list_kernels
     load_suite_modules(suite)      # what an earlier run built counts as held
     registry = {k.name: k for k in list_kernels()}
-    pairs = suite_pairs(suite)
+    pairs = suite_pairs(suite, triangular)
     if only:
         keep = {tuple(o.split("+", 1)) for o in only}
         unknown = keep - set(pairs)
         if unknown:
             raise LookupError(f"not pairs of this suite: {sorted(unknown)}")
         pairs = [p for p in pairs if p in keep]
-    todo = wanted(pairs, registry, forms, chunk)
     hip = os.path.join(suite, "hip")
+    have = set(written(hip))       # units of an earlier, possibly interrupted, run are not written twice
+    todo = [k for k in wanted(pairs, registry, forms, chunk) if k["name"] not in have]
     os.makedirs(hip, exist_ok=True)
     first = len([f for f in os.listdir(hip) if f.startswith("pairs_") and f.endswith(".hip")])
     files = []
@@ -146,16 +212,26 @@ def build(suite: str, forms: str = "both", chunk: int = 256, only: Optional[Sequ
             f.write(source_text(todo[i:i + per_file], chunk))
         files.append(path)
     module = os.path.join(hip, "libbfuse_pairs.so")
-    if not todo and not os.path.exists(module):
-        return {"kernels": [], "files": [], "module": None}
-    if compile_ and (todo or not os.path.exists(module)):
-        r = subprocess.run(["make", "-C", CSRC, f"MODDIR={os.path.abspath(hip)}", f"-j{jobs}", "module"],
-                           capture_output=True, text=True)
+    if not todo and not have:
+        return {"kernels": [], "files": [], "module": None, "dropped": []}
+    dropped: List[str] = []
+    if compile_:      # make decides what is out of date (new units, or headers of the library that changed)
+        cmd = ["make", "-C", CSRC, f"MODDIR={os.path.abspath(hip)}", f"-j{jobs}", "-k", "module"]
+        r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
-            raise RuntimeError(f"building {module} failed:\n{r.stdout[-3000:]}\n{r.stderr[-3000:]}")
+            # A fused kernel that needs more registers than its launch bounds leave (a side that already fills the
+            # register file, thread-fused with another) fails the library's no-spill check: such kernels are taken
+            # out of their translation units and the build is run once more; anything else is an error.
+            dropped = drop_spilling(hip)
+            if not dropped:
+                raise RuntimeError(f"building {module} failed:\n{r.stdout[-3000:]}\n{r.stderr[-3000:]}")
+            r = subprocess.run(cmd, capture_output=True, text=True)
+            if r.returncode != 0:
+                raise RuntimeError(f"building {module} failed:\n{r.stdout[-3000:]}\n{r.stderr[-3000:]}")
+            todo = [k for k in todo if k["name"] not in dropped]
         with open(os.path.join(suite, "config", "modules.yaml"), "w") as f:
             yaml.safe_dump([os.path.join("hip", "libbfuse_pairs.so")], f)
-    return {"kernels": todo, "files": files, "module": module if compile_ else None}
+    return {"kernels": todo, "files": files, "module": module if compile_ else None, "dropped": dropped}
 
 
 def main(argv=None) -> int:
@@ -164,17 +240,20 @@ def main(argv=None) -> int:
     ap.add_argument("--forms", choices=("both", "bfuse", "hfuse"), default="both")
     ap.add_argument("--chunk", type=int, default=256, help="workgroups of one side per chunk of the block-fused dispatch (one round over the CUs)")
     ap.add_argument("--only", nargs="*", metavar="K1+K2", help="registry names of the pairs to build (default: every pair of the suite)")
+    ap.add_argument("--triangular", action="store_true", help="only the pairs (i, j >= i) of two sets that list the same operators, as the reference profiles them")
     ap.add_argument("--per-file", type=int, default=2, help="fused kernels per translation unit")
     ap.add_argument("-j", type=int, default=8, dest="jobs")
     ap.add_argument("--write-only", action="store_true", help="write the .hip files, do not compile")
     args = ap.parse_args(argv)
     try:
-        r = build(args.suite, args.forms, args.chunk, args.only, args.per_file, args.jobs, not args.write_only)
+        r = build(args.suite, args.forms, args.chunk, args.only, args.per_file, args.jobs, not args.write_only, args.triangular)
     except (LookupError, RuntimeError, OSError) as e:
         print(f"build_pairs: {e}", file=sys.stderr)
         return 1
     for k in r["kernels"]:
         print(k["name"])
+    for name in r["dropped"]:
+        print(f"not built (registers): {name}", file=sys.stderr)
     print(f"{len(r['kernels'])} fused kernels in {len(r['files'])} files" + (f"; module {r['module']}" if r["module"] else ""))
     return 0
 

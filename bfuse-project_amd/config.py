@@ -123,7 +123,7 @@ class FusionContext:
         return KernelInfo(self.FusedKernelName, True, self.FusedGridDim, self.FusedBlockDim, 32)
 
 
-def choose_fusion(a: KernelInfo, b: KernelInfo, lds_a: int, lds_b: int, cus: int = 256) -> dict:
+def choose_fusion(a: KernelInfo, b: KernelInfo, lds_a: int, lds_b: int, cus: int = 256, matrix=(False, False)) -> dict:
     """Picks hfuse vs bfuse vs no fusion from each side's footprint (and its ExecTime where known).
 
     * Both sides with barriers -> block fusion (a wave-granular LDS barrier on both sides of
@@ -143,6 +143,12 @@ def choose_fusion(a: KernelInfo, b: KernelInfo, lds_a: int, lds_b: int, cus: int
       (a batched GEMM resident in one round) does not: its displaced workgroups start when the
       partner ends and the pair takes as long as serial, or longer.  Without times, a side that
       does not fit is taken for short-lived only if it has neither barriers nor LDS.
+    * Two sides that each keep every matrix pipe of the chip busy on their own (`matrix`: the side's inner
+      loop is a stream of MFMAs; and its grid puts at least one wave on every SIMD of every CU) have
+      nothing to give each other but their ends: whatever the fused form, one side's workgroups only
+      take the place of the other's.  Such a pair is left unfused.  (Measured on the reference's
+      benchmark arrangement -- 903 pairs of GEMMs, batched products and convolutions at batch 1024,
+      all of this kind: block fusion 0.91x, thread-level fusion 0.79x, two streams 1.00x.)
     """
     ta, tb = a.dims.block[0] * a.dims.block[1] * a.dims.block[2], b.dims.block[0] * b.dims.block[1] * b.dims.block[2]
     wa, wb = -(-ta // 64), -(-tb // 64)
@@ -201,7 +207,12 @@ def choose_fusion(a: KernelInfo, b: KernelInfo, lds_a: int, lds_b: int, cus: int
             else:
                 kx = (a, b)[x]
                 pays = pays or (slots >= 1 and 2 * slots >= needed[x] and not kx.HasBarriers and (lds_a, lds_b)[x] == 0)
-    fuse = "hfuse" if hfuse_ok and ga == gb else ("bfuse" if pays else ("hfuse" if hfuse_ok and max(ga, gb) <= cus else "none"))
+    saturates = (bool(matrix[0]) and ga * wa >= 4 * cus, bool(matrix[1]) and gb * wb >= 4 * cus)
+    if saturates[0] and saturates[1]:
+        pays = False
+        fuse = "none"
+    else:
+        fuse = "hfuse" if hfuse_ok and ga == gb else ("bfuse" if pays else ("hfuse" if hfuse_ok and max(ga, gb) <= cus else "none"))
     return {"hfuse_ok": hfuse_ok, "prefer": "hfuse" if hfuse_ok and ga == gb else "bfuse",
             "wg_per_cu": (na, nb), "rounds": (rounds_a, rounds_b),
             # one chunk per round over the CUs (measured best on MI355X: the compute-bound side lands
@@ -212,4 +223,5 @@ def choose_fusion(a: KernelInfo, b: KernelInfo, lds_a: int, lds_b: int, cus: int
             "ratio_M": max(1, max(ga, gb) // max(1, min(ga, gb))),
             "needed": needed, "cap_lds": min(cap_lds, 1 << 20), "cap_waves": cap_waves, "side_by_side": side_by_side,
             "predicted_us": predicted, "serial_us": (times[0] + times[1]) if known else None,
+            "saturates_matrix_cores": saturates,
             "bfuse_pays": pays, "fuse": fuse}

@@ -382,7 +382,13 @@ struct KernelEntry {
     int (*set_plan)(const BlockPlan*); // bfuse_rt: per-kernel hook called when a plan is installed (0 = ok); the plan itself travels as a kernel argument
     const char* op_type = "";          // single: the operator's C++ type, spelled so that it can be compiled again
     int smem_bytes = -1;               // single: sizeof(Op::Smem), the LDS the operator's body declares
+    bool matrix_cores = false;         // single: the operator declares MATRIX_CORES (its inner loop is a stream of MFMAs)
 };
+
+template <class Op, class = void>
+struct UsesMatrixCores : std::false_type {};
+template <class Op>
+struct UsesMatrixCores<Op, std::void_t<decltype(Op::MATRIX_CORES)>> : std::bool_constant<Op::MATRIX_CORES> {};
 
 // The operator type as the compiler spells it, every template argument written out
 // ("bfuse::GemmF32Dma<512, 768, 768, 32, 48, 4, 0, 3>"): what a module of fused kernels built later for a
@@ -407,8 +413,13 @@ struct ModuleHooks {
 
 std::vector<KernelEntry>& registry();
 
+// Adds an entry to the registry.  A module of fused kernels built against other headers than the library it is
+// loaded into would hand over entries of another layout: the size travels with the entry and such entries are
+// refused (bfuse_load_kernels then fails).
+void register_kernel(const KernelEntry& e, size_t entry_size);
+
 struct Registrar {
-    explicit Registrar(const KernelEntry& e) { registry().push_back(e); }
+    explicit Registrar(const KernelEntry& e) { register_kernel(e, sizeof(KernelEntry)); }
 };
 
 template <class Op>
@@ -427,6 +438,7 @@ KernelEntry make_single_entry(const char* name, const void* func, TensorDesc i, 
     e.set_spin_limit = hooks.set_spin_limit;
     e.op_type = op_type_name<Op>();
     e.smem_bytes = (int)sizeof(typename Op::Smem);
+    e.matrix_cores = UsesMatrixCores<Op>::value;
     return e;
 }
 

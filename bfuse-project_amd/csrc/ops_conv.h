@@ -49,6 +49,7 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 template <int CI_, int CO_, int H_, int W_, int BM_, int PB_, int KS_>
 struct Conv3x3F32Lds {
+    static constexpr bool MATRIX_CORES = true;   // the inner loop is a stream of MFMAs (what the fusion chooser asks)
     static constexpr int CI = CI_, CO = CO_, H = H_, W = W_, BM = BM_, PB = PB_, KS = KS_;
     static constexpr int HW = H * W;
     static constexpr int TM = BM / 16;

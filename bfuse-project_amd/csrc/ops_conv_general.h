@@ -41,6 +41,7 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 template <int CI_, int CO_, int H_, int W_, int KH_, int KW_, int S_, int P_, int BM_, int PB_, int KS_, int NIMG_ = 1>
 struct ConvF32Lds {
+    static constexpr bool MATRIX_CORES = true;   // the inner loop is a stream of MFMAs (what the fusion chooser asks)
     static constexpr int CI = CI_, CO = CO_, H = H_, W = W_, KH = KH_, KW = KW_, S = S_, P = P_, BM = BM_, PB = PB_, KS = KS_, NIMG = NIMG_;
     static constexpr int OH = (H - KH + 2 * P) / S + 1, OW = (W - KW + 2 * P) / S + 1;
     static constexpr int HW = H * W, OHW = OH * OW, T = KH * KW;

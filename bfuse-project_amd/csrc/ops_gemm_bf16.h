@@ -63,6 +63,7 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 template <int M_, int N_, int K_, int BM_, int BN_, int NSTG_ = 3, int PD_ = 4, int WGM_ = 2, int WGN_ = 2, int PW_ = 0, int EARLY_ = 0,
           bool CLK_ = false>
 struct GemmBf16NTDma {
+    static constexpr bool MATRIX_CORES = true;   // the inner loop is a stream of MFMAs (what the fusion chooser asks)
     static constexpr bool CLK = CLK_;
     static constexpr int STAMP_WORDS = 8;   // clock x 3, wall x 3, XCC_ID, HW_ID
     static constexpr int M = M_, N = N_, K = K_, BM = BM_, BN = BN_, NSTG = NSTG_;

@@ -58,6 +58,7 @@ __device__ __forceinline__ float gelu_tanh(float x)
 // scripts/configure_kernels.py:14-19,40-48); workgroup v works on batch v / tiles, tile v % tiles.
 template <int M_, int N_, int K_, int BM_, int BN_, int KS_, int EPI_ = kEpiNone, int NBUF_ = 2, int SCHED_ = 1, bool B_NK_ = false, int BATCH_ = 1>
 struct GemmF32 {
+    static constexpr bool MATRIX_CORES = true;   // the inner loop is a stream of MFMAs (what the fusion chooser asks)
     static constexpr bool B_NK = B_NK_;
     static constexpr int BATCH = BATCH_;
     static constexpr int M = M_, N = N_, K = K_, BM = BM_, BN = BN_, KS = KS_, EPI = EPI_;

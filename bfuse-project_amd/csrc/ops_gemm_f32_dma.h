@@ -42,6 +42,7 @@ namespace bfuse {
 // workgroup barrier per K-stage, which costs about what the six loads per stage did -- no faster.)
 template <int M_, int N_, int K_, int BM_, int BN_, int KS_, int EPI_ = kEpiNone, int NSTG_ = 3>
 struct GemmF32Dma {
+    static constexpr bool MATRIX_CORES = true;   // the inner loop is a stream of MFMAs (what the fusion chooser asks)
     static constexpr int M = M_, N = N_, K = K_, BM = BM_, BN = BN_, KS = KS_, EPI = EPI_, NSTG = NSTG_;
     static constexpr int TM = BM / 16;
     static constexpr int G4 = BN / 64;          // 64-column groups

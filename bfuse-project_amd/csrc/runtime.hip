@@ -25,6 +25,17 @@ std::vector<KernelEntry>& registry()
     static std::vector<KernelEntry> r;
     return r;
 }
+
+static int g_refused_entries = 0;   // entries of another layout (a module built against other headers)
+
+void register_kernel(const KernelEntry& e, size_t entry_size)
+{
+    if (entry_size != sizeof(KernelEntry)) {
+        ++g_refused_entries;
+        return;
+    }
+    registry().push_back(e);
+}
 }  // namespace bfuse
 
 using namespace bfuse;
@@ -395,14 +406,14 @@ __global__ void placement_kernel(unsigned* hw_id, unsigned* xcc_id, unsigned lon
         if (wall_clock64() == 0ull) hw_id[0] = 0u;  // never true: keeps the loop
 }
 
-inline unsigned long long splitmix64(unsigned long long x)
+__host__ __device__ inline unsigned long long splitmix64(unsigned long long x)
 {
     x += 0x9E3779B97F4A7C15ull;
     x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
     x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
     return x ^ (x >> 31);
 }
-inline double u01(unsigned long long seed, unsigned long long i)  // in (0,1)
+__host__ __device__ inline double u01(unsigned long long seed, unsigned long long i)  // in (0,1)
 {
     const unsigned long long r = splitmix64(seed * 0xD1342543DE82EF95ull + i);
     return ((double)(r >> 11) + 0.5) * (1.0 / 9007199254740992.0);
@@ -719,6 +730,7 @@ static void fill_info(const KernelEntry& e, bfuse_kernel_info* o)
     o->pattern = e.pattern;
     o->p0 = e.p0;
     o->p1 = e.p1;
+    o->matrix_cores = e.kind == kSingle && e.matrix_cores;
 }
 
 // Kernels whose names start with `selftest_` exist for the library's own tests (operators that are
@@ -737,8 +749,14 @@ static int load_kernels(const char* path)
     for (const auto& p : loaded)
         if (p == path) return BFUSE_OK;
     const size_t before = registry().size();
+    const int refused = bfuse::g_refused_entries;
     void* h = dlopen(path, RTLD_NOW | RTLD_LOCAL);
     if (!h) return fail(BFUSE_ERR_ARG, "cannot load kernel module '%s': %s", path, dlerror());
+    if (bfuse::g_refused_entries != refused) {
+        // its kernels that did register stay (their code is loaded); the caller is told to rebuild
+        return fail(BFUSE_ERR_ARG, "'%s' was built against other headers than this library (%d kernels refused): rebuild it (build_pairs)",
+                    path, bfuse::g_refused_entries - refused);
+    }
     if (registry().size() == before) {
         dlclose(h);
         return fail(BFUSE_ERR_ARG, "'%s' registered no kernel: not a module built against this library", path);
@@ -1034,6 +1052,41 @@ int bfuse_checksum_output(int side, size_t chunk_bytes, unsigned long long* sums
     HIP_TRY(hipGetLastError());
     HIP_TRY(hipMemcpy(sums, d.p, chunks * 2 * sizeof(unsigned long long), hipMemcpyDeviceToHost));
     return rc;
+}
+
+// The values of bfuse_fill_uniform (and of bfuse_f32_to_bf16 over them), written where they are needed: integer
+// hash, two double operations and a conversion, the same on both sides.
+__global__ void fill_uniform_kernel(void* __restrict__ out, size_t n, int elem, unsigned long long seed, float lo, float hi)
+{
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        const float v = (float)((double)lo + ((double)hi - (double)lo) * u01(seed, i));
+        if (elem == 4) {
+            static_cast<float*>(out)[i] = v;
+        } else {
+            unsigned u = __float_as_uint(v);
+            static_cast<unsigned short*>(out)[i] = (u & 0x7fffffffu) > 0x7f800000u
+                                                       ? (unsigned short)((u >> 16) | 0x0040u)
+                                                       : (unsigned short)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+        }
+    }
+}
+
+int bfuse_fill_uniform_device(int side, int tensor, unsigned long long seed, float lo, float hi)
+{
+    if (side < 1 || side > kMaxKernels) return fail(BFUSE_ERR_ARG, "side must be 1 .. %d", kMaxKernels);
+    Side& s = g.side[side - 1];
+    if (!s.live) return fail(BFUSE_ERR_STATE, "kernel%d is not initialized", side);
+    if (tensor != 0 && tensor != 1) return fail(BFUSE_ERR_ARG, "tensor must be 0 (I) or 1 (F)");
+    if (s.elem[tensor] != 4 && s.elem[tensor] != 2)
+        return fail(BFUSE_ERR_ARG, "device fill writes fp32 or bf16 tensors, this one has %d-byte elements", s.elem[tensor]);
+    const size_t n = s.bytes[tensor] / (size_t)s.elem[tensor];
+    size_t blocks = (n + 256 * 8 - 1) / (256 * 8);
+    if (blocks > 16384) blocks = 16384;
+    if (blocks < 1) blocks = 1;
+    hipLaunchKernelGGL(fill_uniform_kernel, dim3((unsigned)blocks), dim3(256), 0, nullptr, s.buf[tensor], n, s.elem[tensor], seed, lo, hi);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipDeviceSynchronize());
+    return BFUSE_OK;
 }
 
 int bfuse_synchronize(void)

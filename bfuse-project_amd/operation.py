@@ -31,6 +31,7 @@ class KernelHandle:
     p0: int
     p1: int
     n_sides: int = 2          # kernels a fused kernel runs (1 for a standalone kernel)
+    matrix: bool = False      # standalone kernel whose inner loop is a stream of MFMAs (GEMMs, convolutions)
 
 
 def _handle(ci: "_lib.KernelInfoC") -> KernelHandle:
@@ -38,7 +39,7 @@ def _handle(ci: "_lib.KernelInfoC") -> KernelHandle:
                         ci.regs, ci.lds_bytes, tuple(tuple(s) for s in ci.shape), tuple(ci.elem_bytes),
                         tuple([ci.side[0].value.decode(), ci.side[1].value.decode()] +
                               [ci.side_more[i].value.decode() for i in range(max(0, ci.n_sides - 2))]),
-                        ci.pattern, ci.p0, ci.p1, ci.n_sides)
+                        ci.pattern, ci.p0, ci.p1, ci.n_sides, bool(ci.matrix_cores))
 
 
 def kernel_info(name: str) -> KernelHandle:
@@ -182,6 +183,10 @@ class Operation:
         O = np.empty(count, _DT[self.k[side].elem_bytes[2]])
         _lib.check(self.l.bfuse_download_part(side + 1, offset * O.itemsize, O.ctypes.data, O.nbytes))
         return O
+
+    def fill_uniform_device(self, side: int, tensor: int, seed: int, lo: float, hi: float):
+        """Fills tensor 0 (I) or 1 (F) of the side in HBM with the values fill_uniform(seed, n, lo, hi) gives."""
+        _lib.check(self.l.bfuse_fill_uniform_device(side + 1, tensor, seed, lo, hi))
 
     def checksum_output(self, side: int, chunk_elems: int) -> np.ndarray:
         """Device-side checksums of the side's output in chunks of `chunk_elems` elements: an array

@@ -224,9 +224,39 @@ def read_own(path: str, name: str) -> List[float]:
     return [r["Duration"] for r in read_trace(path) if r["Name"] == name][WARMUP_TRIALS:]
 
 
-def run_suite(info: dict, out_dir: str, validate: bool = True, triangular: bool = False, log=print) -> List[dict]:
+def _fill_on_device(op, side: int, seed: int) -> bool:
+    """The operands `_synthetic` would upload, written in HBM instead; False for a side with operands the
+    device fill does not write (byte blobs)."""
+    k = op.k[side]
+    if k.name.startswith("rmsnorm_rope_bf16") or any(e not in (2, 4) for e in k.elem_bytes[:2]):
+        return False
+    op.fill_uniform_device(side, 0, seed, -0.5, 0.5)
+    op.fill_uniform_device(side, 1, seed + 1, -0.5, 0.5)
+    return True
+
+
+def _chunks(handle) -> int:
+    """Elements per checksum chunk of a kernel's output: the output cut into as many chunks (up to 1024) as divide it."""
+    total = int(np.prod(handle.shapes[2]))
+    unit = 4 // handle.elem_bytes[2] if handle.elem_bytes[2] < 4 else 1
+    for n in (1024, 512, 256, 128, 64, 32, 16, 8, 4, 2, 1):
+        if total % n == 0 and (total // n) % unit == 0:
+            return total // n
+    return total
+
+
+def run_suite(info: dict, out_dir: str, validate: bool = True, triangular: bool = False, log=print, resident: bool = False,
+              rows: Optional[Tuple[int, int]] = None) -> List[dict]:
     """Runs the matrix over resident buffers with the library's dispatch timestamps, writes one
-    trace per (method, i, j) under `<out_dir>/exec/` and returns the analysed rows."""
+    trace per (method, i, j) under `<out_dir>/exec/` and returns the analysed rows.
+
+    `resident`: for operators whose operands and results run to GB (the reference's benchmark.yaml: every
+    operator at batch 1024) -- the same uniform operands are written on the device instead of being filled on
+    the host and copied, a fused kernel's outputs are compared with the unfused kernels' through checksums
+    computed on the device (up to 1024 chunks per output) instead of being copied back, and long kernels are
+    sampled fewer than 30 times (at least 5) so that a mode takes about a quarter of a second.
+    `rows` = (lo, hi): only the pairs whose first operator is lo <= i < hi of the first set (a long matrix run in
+    parts; the traces of all parts under one `exec/` are analysed together with --analyze)."""
     from . import tuner
     from .operation import Operation
     a, b = set_names(info)
@@ -247,17 +277,33 @@ def run_suite(info: dict, out_dir: str, validate: bool = True, triangular: bool 
         return rows
 
     for i, j in combos(info, triangular):
+        if rows is not None and not rows[0] <= i < rows[1]:
+            continue
         k1, k2 = a[i], b[j]
         with Operation(k1, k2) as op:
-            I1, F1 = _synthetic(op.k[0], 0xB5F05E + 2 * i)
-            I2, F2 = _synthetic(op.k[1], 0xB5F05E + 1000 + 2 * j)
-            op.upload(0, I1, F1)
-            op.upload(1, I2, F2)
+            on_device = [False, False]
+            for side, seed in ((0, 0xB5F05E + 2 * i), (1, 0xB5F05E + 1000 + 2 * j)):
+                on_device[side] = resident and _fill_on_device(op, side, seed)
+            I1, F1 = (None, None) if on_device[0] else _synthetic(op.k[0], 0xB5F05E + 2 * i)
+            I2, F2 = (None, None) if on_device[1] else _synthetic(op.k[1], 0xB5F05E + 1000 + 2 * j)
+            if not on_device[0]:
+                op.upload(0, I1, F1)
+            if not on_device[1]:
+                op.upload(1, I2, F2)
             base = None
-            if validate:
+            if validate and resident:
+                op.zero_outputs()
+                op.launch("serial")
+                base = (op.checksum_output(0, _chunks(op.k[0])), op.checksum_output(1, _chunks(op.k[1])))
+                if not (base[0][:, 0].any() and base[1][:, 0].any()):
+                    raise RuntimeError(f"{k1} / {k2}: an unfused kernel wrote nothing")
+            elif validate:
                 base = (op.run_kernel(0, I1, F1), op.run_kernel(1, I2, F2))
                 op.upload(0, I1, F1)
                 op.upload(1, I2, F2)
+            if resident:
+                est = float(np.mean(op.time("serial", warmup=1, reps=2)[0]))
+                n_rep = int(min(TIMED_TRIALS, max(5, 0.25e6 / max(est, 1.0))))
             # warm-ups are part of the trace, as in the reference's -n 33 runs
             t = op.time("kernel1", warmup=0, reps=WARMUP_TRIALS + n_rep)
             write_trace(os.path.join(exec_dir, f"0_{i}_0.csv"), trace_of(t[0], t[1], t[2], [k1]))
@@ -284,7 +330,13 @@ def run_suite(info: dict, out_dir: str, validate: bool = True, triangular: bool 
             for kind, idx in (("hfuse", 3), ("bfuse", 4)):
                 best = None
                 for h in fused_variants(k1, k2)[kind]:
-                    if validate:
+                    if validate and resident:
+                        op.zero_outputs()
+                        op.launch(kind, h)
+                        got = (op.checksum_output(0, _chunks(op.k[0])), op.checksum_output(1, _chunks(op.k[1])))
+                        if not (np.array_equal(got[0], base[0]) and np.array_equal(got[1], base[1])):
+                            raise RuntimeError(f"{h.name}: output differs from the unfused kernels")
+                    elif validate:
                         op.zero_outputs()
                         Q1, Q2 = op.run_fuse(h, I1, F1, I2, F2)
                         if not (np.array_equal(Q1.view(np.uint8), base[0].view(np.uint8)) and np.array_equal(Q2.view(np.uint8), base[1].view(np.uint8))):
@@ -410,6 +462,8 @@ def main(argv=None) -> int:
     ap.add_argument("--analyze", action="store_true", help="only analyse traces already under OUT/exec")
     ap.add_argument("--triangular", action="store_true", help="walk the upper triangle as the reference does")
     ap.add_argument("--no-validate", action="store_true")
+    ap.add_argument("--rows", metavar="LO:HI", help="run only the pairs whose first operator is LO <= i < HI of the first set")
+    ap.add_argument("--resident", action="store_true", help="operands written and results compared on the device (operators at batch 1024)")
     ap.add_argument("--benchmark", default=os.path.join(os.path.dirname(os.path.abspath(__file__)), "benchmark"))
     args = ap.parse_args(argv)
     try:
@@ -431,7 +485,8 @@ def main(argv=None) -> int:
         for c in exec_commands(info, args.benchmark, exec_dir, args.triangular, args.file):
             print(prefix + " ".join(c))
         return 0
-    rows = analyze(info, exec_dir, args.triangular) if args.analyze else run_suite(info, args.out, not args.no_validate, args.triangular)
+    rows = analyze(info, exec_dir, args.triangular) if args.analyze else run_suite(info, args.out, not args.no_validate, args.triangular, resident=args.resident,
+                                                                                        rows=tuple(int(x) for x in args.rows.split(":")) if args.rows else None)
     os.makedirs(args.out, exist_ok=True)
     with open(os.path.join(args.out, "summary.json"), "w") as f:
         json.dump(rows, f, indent=1)

@@ -65,7 +65,8 @@ def static_choice(a: KernelHandle, b: KernelHandle, cus: int = 256, times: Optio
     ta, tb = (times if times is not None else (-1.0, -1.0))
     ka = config.KernelInfo(a.name, a.has_barriers, a.grid, a.block, max(a.regs, 1), float(ta))
     kb = config.KernelInfo(b.name, b.has_barriers, b.grid, b.block, max(b.regs, 1), float(tb))
-    return config.choose_fusion(ka, kb, max(a.lds_bytes, 0), max(b.lds_bytes, 0), cus)
+    return config.choose_fusion(ka, kb, max(a.lds_bytes, 0), max(b.lds_bytes, 0), cus,
+                                matrix=(getattr(a, "matrix", False), getattr(b, "matrix", False)))
 
 
 def autotune(op: Operation, candidates: Optional[Sequence[Candidate]] = None, warmup: int = 20, reps: int = 100,

@@ -151,6 +151,7 @@ typedef struct {
     int pattern, p0, p1;     /* bfuse kernels: dispatch pattern */
     int n_sides;             /* 1 for a standalone kernel; fused: how many kernels it runs (3 pointers each, in order) */
     char side_more[BFUSE_MAX_KERNELS - 2][64];   /* fused kernels of more than two: the third, fourth standalone kernel */
+    int matrix_cores;        /* single kernels: 1 if the operator's inner loop is a stream of MFMAs (GEMMs, convolutions) */
 } bfuse_kernel_info;
 
 /* bfuse_kernel_count / bfuse_kernel_at enumerate every kernel except the library's self-test operators
@@ -235,6 +236,11 @@ int bfuse_download_part(int side, size_t offset, void* dst, size_t bytes);
  * (up to collisions) their sums agree -- the comparison the reference makes on the host with check_matrix
  * (operation_cu.py:29-45), for outputs too large to copy back. */
 int bfuse_checksum_output(int side, size_t chunk_bytes, unsigned long long* sums);
+/* Fills tensor 0 (I) or 1 (F) of the side, on the device, with the values bfuse_fill_uniform(seed, n, lo, hi)
+ * writes on the host (fp32 tensors) or their bfuse_f32_to_bf16 roundings (bf16 tensors): the reference's harness
+ * fills host arrays with rand() and copies them (utils_cc.py:28-31); operands of several GB are written where
+ * they are needed instead. */
+int bfuse_fill_uniform_device(int side, int tensor, unsigned long long seed, float lo, float hi);
 
 enum {
     BFUSE_MODE_KERNEL1 = 0,   /* the reference CLI's T = 0..4 (main_cc.py:22-36) */

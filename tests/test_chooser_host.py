@@ -6,6 +6,8 @@ The reference hard-codes pattern and ratio (horizontal-fuser/src/Contexts.cc:64-
 Reg / HasBarriers without using them; here the fused kernel that is measured for each pair must be
 the one the chooser selects.
 """
+import os
+
 import pytest
 
 import bfuse_project_amd as bf
@@ -82,7 +84,7 @@ def test_the_footprint_rule_on_the_48_pairs_of_the_model_operator_matrix(golden_
     log_gain, fused, missed = 0.0, 0, 0
     for p in data["pairs"]:
         (a, la), (b, lb) = ki(p["kernel1"]), ki(p["kernel2"])
-        c = config.choose_fusion(a, b, la, lb)
+        c = config.choose_fusion(a, b, la, lb, matrix=(True, True))    # GEMMs, batched products, convolutions
         assert c["fuse"] in ("bfuse", "none")            # no pair of the matrix has matching grids
         if p["bfuse_speedup"] < 0.98:
             assert c["fuse"] == "none", (p, c)
@@ -126,3 +128,38 @@ def test_the_footprint_rule_on_the_headline_pairs_with_and_without_times():
     c = config.choose_fusion(gate, norm, 135168, 0)
     assert c["fuse"] == "hfuse" and not c["bfuse_pays"]
     assert tuner.static_plan.__defaults__[1] == ("hfuse", "bfuse")      # "none" is an answer only where it is asked for
+
+
+def test_two_kernels_that_each_keep_every_matrix_pipe_busy_are_left_unfused():
+    """The reference's benchmark arrangement (every dense layer, batched product and convolution at batch 1024
+    against every other: bfuse-project_amd/examples/benchmark_batch1024.yaml, 903 pairs): measured on MI355X,
+    block fusion 0.91x, thread-level fusion 0.79x of the two kernels one after the other -- each kernel already
+    has a wave on every SIMD for its whole run.  The rule leaves every such pair unfused, from the registry's
+    metadata alone; a matrix-core kernel that does not cover the chip (196 workgroups of a batch-1 convolution)
+    or a side that is not a matrix-core kernel keeps the decision the footprints give."""
+    import yaml
+    import bfuse_project_amd as bf
+    from bfuse_project_amd import configure, tuner
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    with open(os.path.join(root, "bfuse-project_amd", "examples", "benchmark_batch1024.yaml")) as f:
+        doc = yaml.safe_load(f)
+    registry = {k.name: k for k in bf.list_kernels()}
+    found, missing = configure.resolve(doc, registry)
+    assert not missing
+    s0, s1 = (s["Set"] for s in doc["FusionSet"])
+    n = 0
+    for i, ka in enumerate(s0):
+        for kb in s1[i:]:
+            a, b = found[ka], found[kb]
+            assert a.matrix and b.matrix
+            c = tuner.static_plan(a, b, kinds=("hfuse", "bfuse", "none"), times=(100.0, 100.0))
+            assert c["kind"] == "none" and c["static"]["saturates_matrix_cores"] == (True, True), (a.name, b.name)
+            n += 1
+    assert n == 903
+    # same footprints, but the second side covers 196 of the 256 CUs: the matrix rule does not apply
+    g = config.KernelInfo("g", True, (256, 1, 1), (256, 1, 1), 53, 7.0)
+    conv = config.KernelInfo("c", True, (196, 1, 1), (256, 1, 1), 96, 7.2)
+    assert config.choose_fusion(g, conv, 36864, 40000, matrix=(True, True))["fuse"] == config.choose_fusion(g, conv, 36864, 40000)["fuse"] == "bfuse"
+    big = config.KernelInfo("c", True, (4096, 1, 1), (256, 1, 1), 96, 70.0)
+    assert config.choose_fusion(g, big, 36864, 40000, matrix=(True, True))["fuse"] == "none"
+    assert not bf.kernel_info("layernorm_512x768").matrix and bf.kernel_info("gemm_bf16_512x4096x14336").matrix

@@ -96,3 +96,32 @@ def test_suite_runs_the_built_pairs(modules, tmp_path):
         print(f"[built] {r['kernel1']} + {r['kernel2']}: chooser {r['chooser']['kind']}, {r['chooser_speedup']:.3f}x of the two kernels one after the other; "
               f"block-fused {r['bfuse_speedup']:.3f}x" + (f", thread-fused {r['hfuse_speedup']:.3f}x" if "hfuse_speedup" in r else ""), flush=True)
     perf_report.expect(all(r["chooser_speedup"] >= 0.97 for r in rows), "the chooser's form is not slower than the two kernels one after the other")
+
+
+def test_resident_suite_run_and_device_fill(modules, tmp_path):
+    """The suite's mode for operators of several GB: operands written on the device must be the operands the
+    host fill gives (the same kernel over both gives the same output, bit for bit), and the run -- fused outputs
+    compared with the unfused ones through device-side checksums -- must come out like the host-side one."""
+    from bfuse_project_amd.operation import fill_uniform
+    k1, k2 = "bgemm_f32_1024x208x64x208", "gemm_f32_1024x768x768"
+    with bf.Operation(k1, k2) as op:
+        outs = []
+        for how in ("host", "device"):
+            for side in (0, 1):
+                n = [int(np.prod(op.k[side].shapes[t])) for t in (0, 1)]
+                if how == "host":
+                    op.upload(side, fill_uniform(77 + side, n[0], -0.5, 0.5), fill_uniform(177 + side, n[1], -0.5, 0.5))
+                else:
+                    op.upload(side, np.zeros(n[0], np.float32), np.zeros(n[1], np.float32))
+                    op.fill_uniform_device(side, 0, 77 + side, -0.5, 0.5)
+                    op.fill_uniform_device(side, 1, 177 + side, -0.5, 0.5)
+            op.zero_outputs()
+            op.launch("serial")
+            outs.append((op.download(0), op.download(1)))
+        assert outs[0][0].any() and outs[0][0].tobytes() == outs[1][0].tobytes() and outs[0][1].tobytes() == outs[1][1].tobytes()
+    info = suite.load_info(os.path.join(SUITE, "config", "info.yaml"))
+    rows = suite.run_suite(info, str(tmp_path), validate=True, log=lambda *a: None, resident=True, rows=(1, 2))
+    assert len(rows) == 2 and all("bfuse_ns" in r for r in rows)           # the pairs of the second operator of set 0
+    for r in rows:
+        # two matrix-core kernels that each cover the chip: left unfused
+        assert r["chooser"]["kind"] == "none" and r["chooser_speedup"] == 1.0
