@@ -447,6 +447,8 @@ extern "C" {
 
 const char* bfuse_last_error(void) { return g_err; }
 
+static int load_env_modules();
+
 int bfuse_init(int device)
 {
     int n = 0;
@@ -455,6 +457,7 @@ int bfuse_init(int device)
         return fail(BFUSE_ERR_HIP, "no HIP device available (%s); this library has no CPU path",
                     st == hipSuccess ? "device count is 0" : hipGetErrorString(st));
     if (device < 0 || device >= n) return fail(BFUSE_ERR_ARG, "device %d out of range (0..%d)", device, n - 1);
+    if (int rc = load_env_modules()) return rc;   // a module named in BFUSE_KERNEL_MODULES that does not load is an error here, not a shorter registry
     if (g.inited && device != g.device)
         for (int i = 0; i < kMaxKernels; ++i)
             if (g.side[i].live)

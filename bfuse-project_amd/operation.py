@@ -51,7 +51,10 @@ def kernel_info(name: str) -> KernelHandle:
 def list_kernels() -> List[KernelHandle]:
     l = _lib.lib()
     out = []
-    for i in range(l.bfuse_kernel_count()):
+    n = l.bfuse_kernel_count()
+    if n == 0:      # the library always holds kernels: an empty registry means a module named in the environment did not load
+        raise _lib.BfuseError(-1, l.bfuse_last_error().decode() or "the kernel registry is empty")
+    for i in range(n):
         ci = _lib.KernelInfoC()
         _lib.check(l.bfuse_kernel_at(i, C.byref(ci)))
         out.append(_handle(ci))
