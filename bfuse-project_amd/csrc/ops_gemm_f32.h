@@ -226,11 +226,22 @@ struct GemmF32 {
     __device__ static __forceinline__ void run(int vblock, int tid, Smem& sm, const void* I, const void* F,
                                                void* O, Sync sync)
     {
-        const int batch = BATCH > 1 ? vblock / TILES : 0;
+        // Many products: whole products are dealt to the XCDs (id % 8 is taken as the XCD, as in XcdTiles), so that the
+        // tiles of one product share one L2 and its operands are fetched once -- with 8 x 8 tiles per product a
+        // rectangle per XCD fetches three times as much (measured at 1024 products: 3-7 % on the K = 512 products,
+        // nothing on the others, which are not bound there).  Few products keep the rectangles (every XCD works on each).
+        constexpr bool PRODUCT_PER_XCD = BATCH >= 64 && BATCH % 8 == 0;
+        int batch = BATCH > 1 ? vblock / TILES : 0;
+        if constexpr (PRODUCT_PER_XCD) {
+            const int xcd = vblock & 7, slot = vblock >> 3;
+            batch = (slot / TILES) * 8 + xcd;
+            vblock = slot % TILES;
+        }
         const float* __restrict__ A = static_cast<const float*>(I) + (size_t)batch * M * K;
         const float* __restrict__ B = static_cast<const float*>(F) + (size_t)batch * K * N;
         float* __restrict__ C = static_cast<float*>(O) + (size_t)batch * M * N;
-        const Dims3 vb = XcdTiles<N / BN, M / BM, BM, BN>::tile(BATCH > 1 ? vblock % TILES : vblock);   // tiles dealt so that each XCD's L2 fetches as little as possible
+        const Dims3 vb = PRODUCT_PER_XCD ? Dims3{vblock % (N / BN), vblock / (N / BN), 0}
+                                         : XcdTiles<N / BN, M / BM, BM, BN>::tile(BATCH > 1 ? vblock % TILES : vblock);   // tiles dealt so that each XCD's L2 fetches as little as possible
         const int m0 = vb.y * BM, n0 = vb.x * BN;
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;   // wave-uniform: addresses built on it stay in scalar registers
         const int kbeg = wave * KW;
