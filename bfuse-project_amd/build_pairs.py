@@ -191,7 +191,8 @@ def build(suite: str, forms: str = "both", chunk: int = 256, only: Optional[Sequ
     """Writes <suite>/hip/pairs_*.hip for the suite's pairs that lack a fused kernel and builds the module.
     Returns {"kernels": [...], "files": [...], "module": path or None}."""
     from .operation import list_kernels
-    load_suite_modules(suite)      # what an earlier run built counts as held
+    # the library's own kernels; what an earlier run wrote for this suite is read from its translation units below
+    # (its module is not loaded here: one built against older headers would be refused, and is about to be rebuilt)
     registry = {k.name: k for k in list_kernels()}
     pairs = suite_pairs(suite, triangular)
     if only:
