@@ -44,8 +44,7 @@ def test_dense_layer_against_the_oracle_and_fused_with_layernorm(kid, m, k, n):
 
 @pytest.mark.parametrize("kid,m,k,n", [("dense_4", 512, 4096, 4096), ("dense_7", 512, 14336, 4096)])
 def test_llama_bf16_dense_layer_against_the_oracle_and_fused_with_rmsnorm_rope(kid, m, k, n):
-    """bf16 in, fp32 accumulate, bf16 out, weight [N, K]: a strided 64 x 512 sample of the outputs over
-    the full K against the oracle (1e-2), selector inputs that hit every output element exactly, and the
+    """bf16 in, fp32 accumulate, bf16 out, weight [N, K]: every output against the oracle (1e-2), selector inputs that hit every output element exactly, and the
     kernel block-fused with RMSNorm + RoPE bit-exact against the two kernels launched back to back."""
     from bfuse_project_amd.operation import f32_to_bf16, bf16_to_f32
     from bfuse_project_amd.workloads import PAIRS
@@ -70,11 +69,9 @@ def test_llama_bf16_dense_layer_against_the_oracle_and_fused_with_rmsnorm_rope(k
     assert q1.tobytes() == c.tobytes() and q2.tobytes() == y.tobytes(), "fused output differs from the unfused kernels"
     W = w.reshape(n, k)
     assert np.array_equal(cs.reshape(m, n), W[:, (np.arange(m) * 37) % k].T), "selector inputs: an output element is not the weight it selects"
-    rows, cols = np.arange(3, m, 8), np.arange(5, n, 8)
-    want = orf.gemm_bf16(np.ascontiguousarray(a.reshape(m, k)[rows]), np.ascontiguousarray(W[cols]), b_is_nk=True)
-    got = np.ascontiguousarray(c.reshape(m, n)[np.ix_(rows, cols)])
-    e = oracle_cases.rel_error(bf16_to_f32(got).ravel(), bf16_to_f32(want).ravel())
-    print(f"[parity] {name}: sample {len(rows)} x {len(cols)} over K = {k}: max rel err {e:.3e}; "
+    want = orf.gemm_bf16(a.reshape(m, k), W, b_is_nk=True)          # every output element
+    e = oracle_cases.rel_error(bf16_to_f32(c).ravel(), bf16_to_f32(want).ravel())
+    print(f"[parity] {name}: all {m} x {n} outputs over K = {k}: max rel err {e:.3e}; "
           f"GEMM {t_g:.1f} us = {2.0 * m * n * k / t_g * 1e-6:.0f} TFLOP/s, fused with RMSNorm+RoPE {t_f:.1f} us", flush=True)
     assert e <= 1e-2
 
