@@ -7,13 +7,14 @@ one more instantiation: this module writes, for every pair of `<suite>/config/in
 
     BFUSE_BFUSE_KERNEL(k1, <type of k1>, k2, <type of k2>, _c256, bfuse::kChunked, 256, 1)    block fusion
     BFUSE_HFUSE_KERNEL(k1, <type of k1>, k2, <type of k2>)                                    thread-level fusion
+    BFUSE_BFUSE_RT_KERNEL(k1, <type of k1>, k2, <type of k2>)                                 block fusion, plan at run time (--rt)
 
 into `<suite>/hip/pairs_<n>.hip` -- the operator types exactly as the library spells them
 (bfuse_kernel_op_type) -- and builds `<suite>/hip/libbfuse_pairs.so` with the library's own flags and build
 checks (csrc/Makefile, target `module`).  `<suite>/config/modules.yaml` then names the module; `suite`,
 `quick_start` and `benchmark` (through BFUSE_KERNEL_MODULES) load it and find the new kernels by name.
 
-    python -m bfuse_project_amd.build_pairs SUITE [--forms both|bfuse|hfuse] [--chunk N] [--triangular] [--only K1+K2 ...] [-j J]
+    python -m bfuse_project_amd.build_pairs SUITE [--forms both|bfuse|hfuse] [--rt] [--chunk N] [--triangular] [--only K1+K2 ...] [-j J]
 
 Thread-level fusion is written only where it can work: both workgroups fit one (at most 1024 threads and
 160 KB of LDS together) and at most one side synchronises (config.choose_fusion's rule).
@@ -54,8 +55,10 @@ def hfuse_possible(a, b, lds_a: int, lds_b: int) -> bool:
 
 
 def wanted(pairs: Sequence[Tuple[str, str]], registry: Dict[str, object], forms: str = "both", chunk: int = 256,
-           lds=op_lds) -> List[dict]:
-    """The fused kernels to build: [{k1, k2, form, name}], skipping what the registry already holds."""
+           lds=op_lds, rt: bool = False) -> List[dict]:
+    """The fused kernels to build: [{k1, k2, form, name}], skipping what the registry already holds.
+    `rt`: also the block-fused kernel whose dispatch plan is run-time data (`..._fused_bfuse_rt`), which the tuner
+    times candidate plans and persistent workgroup counts on."""
     out, seen = [], set()
     for k1, k2 in pairs:
         for k in (k1, k2):
@@ -68,6 +71,10 @@ def wanted(pairs: Sequence[Tuple[str, str]], registry: Dict[str, object], forms:
             name = f"{k1}_{k2}_fused_bfuse_c{chunk}"
             if name not in registry:
                 out.append({"k1": k1, "k2": k2, "form": "bfuse", "name": name})
+        if rt:
+            name = f"{k1}_{k2}_fused_bfuse_rt"
+            if name not in registry:
+                out.append({"k1": k1, "k2": k2, "form": "rt", "name": name})
         if forms in ("both", "hfuse") and hfuse_possible(registry[k1], registry[k2], lds(k1), lds(k2)):
             name = f"{k1}_{k2}_fused_hfuse"
             if name not in registry:
@@ -90,6 +97,8 @@ def source_text(kernels: Sequence[dict], chunk: int = 256, types=op_type) -> str
         a, b = sides[k["k1"]], sides[k["k2"]]
         if k["form"] == "bfuse":
             lines.append(f"BFUSE_BFUSE_KERNEL({k['k1']}, {a}, {k['k2']}, {b}, _c{chunk}, bfuse::kChunked, {chunk}, 1)")
+        elif k["form"] == "rt":
+            lines.append(f"BFUSE_BFUSE_RT_KERNEL({k['k1']}, {a}, {k['k2']}, {b})")
         else:
             lines.append(f"BFUSE_HFUSE_KERNEL({k['k1']}, {a}, {k['k2']}, {b})")
     return "\n".join(lines) + "\n"
@@ -113,6 +122,9 @@ def _unit_kernel(line: str) -> Optional[str]:
     if line.startswith("BFUSE_BFUSE_KERNEL("):
         a = [x.strip() for x in line[len("BFUSE_BFUSE_KERNEL("):-1].split(",")]
         return f"{a[0]}_{a[2]}_fused_bfuse{a[4]}"
+    if line.startswith("BFUSE_BFUSE_RT_KERNEL("):
+        a = [x.strip() for x in line[len("BFUSE_BFUSE_RT_KERNEL("):-1].split(",")]
+        return f"{a[0]}_{a[2]}_fused_bfuse_rt"
     if line.startswith("BFUSE_HFUSE_KERNEL("):
         a = [x.strip() for x in line[len("BFUSE_HFUSE_KERNEL("):-1].split(",")]
         return f"{a[0]}_{a[2]}_fused_hfuse"
@@ -187,7 +199,7 @@ def load_suite_modules(suite: str) -> List[str]:
 
 
 def build(suite: str, forms: str = "both", chunk: int = 256, only: Optional[Sequence[str]] = None, per_file: int = 2,
-          jobs: int = 8, compile_: bool = True, triangular: bool = False) -> dict:
+          jobs: int = 8, compile_: bool = True, triangular: bool = False, rt: bool = False) -> dict:
     """Writes <suite>/hip/pairs_*.hip for the suite's pairs that lack a fused kernel and builds the module.
     Returns {"kernels": [...], "files": [...], "module": path or None}."""
     from .operation import list_kernels
@@ -203,7 +215,7 @@ def build(suite: str, forms: str = "both", chunk: int = 256, only: Optional[Sequ
         pairs = [p for p in pairs if p in keep]
     hip = os.path.join(suite, "hip")
     have = set(written(hip))       # units of an earlier, possibly interrupted, run are not written twice
-    todo = [k for k in wanted(pairs, registry, forms, chunk) if k["name"] not in have]
+    todo = [k for k in wanted(pairs, registry, forms, chunk, rt=rt) if k["name"] not in have]
     os.makedirs(hip, exist_ok=True)
     first = len([f for f in os.listdir(hip) if f.startswith("pairs_") and f.endswith(".hip")])
     files = []
@@ -242,12 +254,13 @@ def main(argv=None) -> int:
     ap.add_argument("--chunk", type=int, default=256, help="workgroups of one side per chunk of the block-fused dispatch (one round over the CUs)")
     ap.add_argument("--only", nargs="*", metavar="K1+K2", help="registry names of the pairs to build (default: every pair of the suite)")
     ap.add_argument("--triangular", action="store_true", help="only the pairs (i, j >= i) of two sets that list the same operators, as the reference profiles them")
+    ap.add_argument("--rt", action="store_true", help="also the block-fused kernel with its dispatch plan as run-time data (for tuner.autotune and persistent workgroups)")
     ap.add_argument("--per-file", type=int, default=2, help="fused kernels per translation unit")
     ap.add_argument("-j", type=int, default=8, dest="jobs")
     ap.add_argument("--write-only", action="store_true", help="write the .hip files, do not compile")
     args = ap.parse_args(argv)
     try:
-        r = build(args.suite, args.forms, args.chunk, args.only, args.per_file, args.jobs, not args.write_only, args.triangular)
+        r = build(args.suite, args.forms, args.chunk, args.only, args.per_file, args.jobs, not args.write_only, args.triangular, args.rt)
     except (LookupError, RuntimeError, OSError) as e:
         print(f"build_pairs: {e}", file=sys.stderr)
         return 1

@@ -28,6 +28,7 @@ def test_wanted_skips_what_the_registry_holds_and_writes_thread_fusion_only_wher
                      "a_d_fused_bfuse_c256",                              # 256 + 896 threads do not fit one workgroup
                      "c_b_fused_bfuse_c256", "c_b_fused_hfuse"]
     assert [k["name"] for k in build_pairs.wanted([("c", "b")], reg, "bfuse", 128, lds)] == ["c_b_fused_bfuse_c128"]
+    assert [k["name"] for k in build_pairs.wanted([("c", "b")], reg, "bfuse", 256, lds, rt=True)] == ["c_b_fused_bfuse_c256", "c_b_fused_bfuse_rt"]
     # LDS: 100000 + 70000 bytes exceed a workgroup's 160 KB
     reg["e"] = _k("e", 64, False)
     assert [k["form"] for k in build_pairs.wanted([("c", "e")], reg, "both", 256, {"c": 100000, "e": 70000}.__getitem__)] == ["bfuse"]
@@ -40,13 +41,16 @@ def test_wanted_skips_what_the_registry_holds_and_writes_thread_fusion_only_wher
 def test_source_text_names_each_side_once_by_the_type_the_library_gives():
     todo = [{"k1": "a", "k2": "b", "form": "bfuse", "name": "a_b_fused_bfuse_c256"},
             {"k1": "a", "k2": "b", "form": "hfuse", "name": "a_b_fused_hfuse"},
-            {"k1": "c", "k2": "b", "form": "bfuse", "name": "c_b_fused_bfuse_c256"}]
+            {"k1": "c", "k2": "b", "form": "bfuse", "name": "c_b_fused_bfuse_c256"},
+            {"k1": "c", "k2": "b", "form": "rt", "name": "c_b_fused_bfuse_rt"}]
     text = build_pairs.source_text(todo, 256, {"a": "bfuse::A<1, 2>", "b": "bfuse::B<true>", "c": "bfuse::C<3>"}.__getitem__)
     lines = text.splitlines()
     assert lines.count("using Side0 = bfuse::A<1, 2>;   // a") == 1 and "using Side1 = bfuse::B<true>;   // b" in lines
     assert "BFUSE_BFUSE_KERNEL(a, Side0, b, Side1, _c256, bfuse::kChunked, 256, 1)" in lines
     assert "BFUSE_HFUSE_KERNEL(a, Side0, b, Side1)" in lines
     assert "BFUSE_BFUSE_KERNEL(c, Side2, b, Side1, _c256, bfuse::kChunked, 256, 1)" in lines
+    assert "BFUSE_BFUSE_RT_KERNEL(c, Side2, b, Side1)" in lines
+    assert [build_pairs._unit_kernel(l) for l in lines if l.startswith("BFUSE_")][-4:] == [k["name"] for k in todo]
     assert "BFUSE_MODULE_PROLOGUE()" in lines and '#include "fuse.h"' in lines
     for h in build_pairs.HEADERS:
         assert os.path.exists(os.path.join(build_pairs.CSRC, h))

@@ -125,3 +125,33 @@ def test_resident_suite_run_and_device_fill(modules, tmp_path):
     for r in rows:
         # two matrix-core kernels that each cover the chip: left unfused
         assert r["chooser"]["kind"] == "none" and r["chooser_speedup"] == 1.0
+
+
+def test_tuner_times_plans_on_a_built_run_time_plan_kernel(modules):
+    """build_pairs --rt: the pair's block-fused kernel with its dispatch plan as run-time data.  Every candidate
+    plan and persistent workgroup count must leave both outputs what the unfused kernels write (checksums of
+    all 1024 items), and the tuner ranks them."""
+    from bfuse_project_amd import patterns, tuner
+    k1, k2 = "conv1x1s1p0_f32_1024x1280x8x8_192", "bgemm_f32_1024x208x64x208"
+    with bf.Operation(k1, k2) as op:
+        for side in (0, 1):
+            op.fill_uniform_device(side, 0, 31 + side, -0.5, 0.5)
+            op.fill_uniform_device(side, 1, 41 + side, -0.5, 0.5)
+        op.zero_outputs()
+        op.launch("serial")
+        want = [op.checksum_output(s, int(np.prod(op.k[s].shapes[2])) // 1024) for s in (0, 1)]
+        rt = op.fused_rt()
+        dims = [patterns.LaunchDims(tuple(k.grid), tuple(k.block)) for k in op.k]
+        cands = [tuner.Candidate("ranges", "ranges"), tuner.Candidate("chunk 256", "chunked", 256), tuner.Candidate("zigzag 1:1", "zigzag", 1, 1),
+                 tuner.Candidate("chunk 256, 1024 persistent workgroups", "chunked", 256, 1, 1024)]
+        for c in cands:
+            h = op.set_plan(rt, patterns.plan_blocks(c.pattern, dims, c.p0, c.p1), c.workgroups)
+            op.zero_outputs()
+            op.launch("bfuse", h)
+            for s in (0, 1):
+                got = op.checksum_output(s, int(np.prod(op.k[s].shapes[2])) // 1024)
+                assert np.array_equal(got, want[s]), f"{c.label}: side {s} differs from the unfused kernel"
+        rows = tuner.autotune(op, cands, warmup=2, reps=5)
+        for r in rows:
+            print(f"[built] {k1} + {k2}: {r['label']:42s} {r['us_mean']:.0f} us", flush=True)
+        assert len(rows) == len(cands) and rows[0]["us_mean"] <= rows[-1]["us_mean"]
