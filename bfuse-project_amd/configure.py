@@ -138,7 +138,7 @@ def instantiation_hint(kernel_id: str, args) -> str:
     if op == "conv2d":
         n, h, w, co, ci, kh, kw, stride, pad = args
         if ci % 16 != 0 and ci > 4:
-            return "the library's convolutions take input channels in groups of 16, or at most 4 (csrc/ops_conv_general.h)"
+            return "the library's convolutions take input channels in groups of 16, or at most 4 (csrc/ops_conv_general.h, ops_conv_rect.h)"
         batch = f"{n}x" if n != 1 else ""
         return (f"using Conv = ConvF32Auto<{ci}, {co}, {h}, {w}, {kh}, {kw}, {stride}, {pad}, {n}>;  "
                 f"BFUSE_KERNEL(conv{kh}x{kw}s{stride}p{pad}_f32_{batch}{ci}x{h}x{w}_{co}, Conv, ...)  in csrc/kernels_*.hip")

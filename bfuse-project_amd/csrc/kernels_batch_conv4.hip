@@ -1,8 +1,8 @@
 // Batch-1024 convolutions of the reference's example configurations (test-utils/examples/benchmark.yaml,
-// inception_v3.yaml; argument lists N, H, W, CO, CI, KH, KW, stride, padding) on the general convolution with the
-// library's default tiling.  Names: conv<KH>x<KW>s<stride>p<padding>_f32_<N>x<CI>x<H>x<W>_<CO>.  Part 4 of 4.
+// inception_v3.yaml; argument lists N, H, W, CO, CI, KH, KW, stride, padding) on the general convolutions (64 consecutive pixels or a
+// 4 x 16 rectangle per workgroup) with the library's default tiling.  Names: conv<KH>x<KW>s<stride>p<padding>_f32_<N>x<CI>x<H>x<W>_<CO>.  Part 4 of 4.
 #include "fuse.h"
-#include "ops_conv_general.h"
+#include "ops_conv_rect.h"
 
 using namespace bfuse;
 

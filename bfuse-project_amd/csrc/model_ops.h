@@ -4,6 +4,7 @@
 #pragma once
 #include "ops_conv.h"
 #include "ops_conv_general.h"
+#include "ops_conv_rect.h"
 #include "ops_gemm_bf16.h"
 #include "ops_gemm_f32.h"
 #include "ops_gemm_f32_dma.h"
@@ -74,7 +75,7 @@ using Bgemm17 = GemmF32<1024, 64, 512, 16, 64, 4, kEpiNone, 2, 1, true, 1>;     
 
 // The other ResNet-18 layers (test-utils/examples/resnet-18.yaml) on the general convolution:
 // <CI, CO, H, W, KH, KW, stride, padding, output channels per workgroup, 16-pixel blocks, waves>
-using Conv0 = ConvF32Lds<3, 64, 224, 224, 7, 7, 2, 3, 16, 4, 1>;          // 7x7 stride 2 on RGB: 196 x 4 = 784 one-wave workgroups
+using Conv0 = ConvF32Rect<3, 64, 224, 224, 7, 7, 2, 3, 16, 4, 1>;         // 7x7 stride 2 on RGB: 4 x 16-pixel rectangles (13 x 37 patch instead of 9 x 230), 196 x 4 = 784 one-wave workgroups
 using Conv2 = SwapOperands<GemmF32<64, 3136, 64, 16, 64, 1>>;            // 1x1 stride 1 = Wt[64,64] . X[64,3136]: 4 x 49 = 196
 using Conv3 = ConvF32Lds<64, 128, 56, 56, 3, 3, 2, 1, 32, 1, 4>;          // 49 x 4 = 196 workgroups
 using Conv5 = ConvF32Lds<64, 128, 56, 56, 1, 1, 2, 0, 32, 1, 4>;

@@ -337,40 +337,6 @@ struct ConvF32Lds {
     }
 };
 
-// The tiling the library gives a convolution it has no hand-picked one for: as many output channels per
-// workgroup as keep the filter fragments of a wave within ~72 registers (the staged patch is shared by all
-// of them), 64 pixels (or the whole image when it has fewer), and as many waves over the channel groups as
-// leave room for two workgroups' patches in a CU's LDS.
-template <int CI, int CO, int H, int W, int KH, int KW, int S, int P, int NIMG>
-struct ConvTiling {
-    static constexpr int T = KH * KW;
-    static constexpr int OHW = ((H - KH + 2 * P) / S + 1) * ((W - KW + 2 * P) / S + 1);
-    static constexpr int pick_bm()
-    {
-        if (CI < 16) return 16;
-        if (T == 1)      // a 1x1 filter is one register per row block: as many output channels as divide CO, up to 80
-            for (int bm = 80; bm > 16; bm -= 16)     // (96 measured slower than 64 on the 8x8 and 17x17 layers)
-                if (CO % bm == 0) return bm;
-        if (CO % 64 == 0 && 4 * T <= 18) return 64;
-        if (CO % 48 == 0 && 3 * T <= 18) return 48;
-        if (CO % 32 == 0 && 2 * T <= 18) return 32;
-        return 16;
-    }
-    static constexpr int BM = pick_bm();
-    static constexpr int PB = OHW >= 64 ? 4 : (OHW + 15) / 16;
-    static constexpr int NGROUP = CI >= 16 ? CI / 16 : 1;
-    static constexpr int TILE = ConvF32Lds<CI, CO, H, W, KH, KW, S, P, BM, PB, 1, NIMG>::TILE_BYTES;
-    static constexpr int pick_ks()
-    {
-        if (NGROUP % 4 == 0 && 4 * TILE <= 80 * 1024) return 4;
-        if (NGROUP % 2 == 0 && 2 * TILE <= 80 * 1024) return 2;
-        return 1;
-    }
-    using type = ConvF32Lds<CI, CO, H, W, KH, KW, S, P, BM, PB, pick_ks(), NIMG>;
-};
-template <int CI, int CO, int H, int W, int KH, int KW, int S, int P, int NIMG = 1>
-using ConvF32Auto = typename ConvTiling<CI, CO, H, W, KH, KW, S, P, NIMG>::type;
-
 // An operator with its first two operands exchanged: a 1x1 / stride 1 convolution is the product
 // Wt[CO, CI] . X[CI, H*W], i.e. a GEMM whose first operand is the convolution's SECOND (the weights).
 template <class Op>
