@@ -144,6 +144,29 @@ def written(hip_dir: str) -> List[str]:
     return out
 
 
+def stale_units(hip_dir: str, types=None) -> List[str]:
+    """Translation units that name a side by another type than the library gives that kernel now (the library was
+    rebuilt with another tiling of the operator since they were written)."""
+    types = types or op_type
+    out = []
+    if os.path.isdir(hip_dir):
+        for f in sorted(os.listdir(hip_dir)):
+            if f.startswith("pairs_") and f.endswith(".hip"):
+                with open(os.path.join(hip_dir, f)) as fh:
+                    for line in fh:
+                        if line.startswith("using Side") and ";   // " in line:
+                            typ = line.split(" = ", 1)[1].split(";   // ")[0]
+                            name = line.rsplit("// ", 1)[1].strip()
+                            try:
+                                if types(name) != typ:
+                                    out.append(f)
+                                    break
+                            except LookupError:
+                                out.append(f)
+                                break
+    return out
+
+
 def drop_spilling(hip_dir: str) -> List[str]:
     """Removes, from every pairs_*.hip whose last compilation reported spills, the kernels that spilled."""
     dropped = []
@@ -214,6 +237,11 @@ def build(suite: str, forms: str = "both", chunk: int = 256, only: Optional[Sequ
             raise LookupError(f"not pairs of this suite: {sorted(unknown)}")
         pairs = [p for p in pairs if p in keep]
     hip = os.path.join(suite, "hip")
+    if stale_units(hip):
+        # the library's operators changed under the suite's units: everything written for it is written again
+        for f in os.listdir(hip):
+            if f.startswith("pairs_") or f == "libbfuse_pairs.so":
+                os.remove(os.path.join(hip, f))
     have = set(written(hip))       # units of an earlier, possibly interrupted, run are not written twice
     todo = [k for k in wanted(pairs, registry, forms, chunk, rt=rt) if k["name"] not in have]
     os.makedirs(hip, exist_ok=True)

@@ -87,3 +87,16 @@ def test_sample_suite_lists_six_kernels_to_build(tmp_path):
     with open(out / "config" / "modules.yaml", "w") as f:
         yaml.safe_dump(["hip/libbfuse_pairs.so"], f)
     assert build_pairs.module_paths(str(out)) == [os.path.join(str(out), "hip", "libbfuse_pairs.so")]
+
+
+def test_units_written_for_another_tiling_of_an_operator_are_found(tmp_path):
+    """A suite's translation units name each side by the operator type the library gave it when they were written;
+    after a rebuild of the library with another tiling they are stale and must be written again."""
+    d = tmp_path / "hip"
+    d.mkdir()
+    (d / "pairs_0.hip").write_text("using Side0 = bfuse::A<1>;   // a\nusing Side1 = bfuse::B<2>;   // b\nBFUSE_HFUSE_KERNEL(a, Side0, b, Side1)\n")
+    (d / "pairs_1.hip").write_text("using Side0 = bfuse::A<1>;   // a\nBFUSE_HFUSE_KERNEL(a, Side0, a, Side0)\n")
+    now = {"a": "bfuse::A<1>", "b": "bfuse::B<3>"}.__getitem__
+    assert build_pairs.stale_units(str(d), now) == ["pairs_0.hip"]
+    assert build_pairs.stale_units(str(d), {"a": "bfuse::A<1>", "b": "bfuse::B<2>"}.__getitem__) == []
+    assert build_pairs.stale_units(str(tmp_path / "none")) == []
