@@ -26,8 +26,9 @@
 // loads (one image) or from aligned 16-byte loads over the contiguous span of rows (a batch).  A last pixel block that runs past the image (14x14 and 7x7 outputs are not multiples of 16
 // pixels) computes on the last pixel again and is not stored.
 //
-// A batch of NIMG images is NIMG times the workgroups of one image, image after image: every image is tiled
-// alike, so what holds for one (placement of the tiles over the XCDs, the staged patch) holds for all.
+// A batch of NIMG images is NIMG times the workgroups of one image; every image is tiled alike.  The pixel tiles
+// of the whole batch, image after image, are what is dealt over the XCDs (tile_of): each XCD owns consecutive
+// tiles and every channel tile of each.
 #pragma once
 #include <hip/hip_runtime.h>
 
@@ -88,7 +89,11 @@ struct ConvF32Lds {
     // (as in Conv3x3F32Lds).
     __device__ static __forceinline__ void tile_of(int vblock, int& pt, int& ct)
     {
-        constexpr int PER_XCD = NPT / 8;
+        // over the pixel tiles of the WHOLE batch (image-major): with few tiles per image (an 8 x 8 image is one)
+        // the channel tiles of one image would otherwise be consecutive ids, one per XCD, and each XCD would
+        // fetch the image for itself (measured on the 1 x 1 layers of 8 x 8 images: 7.8 times the operands)
+        constexpr int NPTB = NPT * NIMG;
+        constexpr int PER_XCD = NPTB / 8;
         constexpr int FULL = 8 * PER_XCD * NCT;
         if (vblock < FULL) {
             const int xcd = vblock & 7, slot = vblock >> 3;
@@ -120,14 +125,14 @@ struct ConvF32Lds {
         const float* __restrict__ X = static_cast<const float*>(I);
         const float* __restrict__ Wt = static_cast<const float*>(F);
         float* __restrict__ Y = static_cast<float*>(O);
+        int pt, ct;
+        tile_of(vblock, pt, ct);
         if constexpr (NIMG > 1) {
-            const int img = vblock / WG_PER_IMAGE;
-            vblock -= img * WG_PER_IMAGE;
+            const int img = pt / NPT;
+            pt -= img * NPT;
             X += (size_t)img * CI * HW;
             Y += (size_t)img * CO * OHW;
         }
-        int pt, ct;
-        tile_of(vblock, pt, ct);
         const int p0 = pt * TP, co0 = ct * BM;
         const int oy_lo = p0 / OW;                     // first output row of the tile
         const int iy_lo = oy_lo * S - P;               // image row of staged row 0

@@ -75,7 +75,11 @@ struct ConvF32Rect {
     // pixel tiles and every channel tile of each, so that the workgroups sharing a patch use one L2.
     __device__ static __forceinline__ void tile_of(int vblock, int& pt, int& ct)
     {
-        constexpr int PER_XCD = NPT / 8;
+        // over the pixel tiles of the WHOLE batch (image-major): with few tiles per image (an 8 x 8 image is one)
+        // the channel tiles of one image would otherwise be consecutive ids, one per XCD, and each XCD would
+        // fetch the image for itself (measured on the 1 x 1 layers of 8 x 8 images: 7.8 times the operands)
+        constexpr int NPTB = NPT * NIMG;
+        constexpr int PER_XCD = NPTB / 8;
         constexpr int FULL = 8 * PER_XCD * NCT;
         if (vblock < FULL) {
             const int xcd = vblock & 7, slot = vblock >> 3;
@@ -107,14 +111,14 @@ struct ConvF32Rect {
         const float* __restrict__ X = static_cast<const float*>(I);
         const float* __restrict__ Wt = static_cast<const float*>(F);
         float* __restrict__ Y = static_cast<float*>(O);
+        int pt, ct;
+        tile_of(vblock, pt, ct);
         if constexpr (NIMG > 1) {
-            const int img = vblock / WG_PER_IMAGE;
-            vblock -= img * WG_PER_IMAGE;
+            const int img = pt / NPT;
+            pt -= img * NPT;
             X += (size_t)img * CI * HW;
             Y += (size_t)img * CO * OHW;
         }
-        int pt, ct;
-        tile_of(vblock, pt, ct);
         const int co0 = ct * BM;
         const int oy0 = (pt / NTX) * TH, ox0 = (pt % NTX) * 16;   // first output row / column of the tile
         const int iy0 = oy0 * S - P, ix0 = ox0 * S - P;           // image row / column of patch position (0, 0)
