@@ -1,7 +1,7 @@
 // benchmark -- command-line driver over libbfuse_rt, the counterpart of the reference's
 // generated main.cc (test-utils/test-suite-files/main_cc.py:22-36,139-299):
 //
-//     benchmark [-vhd] [-n num_iterations] [-s seed] [-x suffix] [-i info.yaml] T K1 K2
+//     benchmark [-vhdr] [-n num_iterations] [-s seed] [-x suffix] [-i info.yaml] T K1 K2
 //
 //      T : type of operation: 0 kernel1, 1 kernel2, 2 parallel (two streams), 3 hfuse, 4 bfuse,
 //          5 serial (kernel1 then kernel2 on one stream; not in the reference)
@@ -16,6 +16,10 @@
 //          must be bit-identical to the unfused ones; check_matrix (eps 1e-3) is reported too.
 //          Exit status 1 on mismatch (main_cc.py:288-292).
 //     -d : dry run: print the kernels T K1 K2 resolve to and exit (needs no device).
+//     -r : resident: for operators whose operands and results run to GB (the reference's benchmark.yaml is batch
+//          1024) -- the same uniform operands are written on the device instead of being filled on the host and
+//          copied, the variant is launched over them, and -v compares the variant's outputs with the unfused
+//          kernels' through checksums computed on the device (up to 1024 chunks per output) instead of copies.
 //     -x : variant suffix of a bfuse kernel (e.g. _c256); default is the plain name, or the
 //          only fused kernel of that kind the library holds for the pair.
 //
@@ -40,11 +44,12 @@ static unsigned long long seed = 0xB5F05E;
 static std::string suffix;
 static std::string info_path;
 static bool dry_run = false;
+static bool resident = false;
 static const char* operation_type_string[] = {"kernel1", "kernel2", "parallel", "hfuse", "bfuse", "serial"};
 
 static void print_help(const char* prog)
 {
-    printf("Usage: %s [-vhd] [-n num_iterations] [-s seed] [-x suffix] [-i info.yaml] T K1 K2\n", prog);
+    printf("Usage: %s [-vhdr] [-n num_iterations] [-s seed] [-x suffix] [-i info.yaml] T K1 K2\n", prog);
     printf("Options:\n");
     printf("     -v : validate test.                (default: off)\n");
     printf("     -h : print this page.\n");
@@ -53,6 +58,7 @@ static void print_help(const char* prog)
     printf("     -x : suffix of the bfuse variant.   (default: none)\n");
     printf("     -i : info.yaml of the suite.        (default: ./config/info.yaml if present)\n");
     printf("     -d : only print the kernels the command resolves to (no device needed).\n");
+    printf("     -r : operands written and outputs compared on the device (operators of several GB).\n");
     printf("      T : type of operation (0 kernel1, 1 kernel2, 2 parallel, 3 hfuse, 4 bfuse, 5 serial).\n");
     printf("     K1 : idx (position in the first FusionSet of info.yaml) or name of kernel1.\n");
     printf("     K2 : idx (position in the second FusionSet of info.yaml) or name of kernel2.\n");
@@ -215,11 +221,35 @@ static void setup(HostSide& h, const std::string& name, int side)
         fprintf(stderr, "%s is a fused kernel; K%d must name a standalone kernel\n", name.c_str(), side);
         exit(EXIT_FAILURE);
     }
+    CHECK(bfuse_set_elem_bytes(side, h.ki.elem_bytes[0], h.ki.elem_bytes[1], h.ki.elem_bytes[2]));
+    if (resident) return;   // nothing on the host
     fill(h.I, h.ki.shape[0], h.ki.elem_bytes[0], seed * 16 + 4 * side);
     fill(h.F, h.ki.shape[1], h.ki.elem_bytes[1], seed * 16 + 4 * side + 1);
     h.O.assign(nelem(h.ki.shape[2]) * h.ki.elem_bytes[2], 0);
     h.O_ans = h.O;
-    CHECK(bfuse_set_elem_bytes(side, h.ki.elem_bytes[0], h.ki.elem_bytes[1], h.ki.elem_bytes[2]));
+}
+
+// resident mode: the operands fill() would give, written in HBM (fp32 and bf16 tensors)
+static void fill_on_device(const HostSide& h, int side)
+{
+    for (int t = 0; t < 2; ++t) {
+        if (h.ki.elem_bytes[t] != 4 && h.ki.elem_bytes[t] != 2) {
+            fprintf(stderr, "%s: -r writes fp32 and bf16 operands; this kernel takes a byte operand\n", h.ki.name);
+            exit(EXIT_FAILURE);
+        }
+        CHECK(bfuse_fill_uniform_device(side, t, seed * 16 + 4 * side + t, -0.5f, 0.5f));
+    }
+}
+
+// resident mode: checksums of a side's output, cut into as many chunks (up to 1024) as divide it
+static std::vector<unsigned long long> output_sums(const HostSide& h, int side)
+{
+    const size_t bytes = nelem(h.ki.shape[2]) * (size_t)h.ki.elem_bytes[2];
+    size_t chunks = 1024;
+    while (chunks > 1 && (bytes % chunks != 0 || (bytes / chunks) % 4 != 0)) chunks /= 2;
+    std::vector<unsigned long long> sums(2 * chunks);
+    CHECK(bfuse_checksum_output(side, bytes / chunks, sums.data()));
+    return sums;
 }
 
 static bool compare(const HostSide& h, const char* what)
@@ -247,7 +277,7 @@ static void stats(const char* label, const std::vector<float>& v)
 int main(int argc, char** argv)
 {
     int c;
-    while ((c = getopt(argc, argv, "vhdn:s:x:i:")) != -1) {
+    while ((c = getopt(argc, argv, "vhdrn:s:x:i:")) != -1) {
         switch (c) {
             case 'v': validation = true; break;
             case 'n': {
@@ -264,6 +294,7 @@ int main(int argc, char** argv)
             case 'x': suffix = optarg; break;
             case 'i': info_path = optarg; break;
             case 'd': dry_run = true; break;
+            case 'r': resident = true; break;
             case 'h':
             default: print_help(argv[0]); exit(0);
         }
@@ -310,6 +341,34 @@ int main(int argc, char** argv)
            operation_type_string[T], k1.c_str(), k2.c_str());
     if (fused.func) printf("- Fused kernel: %s  grid %u block %u regs %d lds %d\n", fused.name, fused.grid[0], fused.block[0], fused.regs, fused.lds_bytes);
 
+    const void* fa = T == 1 ? b.ki.func : (T >= 3 && T <= 4 ? fused.func : a.ki.func);
+    const unsigned* ga = T == 1 ? b.ki.grid : (T >= 3 && T <= 4 ? fused.grid : a.ki.grid);
+    const unsigned* ba = T == 1 ? b.ki.block : (T >= 3 && T <= 4 ? fused.block : a.ki.block);
+    bool is_valid = true;
+    if (resident) {
+        fill_on_device(a, 1);
+        fill_on_device(b, 2);
+        CHECK(bfuse_zero_output(1));
+        CHECK(bfuse_zero_output(2));
+        CHECK(bfuse_launch((int)T, fa, ga, ba, b.ki.func, b.ki.grid, b.ki.block));
+        if (validation) {
+            const std::vector<unsigned long long> got1 = output_sums(a, 1), got2 = output_sums(b, 2);
+            CHECK(bfuse_zero_output(1));
+            CHECK(bfuse_zero_output(2));
+            if (T != BFUSE_MODE_KERNEL2) {
+                CHECK(bfuse_launch(BFUSE_MODE_KERNEL1, a.ki.func, a.ki.grid, a.ki.block, nullptr, nullptr, nullptr));
+                const bool same = output_sums(a, 1) == got1;
+                printf("Validation kernel1: %s (checksums of %zu chunks)\n", same ? "VALID" : "INVALID", got1.size() / 2);
+                is_valid &= same;
+            }
+            if (T != BFUSE_MODE_KERNEL1) {
+                CHECK(bfuse_launch(BFUSE_MODE_KERNEL2, b.ki.func, b.ki.grid, b.ki.block, nullptr, nullptr, nullptr));
+                const bool same = output_sums(b, 2) == got2;
+                printf("Validation kernel2: %s (checksums of %zu chunks)\n", same ? "VALID" : "INVALID", got2.size() / 2);
+                is_valid &= same;
+            }
+        }
+    } else {
     // one run through the reference's copy-in / launch / copy-out entry points
     switch (T) {
         case BFUSE_MODE_KERNEL1:
@@ -343,7 +402,6 @@ int main(int argc, char** argv)
                            (bfuse_kernel6_fn)fused.func, fused.grid, fused.block, 0, 0));
     }
 
-    bool is_valid = true;
     if (validation) {
         if (T != BFUSE_MODE_KERNEL2) {
             CHECK(run_kernel1(a.I.data(), a.F.data(), a.O_ans.data(), a.ki.shape[0], a.ki.shape[1], a.ki.shape[2],
@@ -356,11 +414,9 @@ int main(int argc, char** argv)
             is_valid &= compare(b, "kernel2");
         }
     }
+    }
 
     // GPU-side durations over device-resident operands
-    const void* fa = T == 1 ? b.ki.func : (T >= 3 && T <= 4 ? fused.func : a.ki.func);
-    const unsigned* ga = T == 1 ? b.ki.grid : (T >= 3 && T <= 4 ? fused.grid : a.ki.grid);
-    const unsigned* ba = T == 1 ? b.ki.block : (T >= 3 && T <= 4 ? fused.block : a.ki.block);
     std::vector<float> tot(num_iterations), ta(num_iterations), tb(num_iterations);
     CHECK(bfuse_time((int)T, fa, ga, ba, b.ki.func, b.ki.grid, b.ki.block, 3, (int)num_iterations, tot.data(), ta.data(), tb.data()));
     stats(operation_type_string[T], tot);

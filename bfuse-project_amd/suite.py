@@ -89,11 +89,13 @@ def bfuse_suffix(k1: str, k2: str) -> List[str]:
     return ["-x", pick.name[len(stem):]]
 
 
-def valid_commands(info: dict, benchmark_path: str, triangular: bool = False, info_path: Optional[str] = None) -> List[List[str]]:
-    """`benchmark -v T K1 K2` for every method and pair (profile_test_suite.py:13-47)."""
+def valid_commands(info: dict, benchmark_path: str, triangular: bool = False, info_path: Optional[str] = None,
+                   resident: bool = False) -> List[List[str]]:
+    """`benchmark -v T K1 K2` for every method and pair (profile_test_suite.py:13-47); `resident`: with the driver's
+    -r (operands written and outputs compared on the device, for operators of several GB)."""
     a, b = set_names(info)
     opts, k1, k2 = _ids(info, info_path)
-    common = [os.path.abspath(benchmark_path), "-v"] + opts
+    common = [os.path.abspath(benchmark_path), "-v"] + (["-r"] if resident else []) + opts
     out = []
     for idx, _ in enumerate(METHODS):
         if idx == 0:
@@ -105,7 +107,8 @@ def valid_commands(info: dict, benchmark_path: str, triangular: bool = False, in
     return out
 
 
-def exec_commands(info: dict, benchmark_path: str, exec_path: str, triangular: bool = False, info_path: Optional[str] = None) -> List[List[str]]:
+def exec_commands(info: dict, benchmark_path: str, exec_path: str, triangular: bool = False, info_path: Optional[str] = None,
+                  resident: bool = False) -> List[List[str]]:
     """One rocprofv3 kernel-trace run per (method, k1, k2); the trace lands in
     `<exec_path>/<method index>_<i>_<j>_kernel_trace.csv` (the reference's file naming with the
     profiler's suffix)."""
@@ -116,7 +119,7 @@ def exec_commands(info: dict, benchmark_path: str, exec_path: str, triangular: b
 
     def one(idx, i, j):
         return ["rocprofv3", "--kernel-trace", "--output-format", "csv", "-d", exec_path, "-o", f"{idx}_{i}_{j}", "--",
-                bench, "-n", n] + opts + (bfuse_suffix(a[i], b[j]) if idx == 4 else []) + [str(idx), k1(i), k2(j)]
+                bench, "-n", n] + (["-r"] if resident else []) + opts + (bfuse_suffix(a[i], b[j]) if idx == 4 else []) + [str(idx), k1(i), k2(j)]
     out = []
     for idx, _ in enumerate(METHODS):
         if idx == 0:
@@ -482,7 +485,7 @@ def main(argv=None) -> int:
         return 1
     if args.commands:
         prefix = f"BFUSE_KERNEL_MODULES={':'.join(modules)} " if modules else ""
-        for c in exec_commands(info, args.benchmark, exec_dir, args.triangular, args.file):
+        for c in exec_commands(info, args.benchmark, exec_dir, args.triangular, args.file, resident=args.resident):
             print(prefix + " ".join(c))
         return 0
     rows = analyze(info, exec_dir, args.triangular) if args.analyze else run_suite(info, args.out, not args.no_validate, args.triangular, resident=args.resident,

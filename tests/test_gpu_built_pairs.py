@@ -80,6 +80,12 @@ def test_driver_finds_the_module_through_the_environment(modules):
     r = subprocess.run([BENCH, "-v", "-n", "1", "-i", info_path, "-x", "_c256", "4", "1", "0"], env=env, capture_output=True, text=True, timeout=300)
     print(r.stdout[-600:], r.stderr[-600:], flush=True)
     assert r.returncode == 0, r.stderr
+    # the same through the driver's resident mode: operands written and outputs compared on the device
+    r = subprocess.run([BENCH, "-v", "-r", "-n", "3", "-i", info_path, "-x", "_c256", "4", "1", "0"], env=env, capture_output=True, text=True, timeout=300)
+    print(r.stdout[-600:], r.stderr[-600:], flush=True)
+    assert r.returncode == 0 and r.stdout.count("VALID (checksums") == 2 and "INVALID" not in r.stdout, r.stdout + r.stderr
+    r = subprocess.run([BENCH, "-v", "-r", "-n", "3", "-i", info_path, "3", "1", "0"], env=env, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and "INVALID" not in r.stdout, r.stdout + r.stderr          # thread-level fusion of the same pair
     # without the module the same command has no fused kernel to run
     r = subprocess.run([BENCH, "-d", "-i", info_path, "-x", "_c256", "4", "1", "0"], env={k: v for k, v in os.environ.items() if k != "BFUSE_KERNEL_MODULES"},
                        capture_output=True, text=True, timeout=60)

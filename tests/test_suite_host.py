@@ -49,6 +49,10 @@ def test_command_matrix_follows_the_reference(info):
     assert last[-3:] == ["4", "a2", "b3"] and last[last.index("-o") + 1] == "4_2_3"
     v = suite.valid_commands(info, "/x/benchmark")
     assert all(x[1] == "-v" for x in v) and len(v) == len(full)
+    # operators of several GB: the driver's resident mode in every command
+    r = suite.exec_commands(info, "/x/benchmark", "/out/exec", resident=True)
+    assert r[0][r[0].index("--") + 1:] == ["/x/benchmark", "-n", "33", "-r", "0", "a0", "b0"]
+    assert all(x[1:3] == ["-v", "-r"] for x in suite.valid_commands(info, "/x/benchmark", resident=True))
 
 
 def test_single_and_parallel_statistics():
