@@ -1082,6 +1082,7 @@ int bfuse_fill_uniform_device(int side, int tensor, unsigned long long seed, flo
     if (tensor != 0 && tensor != 1) return fail(BFUSE_ERR_ARG, "tensor must be 0 (I) or 1 (F)");
     if (s.elem[tensor] != 4 && s.elem[tensor] != 2)
         return fail(BFUSE_ERR_ARG, "device fill writes fp32 or bf16 tensors, this one has %d-byte elements", s.elem[tensor]);
+    if (int rc = sync_and_check()) return rc;   // nothing launched earlier may still be reading the operand
     const size_t n = s.bytes[tensor] / (size_t)s.elem[tensor];
     size_t blocks = (n + 256 * 8 - 1) / (256 * 8);
     if (blocks > 16384) blocks = 16384;
