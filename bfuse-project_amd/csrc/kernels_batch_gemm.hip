@@ -41,3 +41,6 @@ BGEMM_F32(1024, 208, 64, 208, 16, 208, 1)
 BGEMM_F32(1024, 208, 208, 64, 16, 64, 1)
 BGEMM_F32(1024, 208, 80, 208, 16, 208, 1)
 BGEMM_F32(1024, 208, 208, 80, 16, 80, 1)
+// tests/interleave_scheduler/config/info.yaml: bgemm_6, bgemm_7
+BGEMM_F32_RESERVE(1024, 1024, 64, 512, 64, 64, 1, 32768)
+BGEMM_F32(1024, 1024, 512, 64, 32, 64, 2)

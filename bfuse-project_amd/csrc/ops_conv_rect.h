@@ -291,21 +291,41 @@ struct ConvF32Rect {
 // The tiling the library gives a convolution it has no hand-picked one for: as many output channels per
 // workgroup as keep the filter fragments of a wave within ~72 registers (the staged patch is shared by all
 // of them), 64 pixels (or the whole image when it has fewer), and as many waves over the channel groups as
-// leave room for two workgroups' patches in a CU's LDS.  The pixels are a 4 x 16 rectangle (ConvF32Rect) for
-// filters larger than 1 x 1 on images at least 56 outputs wide, else 64 consecutive pixels (ConvF32Lds).
-// Measured at batch 1024, rectangle against consecutive pixels: 2.3-2.5x on 147-, 149- and 299-wide images,
-// 1.6x for the 7 x 7 on 224, 1.3x on 73, 1.1x on 56; 0.8-0.9x on 35- and 28-wide images and 0.45-0.55x on 17-,
-// 8- and 7-wide ones, whose rows fill half of a 16-column tile or less; 1 x 1 filters have no halo to save.
+// leave room for two workgroups' patches in a CU's LDS.
+//
+// The pixels are a rectangle of 16 columns (ConvF32Rect) for filters larger than 1 x 1 on wide images whose
+// rows fill their 16-column tiles well -- at least 64 outputs wide, or at least 44 with five sixths of the
+// tile columns in use -- else 64 consecutive pixels (ConvF32Lds).  Measured at batch 1024, rectangle against
+// consecutive pixels: 2.3-2.5x on 147-, 149- and 299-wide images, 2.2x on 55 outputs at stride 2, 1.6x for the
+// 7 x 7 on 224, 1.3x on 73 and on 48, 1.1x on 56, 54 and 44; 1.0x on 50 (14 of its 64 tile columns idle);
+// 0.8-0.9x on 35- and 28-wide images and 0.45-0.55x on 17-, 8- and 7-wide ones, whose rows fill half of a
+// tile or less; 1 x 1 filters have no halo to save.
+//
+// The rectangle has 4 rows while a wave's patch of 16 channels stays within 12.5 KB, else 2, else 1: a stride
+// widens the patch (9 x 33 pixels for 4 rows of a 3 x 3 filter at stride 2, 7 x 63 for 2 rows at stride 4), and
+// the smaller patch lets more workgroups share a CU and hide the staging of each other's patches: 2 rows against
+// 4 at stride 2, 1.20x (112-wide, 64 channels) and 1.12x (147-wide, 32 channels); 1 row against 2 at stride 4,
+// 1.4x (227-wide).
+//
+// A strided layer with so few output channels that it computes less per byte of image than the chip can
+// (CO x taps / (2 x stride^2) flops per byte against ~20) is bound by reading the image: one workgroup then
+// computes all output channels (up to 64), so that the image is read once (1.14x on the 227-wide layer).
 template <int CI, int CO, int H, int W, int KH, int KW, int S, int P, int NIMG>
 struct ConvTiling {
     static constexpr int T = KH * KW;
     static constexpr int OH = (H - KH + 2 * P) / S + 1, OW = (W - KW + 2 * P) / S + 1;
     static constexpr int OHW = OH * OW;
+    static constexpr bool RECT = T > 1 && (OW >= 64 || (OW >= 44 && 6 * OW >= 5 * ((OW + 15) / 16 * 16)));
+    static constexpr int patch_bytes(int th) { return ((th - 1) * S + KH) * (15 * S + KW) * (CI >= 16 ? 64 : 16); }
+    static constexpr int TH = patch_bytes(4) <= 12800 ? 4 : patch_bytes(2) <= 12800 ? 2 : 1;
     static constexpr int pick_bm()
     {
         if (CI < 16) return 16;
         if (T == 1)      // a 1x1 filter is one register per row block: as many output channels as divide CO, up to 80
             for (int bm = 80; bm > 16; bm -= 16)     // (96 measured slower than 64 on the 8x8 and 17x17 layers)
+                if (CO % bm == 0) return bm;
+        if (RECT && CO * T < 40 * S * S)             // bound by reading the image
+            for (int bm = 64; bm > 16; bm -= 16)
                 if (CO % bm == 0) return bm;
         if (CO % 64 == 0 && 4 * T <= 18) return 64;
         if (CO % 48 == 0 && 3 * T <= 18) return 48;
@@ -313,19 +333,22 @@ struct ConvTiling {
         return 16;
     }
     static constexpr int BM = pick_bm();
-    static constexpr bool RECT = T > 1 && OW >= 56;
     static constexpr int PB = OHW >= 64 ? 4 : (OHW + 15) / 16;
     static constexpr int NGROUP = CI >= 16 ? CI / 16 : 1;
-    static constexpr int TILE = RECT ? ConvF32Rect<CI, CO, H, W, KH, KW, S, P, BM, 4, 1, NIMG>::TILE_BYTES
-                                     : ConvF32Lds<CI, CO, H, W, KH, KW, S, P, BM, PB, 1, NIMG>::TILE_BYTES;
+    // (only the chosen form is instantiated: the other may not fit this shape at all)
+    static constexpr int TILE = std::conditional_t<RECT, ConvF32Rect<CI, CO, H, W, KH, KW, S, P, BM, TH, 1, NIMG>,
+                                                   ConvF32Lds<CI, CO, H, W, KH, KW, S, P, BM, PB, 1, NIMG>>::TILE_BYTES;
     static constexpr int pick_ks()
     {
-        if (NGROUP % 4 == 0 && 4 * TILE <= 80 * 1024) return 4;
-        if (NGROUP % 2 == 0 && 2 * TILE <= 80 * 1024) return 2;
+        // a rectangle gets no more waves than it has rows: the sum of the waves' partial tiles costs the same
+        // whatever the rows' arithmetic (4 waves on 2 rows: 0.92x of 2 waves on the 112-wide stride-2 layer)
+        const int most = RECT ? TH : 4;
+        if (most >= 4 && NGROUP % 4 == 0 && 4 * TILE <= 80 * 1024) return 4;
+        if (most >= 2 && NGROUP % 2 == 0 && 2 * TILE <= 80 * 1024) return 2;
         return 1;
     }
     static constexpr int KS = pick_ks();
-    using type = std::conditional_t<RECT, ConvF32Rect<CI, CO, H, W, KH, KW, S, P, BM, 4, KS, NIMG>,
+    using type = std::conditional_t<RECT, ConvF32Rect<CI, CO, H, W, KH, KW, S, P, BM, TH, KS, NIMG>,
                                     ConvF32Lds<CI, CO, H, W, KH, KW, S, P, BM, PB, KS, NIMG>>;
 };
 template <int CI, int CO, int H, int W, int KH, int KW, int S, int P, int NIMG = 1>

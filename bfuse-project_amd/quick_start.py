@@ -1,7 +1,7 @@
 """One command from a user config to the speed-up table: the reference's scripts/quick_start.py
 (`quick_start.py example -o file`, its six steps :27-160).
 
-    python -m bfuse_project_amd.quick_start example.yaml -o OUT [--dtype f32|bf16] [--skip-missing] [--build-pairs]
+    python -m bfuse_project_amd.quick_start example.yaml -o OUT [--dtype f32|bf16] [--skip-missing] [--build-pairs] [--resident]
 
   reference step                                   here
   [1/6] configure test-suite (TVM kernels)         [1/3] `configure`: ids resolved against the registry
@@ -9,6 +9,8 @@
                                                    --build-pairs: `build_pairs` writes and compiles the pairs it lacks
   [3/6] generate benchmark, [4/6] make             -- the harness is the library; nothing is generated or compiled
   [5/6] profile the benchmark                      [2/3] `suite`: every pair in every mode, validated, traces under OUT/exec
+                                                   (--resident: operands written and outputs compared on the device, for
+                                                   operators at batch 1024 whose tensors run to GB)
   [6/6] draw profile results                       [3/3] speed-up table: OUT/summary.md, OUT/summary.json
 """
 import argparse
@@ -24,6 +26,7 @@ def main(argv=None) -> int:
     ap.add_argument("--dtype", choices=("f32", "bf16"), default=None)
     ap.add_argument("--skip-missing", action="store_true", help="drop operator ids the library has no kernel for")
     ap.add_argument("--build-pairs", action="store_true", help="build the fused kernels the library lacks for this suite's pairs (hipcc)")
+    ap.add_argument("--resident", action="store_true", help="operands written and results compared on the device (operators at batch 1024)")
     args = ap.parse_args(argv)
     from . import build_pairs, configure, suite
 
@@ -48,7 +51,7 @@ def main(argv=None) -> int:
             built = build_pairs.build(args.file)
             print(f"  built {len(built['kernels'])} fused kernels", flush=True)
         build_pairs.load_suite_modules(args.file)
-        rows = suite.run_suite(info, args.file, validate=True)
+        rows = suite.run_suite(info, args.file, validate=True, resident=args.resident)
     except Exception as e:   # a failed validation or a device error ends the run, as the reference's check=True does
         print(f"Error occurs while profiling the benchmark: {e}", file=sys.stderr)
         return 1

@@ -142,3 +142,27 @@ def test_the_references_own_example_configs_resolve_completely(tmp_path, name, c
     if name == "llm.yaml":
         rb = configure.configure(str(p), str(tmp_path / "ob"), dtype="bf16")
         assert {k for k, d in rb["resolved"].items() if d["dtype"] == "bf16"} == {"dense_4", "dense_6", "dense_7"}
+
+
+REF_SUITE = "/root/reference/tests/interleave_scheduler/config/info.yaml"
+
+
+@pytest.mark.skipif(not os.path.exists(REF_SUITE), reason="the reference's generated suites are not on this machine")
+def test_the_references_interleave_scheduler_suite_resolves_completely(tmp_path):
+    """The reference's third generated suite (its info.yaml read in place: 8 batched products x 8 convolutions at
+    batch 1024): the example config in this tree lists the same ids with the same arguments and the same two
+    sets, and every id resolves to a kernel of the reference's shapes."""
+    with open(REF_SUITE) as f:
+        ref = yaml.safe_load(f)
+    here = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "bfuse-project_amd", "examples", "interleave_scheduler_batch1024.yaml")
+    with open(here) as f:
+        doc = yaml.safe_load(f)
+    assert doc["KernelInfo"] == ref["KernelInfo"]
+    assert [s["Set"] for s in doc["FusionSet"]] == [s["Set"] for s in ref["FusionSet"]]
+    r = configure.configure(here, str(tmp_path / "o"))
+    assert len(r["found"]) == 16 and not r["missing"]
+    reg = {k.name: k for k in bf.operation.list_kernels()}
+    for kid, args in doc["KernelInfo"].items():
+        data, weight, out = configure.shapes_of(kid, args)
+        k = reg[r["found"][kid]]
+        assert configure._dims(k.shapes[0]) == configure._dims(data) and configure._dims(k.shapes[2]) == configure._dims(out)

@@ -1,4 +1,5 @@
-"""The operators of the reference's test-utils/examples/benchmark.yaml and inception_v3.yaml: every operator at
+"""The operators of the reference's test-utils/examples/benchmark.yaml and inception_v3.yaml and of its generated suite
+tests/interleave_scheduler (config/info.yaml): every operator at
 batch 1024 (convolutions of 1024 images, 1024 independent batched products, dense layers of 1024 rows).
 
 Operands and results of these run to several GB, so nothing passes through one host array: the batch is made of
@@ -65,7 +66,10 @@ CONVS = [
     (73, 73, 192, 80, 3, 3, 1, 0), (35, 35, 64, 192, 1, 1, 1, 0), (35, 35, 48, 192, 1, 1, 1, 0), (35, 35, 64, 48, 5, 5, 1, 2),
     (35, 35, 96, 64, 3, 3, 1, 1), (35, 35, 96, 96, 3, 3, 1, 1), (35, 35, 32, 192, 1, 1, 1, 0), (8, 8, 320, 1280, 1, 1, 1, 0),
     (8, 8, 384, 1280, 1, 1, 1, 0), (8, 8, 448, 1280, 1, 1, 1, 0), (8, 8, 384, 448, 3, 3, 1, 1), (8, 8, 192, 1280, 1, 1, 1, 0),
-    (8, 8, 320, 2048, 1, 1, 1, 0), (8, 8, 384, 2048, 1, 1, 1, 0), (8, 8, 448, 2048, 1, 1, 1, 0), (8, 8, 192, 2048, 1, 1, 1, 0)]
+    (8, 8, 320, 2048, 1, 1, 1, 0), (8, 8, 384, 2048, 1, 1, 1, 0), (8, 8, 448, 2048, 1, 1, 1, 0), (8, 8, 192, 2048, 1, 1, 1, 0),
+    # tests/interleave_scheduler/config/info.yaml (its two 56 x 56, 64 -> 64, 1 x 1 layers are in the list above)
+    (112, 112, 192, 64, 3, 3, 2, 0), (147, 147, 64, 32, 3, 3, 2, 0), (56, 56, 128, 64, 3, 3, 1, 0), (28, 28, 256, 128, 3, 3, 1, 0),
+    (227, 227, 64, 16, 3, 3, 4, 0), (56, 56, 256, 256, 1, 1, 1, 0)]
 
 
 @pytest.mark.parametrize("h,w,co,ci,kh,kw,s,p", CONVS)
@@ -108,7 +112,8 @@ def test_convolution_of_1024_images(h, w, co, ci, kh, kw, s, p):
 
 # ---- batched products: batch, M, K, N; C[b] = A[b] . B[b]^T with B [b, N, K] (configure_kernels.py:14-19) -----
 BGEMMS = [(512, 64, 512), (512, 512, 64), (512, 128, 512), (512, 512, 128), (256, 64, 256), (256, 256, 64), (256, 80, 256),
-          (256, 256, 80), (208, 64, 208), (208, 208, 64), (208, 80, 208), (208, 208, 80)]
+          (256, 256, 80), (208, 64, 208), (208, 208, 64), (208, 80, 208), (208, 208, 80),
+          (1024, 64, 512), (1024, 512, 64)]     # the last two: tests/interleave_scheduler/config/info.yaml
 
 
 @pytest.mark.parametrize("m,k,n", BGEMMS)
