@@ -30,7 +30,7 @@ import yaml
 PKG = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG, "csrc")
 LDS_PER_WORKGROUP = 160 * 1024
-HEADERS = ("fuse.h", "ops_conv.h", "ops_conv_general.h", "ops_conv_rect.h", "ops_gemm_bf16.h", "ops_gemm_f32.h", "ops_gemm_f32_dma.h",
+HEADERS = ("fuse.h", "ops_conv.h", "ops_conv_1x1.h", "ops_conv_general.h", "ops_conv_rect.h", "ops_gemm_bf16.h", "ops_gemm_f32.h", "ops_gemm_f32_dma.h",
            "ops_layout.h", "ops_pool.h", "ops_rowwise.h")
 
 
