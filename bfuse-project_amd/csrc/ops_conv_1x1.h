@@ -174,7 +174,7 @@ struct Conv1x1F32 {
             for (int s = 0; s < 4; ++s) xc[s] = load_x(xq + (size_t)s * HW, p, off, tail);
         }
         put_w(0);
-        sync();
+        if constexpr (NW > 1) sync();     // (one wave orders its own LDS accesses)
 
 #pragma unroll 1
         for (int c = 0; c < NC; ++c) {
@@ -206,7 +206,7 @@ struct Conv1x1F32 {
             }
             if (c + 1 < NC) {
                 put_w((c + 1) & 1);
-                sync();     // everyone is done with this chunk's buffer, and the next chunk is in place
+                if constexpr (NW > 1) sync();     // everyone is done with this chunk's buffer, and the next chunk is in place
             }
         }
 

@@ -152,3 +152,27 @@ def test_clock_stamped_gemm_computes_what_the_product_kernel_computes():
     table = clock_table(20)
     print(table, flush=True)
     assert "shader clocks per K-stage" in table and table.count("| 7 |") == 2
+
+
+def test_scheduler_probe_reports_the_mix_of_two_operators_per_cu_and_xcd():
+    """The reference's scheduler experiment (tests/interleave_scheduler/test/test_scheduler.py) on this chip: under
+    the 1:1 interleave every XCD, and so every CU, sees one operator only; in chunks of 256 every XCD sees both
+    alike.  (What an XCD receives follows from id % 8 and is asserted; how an XCD spreads its workgroups over its
+    CUs while others are resident is the hardware's business and is printed.)"""
+    import numpy as np
+    from bfuse_project_amd import scheduler_probe as sp
+    print("scheduler probe: zigzag", flush=True)
+    z = sp.probe("zigzag", (2048, 2048), 256, 1, 1)
+    assert z["fused_grid"] == 4096 and z["side"].size == 4096 and z["cu"].max() <= 255
+    zx = sp.mix_statistics(z["xcd"], z["side"])
+    assert zx["units"] == 8 and zx["mean_diff"] == 1.0
+    assert sp.mix_statistics(z["cu"], z["side"])["mean_diff"] == 1.0
+    print(sp.report(z, color=False), flush=True)
+    print("scheduler probe: chunked", flush=True)
+    c = sp.probe("chunked", (2048, 2048), 256, 256, 1)
+    cx = sp.mix_statistics(c["xcd"], c["side"])
+    assert cx["mean_diff"] == 0.0 and np.all(cx["n0"] == 256) and np.all(cx["n1"] == 256)
+    cc = sp.mix_statistics(c["cu"], c["side"])
+    print(sp.report(c, color=False), flush=True)
+    assert cc["mean_diff"] < 0.5
+    assert sp.main(["--pattern", "ranges", "--grids", "512", "256", "--first", "600", "--rows", "3", "--no-color"]) == 0
