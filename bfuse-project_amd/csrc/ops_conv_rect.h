@@ -295,12 +295,14 @@ struct ConvF32Rect {
 // leave room for two workgroups' patches in a CU's LDS.
 //
 // The pixels are a rectangle of 16 columns (ConvF32Rect) for filters larger than 1 x 1 on wide images whose
-// rows fill their 16-column tiles well -- at least 64 outputs wide, or at least 44 with five sixths of the
-// tile columns in use -- else 64 consecutive pixels (ConvF32Lds).  Measured at batch 1024, rectangle against
+// rows fill their 16-column tiles well -- at least 64 outputs wide, or at least 44 (any width at a stride: 64
+// consecutive outputs of a strided layer need twice the image rows) with five sixths of the tile columns in
+// use -- else 64 consecutive pixels (ConvF32Lds).  Measured at batch 1024, rectangle against
 // consecutive pixels: 2.3-2.5x on 147-, 149- and 299-wide images, 2.2x on 55 outputs at stride 2, 1.6x for the
 // 7 x 7 on 224, 1.3x on 73 and on 48, 1.1x on 56, 54 and 44; 1.0x on 50 (14 of its 64 tile columns idle);
 // 0.8-0.9x on 35- and 28-wide images and 0.45-0.55x on 17-, 8- and 7-wide ones, whose rows fill half of a
-// tile or less; 1 x 1 filters have no halo to save.
+// tile or less; at stride 2 1.14x on 28 and 1.23x on 14 outputs, 0.72x on 17, 0.55x on 8, 0.41x on 7; 1 x 1
+// filters have no halo to save.
 //
 // The rectangle has 4 rows while a wave's patch of 16 channels stays within 12.5 KB, else 2, else 1: a stride
 // widens the patch (9 x 33 pixels for 4 rows of a 3 x 3 filter at stride 2, 7 x 63 for 2 rows at stride 4), and
@@ -316,7 +318,7 @@ struct ConvTiling {
     static constexpr int T = KH * KW;
     static constexpr int OH = (H - KH + 2 * P) / S + 1, OW = (W - KW + 2 * P) / S + 1;
     static constexpr int OHW = OH * OW;
-    static constexpr bool RECT = T > 1 && (OW >= 64 || (OW >= 44 && 6 * OW >= 5 * ((OW + 15) / 16 * 16)));
+    static constexpr bool RECT = T > 1 && (OW >= 64 || ((OW >= 44 || S > 1) && 6 * OW >= 5 * ((OW + 15) / 16 * 16)));
     static constexpr int patch_bytes(int th) { return ((th - 1) * S + KH) * (15 * S + KW) * (CI >= 16 ? 64 : 16); }
     static constexpr int TH = patch_bytes(4) <= 12800 ? 4 : patch_bytes(2) <= 12800 ? 2 : 1;
     static constexpr int pick_bm()
