@@ -25,22 +25,24 @@ DENSE_F32(1024, 14336, 4096, 64, 128, 4)
 #define BGEMM_F32(B, M, K, N, BM, BN, KS)                                                                        \
     using Bgemm_##B##x##M##x##K##x##N = GemmF32<M, N, K, BM, BN, KS, kEpiNone, 2, 1, true, B>;                    \
     BFUSE_KERNEL(bgemm_f32_##B##x##M##x##K##x##N, Bgemm_##B##x##M##x##K##x##N, ({{B, M, K, 1}, 4}), ({{B, N, K, 1}, 4}), ({{B, M, N, 1}, 4}))
-// the one-wave products reserve 32 KB of LDS per workgroup: four workgroups per CU, one wave per SIMD (see LdsReserve)
+// the one-wave products reserve 32 KB of LDS per workgroup: four workgroups per CU, one wave per SIMD (see LdsReserve).
+// (128 x 64 tiles run the K <= 128 products 7-16 % faster but need 300 registers: a fused kernel, which is compiled
+// for two waves per SIMD, has 256, so those stay on 64 x 64.)
 #define BGEMM_F32_RESERVE(B, M, K, N, BM, BN, KS, BYTES)                                                         \
     using Bgemm_##B##x##M##x##K##x##N = LdsReserve<GemmF32<M, N, K, BM, BN, KS, kEpiNone, 2, 1, true, B>, BYTES>; \
     BFUSE_KERNEL(bgemm_f32_##B##x##M##x##K##x##N, Bgemm_##B##x##M##x##K##x##N, ({{B, M, K, 1}, 4}), ({{B, N, K, 1}, 4}), ({{B, M, N, 1}, 4}))
-BGEMM_F32_RESERVE(1024, 512, 64, 512, 128, 64, 1, 32768)
+BGEMM_F32_RESERVE(1024, 512, 64, 512, 64, 64, 1, 32768)
 BGEMM_F32(1024, 512, 512, 64, 64, 64, 2)
-BGEMM_F32_RESERVE(1024, 512, 128, 512, 128, 64, 1, 32768)
+BGEMM_F32_RESERVE(1024, 512, 128, 512, 64, 64, 1, 32768)
 BGEMM_F32(1024, 512, 512, 128, 64, 64, 2)
-BGEMM_F32_RESERVE(1024, 256, 64, 256, 128, 64, 1, 32768)
+BGEMM_F32_RESERVE(1024, 256, 64, 256, 64, 64, 1, 32768)
 BGEMM_F32_RESERVE(1024, 256, 256, 64, 64, 64, 1, 32768)
-BGEMM_F32_RESERVE(1024, 256, 80, 256, 128, 64, 1, 32768)
+BGEMM_F32_RESERVE(1024, 256, 80, 256, 64, 64, 1, 32768)
 BGEMM_F32_RESERVE(1024, 256, 256, 80, 64, 80, 1, 32768)
 BGEMM_F32(1024, 208, 64, 208, 16, 208, 1)
 BGEMM_F32_RESERVE(1024, 208, 208, 64, 208, 32, 1, 32768)
 BGEMM_F32(1024, 208, 80, 208, 16, 208, 1)
 BGEMM_F32(1024, 208, 208, 80, 208, 16, 1)
 // tests/interleave_scheduler/config/info.yaml: bgemm_6, bgemm_7
-BGEMM_F32_RESERVE(1024, 1024, 64, 512, 128, 64, 1, 32768)
+BGEMM_F32_RESERVE(1024, 1024, 64, 512, 64, 64, 1, 32768)
 BGEMM_F32(1024, 1024, 512, 64, 64, 64, 2)
