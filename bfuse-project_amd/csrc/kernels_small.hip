@@ -6,6 +6,7 @@
 #include "fuse.h"
 #include "ops_ceiling.h"
 #include "ops_conv.h"
+#include "ops_conv_1x1.h"
 #include "ops_gemm_bf16.h"
 #include "ops_gemm_f32.h"
 #include "ops_gemm_f32_dma.h"
@@ -58,6 +59,9 @@ using ConvS1 = Conv3x3F32Lds<16, 16, 8, 8, 16, 1, 1>;                 // one cha
 using ConvS2 = Conv3x3F32Lds<32, 32, 12, 12, 16, 1, 2>;               // two channel groups on two waves
 using ConvS3 = Conv3x3F32Lds<64, 16, 8, 16, 16, 2, 2>;                // two groups per wave, two pixel blocks
 using PoolS = MaxPool3x3S2<4, 16, 16, 64>;
+using Conv1S1 = Conv1x1F32<32, 32, 5, 5, 1, 32, 4, 3>;                 // streamed 1x1: three images of 25 pixels = three ragged tiles in one workgroup, its fourth wave without a tile
+using Conv1S2 = Conv1x1F32<96, 48, 9, 9, 1, 16, 2, 5>;                 // 64 + 17 pixels per image, three channel tiles, two filter chunks of 48 channels (192 staging units on 128 threads)
+using Conv1S3 = Conv1x1F32<16, 16, 9, 7, 2, 16, 1, 2>;                 // stride 2 (9 x 7 -> 5 x 4), one wave per workgroup: no barrier
 using GemmB1 = GemmBf16NTDma<128, 1792, 64, 128, 224, 2>;             // one K-step
 using GemmB2 = GemmBf16NTDma<128, 1792, 192, 128, 224, 2>;            // two stages, three K-steps
 using GemmB3 = GemmBf16NTDma<256, 1792, 320, 128, 224, 3>;            // two M-tiles, ring of three, five K-steps
@@ -78,6 +82,9 @@ BFUSE_KERNEL(softmax_causal_2x256x256, SoftmaxS, ({{2, 256, 256, 1}, 4}), ({{1, 
 BFUSE_KERNEL(conv3x3_f32_16x8x8_16, ConvS1, ({{1, 16, 8, 8}, 4}), ({{16, 16, 3, 3}, 4}), ({{1, 16, 8, 8}, 4}))
 BFUSE_KERNEL(conv3x3_f32_32x12x12_32, ConvS2, ({{1, 32, 12, 12}, 4}), ({{32, 32, 3, 3}, 4}), ({{1, 32, 12, 12}, 4}))
 BFUSE_KERNEL(conv3x3_f32_64x8x16_16, ConvS3, ({{1, 64, 8, 16}, 4}), ({{16, 64, 3, 3}, 4}), ({{1, 16, 8, 16}, 4}))
+BFUSE_KERNEL(conv1x1s1p0_f32_3x32x5x5_32, Conv1S1, ({{3, 32, 5, 5}, 4}), ({{32, 32, 1, 1}, 4}), ({{3, 32, 5, 5}, 4}))
+BFUSE_KERNEL(conv1x1s1p0_f32_5x96x9x9_48, Conv1S2, ({{5, 96, 9, 9}, 4}), ({{48, 96, 1, 1}, 4}), ({{5, 48, 9, 9}, 4}))
+BFUSE_KERNEL(conv1x1s2p0_f32_2x16x9x7_16, Conv1S3, ({{2, 16, 9, 7}, 4}), ({{16, 16, 1, 1}, 4}), ({{2, 16, 5, 4}, 4}))
 BFUSE_KERNEL(maxpool3x3s2_f32_4x16x16, PoolS, ({{1, 4, 16, 16}, 4}), ({{1, 1, 1, 1}, 4}), ({{1, 4, 8, 8}, 4}))
 BFUSE_KERNEL(gemm_bf16_128x64x1792, GemmB1, ({{128, 64, 1, 1}, 2}), ({{1792, 64, 1, 1}, 2}), ({{128, 1792, 1, 1}, 2}))
 BFUSE_KERNEL(gemm_bf16_128x192x1792, GemmB2, ({{128, 192, 1, 1}, 2}), ({{1792, 192, 1, 1}, 2}), ({{128, 1792, 1, 1}, 2}))
@@ -134,6 +141,12 @@ BFUSE_HFUSE_KERNEL(conv3x3_f32_32x12x12_32, ConvS2, bias_relu_4096, BiasReluS)
 BFUSE_BFUSE_KERNEL(conv3x3_f32_64x8x16_16, ConvS3, layernorm_8x256, LayerNormS, _c4, bfuse::kChunked, 4, 1)
 // both sides synchronise (each split-K GEMM's reduction barriers): each side gets LDS arrival counters of its own
 BFUSE_HFUSE_KERNEL(gemm_f32_128x160x192_d, GemmS5, gemm_gelu_f32_64x192x288_d, GemmS6)
+// the streamed 1x1 convolution (a barrier per filter chunk): block-fused, thread-fused with a side that never
+// synchronises, and with one that does
+BFUSE_BFUSE_KERNEL(conv1x1s1p0_f32_3x32x5x5_32, Conv1S1, layernorm_8x256, LayerNormS, _c4, bfuse::kChunked, 4, 1)
+BFUSE_HFUSE_KERNEL(conv1x1s1p0_f32_5x96x9x9_48, Conv1S2, bias_relu_4096, BiasReluS)
+BFUSE_HFUSE_KERNEL(conv1x1s1p0_f32_5x96x9x9_48, Conv1S2, conv3x3_f32_32x12x12_32, ConvS2)
+BFUSE_BFUSE_KERNEL(conv1x1s2p0_f32_2x16x9x7_16, Conv1S3, bias_relu_4096, BiasReluS, , bfuse::kZigzag, 1, 1)
 // the give-up path of the side barrier, forced from the host with a small spin limit
 BFUSE_KERNEL(selftest_sync_a, SyncProbeA, ({{512, 1, 1, 1}, 4}), ({{512, 1, 1, 1}, 4}), ({{512, 1, 1, 1}, 4}))
 BFUSE_KERNEL(selftest_sync_b, SyncProbeB, ({{768, 1, 1, 1}, 4}), ({{768, 1, 1, 1}, 4}), ({{768, 1, 1, 1}, 4}))

@@ -55,6 +55,12 @@ def _cases():
                                     lambda I, F: orf.conv2d(I.reshape(1, 32, 12, 12), F.reshape(32, 32, 3, 3)), 1e-5, False),
         "conv3x3_f32_64x8x16_16": (lambda s: (fill_normal(s, 64 * 128, 0, 1), fill_normal(s + 1, 16 * 64 * 9, 0, 0.05)),
                                    lambda I, F: orf.conv2d(I.reshape(1, 64, 8, 16), F.reshape(16, 64, 3, 3)), 1e-5, False),
+        "conv1x1s1p0_f32_3x32x5x5_32": (lambda s: (fill_normal(s, 3 * 32 * 25, 0, 1), fill_normal(s + 1, 32 * 32, 0, 0.2)),
+                                        lambda I, F: orf.conv2d(I.reshape(3, 32, 5, 5), F.reshape(32, 32, 1, 1), s=1, p=0), 1e-5, False),
+        "conv1x1s1p0_f32_5x96x9x9_48": (lambda s: (fill_normal(s, 5 * 96 * 81, 0, 1), fill_normal(s + 1, 48 * 96, 0, 0.1)),
+                                        lambda I, F: orf.conv2d(I.reshape(5, 96, 9, 9), F.reshape(48, 96, 1, 1), s=1, p=0), 1e-5, False),
+        "conv1x1s2p0_f32_2x16x9x7_16": (lambda s: (fill_normal(s, 2 * 16 * 63, 0, 1), fill_normal(s + 1, 16 * 16, 0, 0.25)),
+                                        lambda I, F: orf.conv2d(I.reshape(2, 16, 9, 7), F.reshape(16, 16, 1, 1), s=2, p=0), 1e-5, False),
         "maxpool3x3s2_f32_4x16x16": (lambda s: (fill_normal(s, 4 * 256, -3, 1), z),        # all-negative: padding must not win
                                      lambda I, F: orf.maxpool2d(I.reshape(1, 4, 16, 16)), 0.0, False),
         "gemm_bf16_128x64x1792": (lambda s: (f32_to_bf16(fill_normal(s, 128 * 64, 0, 1)), f32_to_bf16(fill_normal(s + 1, 1792 * 64, 0, 0.1))),
@@ -93,6 +99,10 @@ FUSIONS = [
     ("gemm_f32_128x160x192_d", "gemm_gelu_f32_64x192x288_d", "hfuse", ""),    # both sides synchronise: LDS arrival counters
     ("conv3x3_f32_32x12x12_32", "bias_relu_4096", "hfuse", ""),
     ("conv3x3_f32_64x8x16_16", "layernorm_8x256", "bfuse", "_c4"),
+    ("conv1x1s1p0_f32_3x32x5x5_32", "layernorm_8x256", "bfuse", "_c4"),
+    ("conv1x1s1p0_f32_5x96x9x9_48", "bias_relu_4096", "hfuse", ""),                # a barrier per filter chunk beside a side without any: LDS arrival counters
+    ("conv1x1s1p0_f32_5x96x9x9_48", "conv3x3_f32_32x12x12_32", "hfuse", ""),       # both sides synchronise
+    ("conv1x1s2p0_f32_2x16x9x7_16", "bias_relu_4096", "bfuse", ""),
 ]
 
 
