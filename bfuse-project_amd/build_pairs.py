@@ -225,9 +225,13 @@ def build(suite: str, forms: str = "both", chunk: int = 256, only: Optional[Sequ
           jobs: int = 8, compile_: bool = True, triangular: bool = False, rt: bool = False) -> dict:
     """Writes <suite>/hip/pairs_*.hip for the suite's pairs that lack a fused kernel and builds the module.
     Returns {"kernels": [...], "files": [...], "module": path or None}."""
+    from . import build_operators
     from .operation import list_kernels
-    # the library's own kernels; what an earlier run wrote for this suite is read from its translation units below
-    # (its module is not loaded here: one built against older headers would be refused, and is about to be rebuilt)
+    # the library's own kernels and the operators built for this suite's config (configure --build-missing: their
+    # module is brought up to date and loaded); what an earlier run wrote for this suite is read from its
+    # translation units below (the module of fused kernels is not loaded here: one built against older headers
+    # would be refused, and is about to be rebuilt)
+    build_operators.rebuild_and_load(suite, jobs)
     registry = {k.name: k for k in list_kernels()}
     pairs = suite_pairs(suite, triangular)
     if only:
@@ -270,8 +274,7 @@ def build(suite: str, forms: str = "both", chunk: int = 256, only: Optional[Sequ
             if r.returncode != 0:
                 raise RuntimeError(f"building {module} failed:\n{r.stdout[-3000:]}\n{r.stderr[-3000:]}")
             todo = [k for k in todo if k["name"] not in dropped]
-        with open(os.path.join(suite, "config", "modules.yaml"), "w") as f:
-            yaml.safe_dump([os.path.join("hip", "libbfuse_pairs.so")], f)
+        build_operators.name_module(suite, os.path.join("hip", "libbfuse_pairs.so"))
     return {"kernels": todo, "files": files, "module": module if compile_ else None, "dropped": dropped}
 
 

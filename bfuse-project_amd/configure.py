@@ -8,7 +8,7 @@ writes `<out>/cuda/kernels.cu` and `<out>/config/{kernels,fusions,info}.yaml`.  
 generated: every id is resolved against the library's registry of hand-written gfx950 kernels, whose
 shapes are compile-time, and the same three config files are written for what resolved:
 
-    python -m bfuse_project_amd.configure example.yaml -o OUT [--dtype f32|bf16] [--skip-missing]
+    python -m bfuse_project_amd.configure example.yaml -o OUT [--dtype f32|bf16] [--skip-missing | --build-missing]
 
 Arithmetic and weight layout are part of what an id resolves to, and are written down per id: by default
 every id resolves to an fp32 kernel, the reference's arithmetic; `--dtype bf16` takes the bf16 kernel where
@@ -29,7 +29,10 @@ to that one stated transposition.
   OUT/config/fused.yaml     for every pair, the fused kernels the library holds for it
 
 An id no registry kernel matches is reported with the lines that would instantiate it; the run then
-fails (exit status 1) unless --skip-missing drops such ids from the sets.
+fails (exit status 1) unless --skip-missing drops such ids from the sets, or --build-missing writes those
+instantiations (the templates' default tilings) into OUT/hip/operators/, compiles them into a kernel module of
+the suite and resolves the ids against it (build_operators: the counterpart of the reference generating a
+kernel for whatever arguments an id has).
 """
 import argparse
 import os
@@ -75,7 +78,8 @@ def candidate_names(kernel_id: str, args, dtype: Optional[str]) -> List[str]:
     types = ["bf16", "f32"] if dtype == "bf16" else ["f32"]
     if op == "dense":
         b, i, o = args
-        return [f"gemm_{t}_{b}x{i}x{o}" for t in types]
+        # (`..._nk`: an fp32 kernel that takes the weight as the reference stores it, (out, in): build_operators)
+        return [n for t in types for n in ([f"gemm_{t}_{b}x{i}x{o}"] + ([f"gemm_f32_{b}x{i}x{o}_nk"] if t == "f32" else []))]
     if op == "conv2d":
         n, h, w, co, ci, kh, kw, stride, pad = args
         names = []
@@ -115,7 +119,7 @@ def describe(kernel_id: str, args, kernel, registry) -> dict:
     if have[0] != want[0] or have[2] != want[2]:
         raise ValueError(f"{kernel_id}: {kernel.name} is registered for data {have[0]} -> {have[2]}, the id asks for {want[0]} -> {want[2]}")
     info = {"kernel": kernel.name, "dtype": dtype, "weight_layout": "reference", "weight_transpose": None}
-    if operator_of(kernel_id) == "dense" and WEIGHT_IS_IN_OUT.get(kernel.name.split("_")[0] + "_" + dtype, False):
+    if operator_of(kernel_id) == "dense" and not kernel.name.endswith("_nk") and WEIGHT_IS_IN_OUT.get(kernel.name.split("_")[0] + "_" + dtype, False):
         # the kernel family takes [in, out]; a square weight has the same shape either way, so the family decides
         if have[1] != want[1][::-1]:
             raise ValueError(f"{kernel_id}: {kernel.name} takes a weight of shape {have[1]}, [in, out] of the id's is {want[1][::-1]}")
@@ -185,14 +189,32 @@ def resolve(doc: dict, registry: Dict[str, object], dtype: Optional[str] = None)
     return found, missing
 
 
-def configure(path: str, out: str, dtype: Optional[str] = None, skip_missing: bool = False, registry=None) -> dict:
-    """Writes OUT/config/*.yaml and returns {"found", "missing", "pairs", "fused"}."""
+def configure(path: str, out: str, dtype: Optional[str] = None, skip_missing: bool = False, registry=None,
+              build_missing: bool = False) -> dict:
+    """Writes OUT/config/*.yaml and returns {"found", "missing", "pairs", "fused"}.  `build_missing`: the ids no
+    kernel implements are instantiated from the library's templates, built into OUT/hip/operators/ and loaded."""
     from . import config as cfg
-    if registry is None:
+    own_registry = registry is None
+    if own_registry:
         from .operation import list_kernels
         registry = {k.name: k for k in list_kernels()}
     doc = load_user_config(path)
+    if os.path.exists(out):
+        raise FileExistsError(f'"{out}" already exists.')                # configure_kernels.py:239-241
     found, missing = resolve(doc, registry, dtype)
+    built = {}
+    if missing and build_missing:
+        if not own_registry:
+            raise ValueError("build_missing works on the library's own registry")
+        from . import build_operators
+        try:
+            built = build_operators.build(out, {kid: doc["KernelInfo"][kid] for kid in missing})["kernels"]
+        except Exception:
+            import shutil
+            shutil.rmtree(out, ignore_errors=True)       # nothing half-configured is left behind
+            raise
+        registry = {k.name: k for k in list_kernels()}
+        found, missing = resolve(doc, registry, dtype)
     if missing and not skip_missing:
         lines = [f"  {kid} {doc['KernelInfo'][kid]}: {hint}" for kid, hint in missing.items()]
         raise LookupError("no kernel of the library implements:\n" + "\n".join(lines))
@@ -200,9 +222,7 @@ def configure(path: str, out: str, dtype: Optional[str] = None, skip_missing: bo
     if not sets[0] or not sets[1]:
         raise LookupError("a fusion set is empty" + (" after dropping the ids the library has no kernel for" if missing else ""))
     config_dir = os.path.join(out, "config")
-    if os.path.exists(out):
-        raise FileExistsError(f'"{out}" already exists.')                # configure_kernels.py:239-241
-    os.makedirs(config_dir)
+    os.makedirs(config_dir, exist_ok=True)
 
     infos = {}
     for kid, k in found.items():
@@ -226,7 +246,8 @@ def configure(path: str, out: str, dtype: Optional[str] = None, skip_missing: bo
             "Resolved": resolved}
     with open(os.path.join(config_dir, "info.yaml"), "w") as f:
         yaml.safe_dump(info, f, sort_keys=False)
-    return {"found": {k: v.name for k, v in found.items()}, "missing": missing, "pairs": pairs, "fused": fused, "resolved": resolved}
+    return {"found": {k: v.name for k, v in found.items()}, "missing": missing, "pairs": pairs, "fused": fused, "resolved": resolved,
+            "built": built}
 
 
 def main(argv=None) -> int:
@@ -236,13 +257,14 @@ def main(argv=None) -> int:
     ap.add_argument("--dtype", choices=("f32", "bf16"), default=None,
                     help="arithmetic type to resolve to: f32 (default, the reference's) or bf16 where the library holds a bf16 kernel (the others stay f32 and are listed)")
     ap.add_argument("--skip-missing", action="store_true", help="drop ids the library has no kernel for instead of failing")
+    ap.add_argument("--build-missing", action="store_true", help="instantiate the ids the library has no kernel for from its templates and compile them into a module of the suite (hipcc)")
     args = ap.parse_args(argv)
     if not os.path.exists(args.config):
         print(f'Given config path "{args.config}" doesn\'t exist.', file=sys.stderr)
         return 1
     try:
-        r = configure(args.config, args.file, args.dtype, args.skip_missing)
-    except (ValueError, LookupError, FileExistsError) as e:
+        r = configure(args.config, args.file, args.dtype, args.skip_missing, build_missing=args.build_missing)
+    except (ValueError, LookupError, FileExistsError, RuntimeError) as e:
         print(f"configure: {e}", file=sys.stderr)
         return 1
     for kid, d in r["resolved"].items():
@@ -254,6 +276,8 @@ def main(argv=None) -> int:
             print(f"no bf16 kernel, resolved to f32: {', '.join(kept)}", file=sys.stderr)
     for kid, hint in r["missing"].items():
         print(f"{kid}: dropped, no kernel ({hint})", file=sys.stderr)
+    for kid, name in r["built"].items():
+        print(f"{kid}: built {name}")
     print(f"{len(r['pairs'])} pairs, {sum(1 for v in r['fused'].values() if v)} with a fused kernel; wrote {os.path.join(args.file, 'config')}")
     return 0
 

@@ -1,10 +1,11 @@
 """One command from a user config to the speed-up table: the reference's scripts/quick_start.py
 (`quick_start.py example -o file`, its six steps :27-160).
 
-    python -m bfuse_project_amd.quick_start example.yaml -o OUT [--dtype f32|bf16] [--skip-missing] [--build-pairs] [--resident]
+    python -m bfuse_project_amd.quick_start example.yaml -o OUT [--dtype f32|bf16] [--skip-missing | --build-missing] [--build-pairs] [--resident]
 
   reference step                                   here
-  [1/6] configure test-suite (TVM kernels)         [1/3] `configure`: ids resolved against the registry
+  [1/6] configure test-suite (TVM kernels)         [1/3] `configure`: ids resolved against the registry (--build-missing: ids of
+                                                   shapes the library lacks are instantiated from its templates and compiled)
   [2/6] generate fused kernels (hfuse, bfuse)      -- the fused kernels are in the library (OUT/config/fused.yaml lists them);
                                                    --build-pairs: `build_pairs` writes and compiles the pairs it lacks
   [3/6] generate benchmark, [4/6] make             -- the harness is the library; nothing is generated or compiled
@@ -25,6 +26,7 @@ def main(argv=None) -> int:
     ap.add_argument("-o", dest="file", default="test-suite", help="output directory of the generated test-suite")
     ap.add_argument("--dtype", choices=("f32", "bf16"), default=None)
     ap.add_argument("--skip-missing", action="store_true", help="drop operator ids the library has no kernel for")
+    ap.add_argument("--build-missing", action="store_true", help="build the operator ids the library has no kernel for from its templates (hipcc)")
     ap.add_argument("--build-pairs", action="store_true", help="build the fused kernels the library lacks for this suite's pairs (hipcc)")
     ap.add_argument("--resident", action="store_true", help="operands written and results compared on the device (operators at batch 1024)")
     args = ap.parse_args(argv)
@@ -35,8 +37,8 @@ def main(argv=None) -> int:
         print(f'Given config path "{args.example}" doesn\'t exist.', file=sys.stderr)
         return 1
     try:
-        r = configure.configure(args.example, args.file, args.dtype, args.skip_missing)
-    except (ValueError, LookupError, FileExistsError) as e:
+        r = configure.configure(args.example, args.file, args.dtype, args.skip_missing, build_missing=args.build_missing)
+    except (ValueError, LookupError, FileExistsError, RuntimeError) as e:
         print(f"Error occurs while configuring '{args.file}': {e}", file=sys.stderr)
         return 1
     for kid, name in r["found"].items():

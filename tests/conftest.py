@@ -13,7 +13,7 @@ if ROOT not in sys.path:
 # entry point that allocates nothing last.  Files not listed keep their alphabetical place in the
 # middle group.
 FIRST = ("test_gpu_pairs.py", "test_gpu_small.py", "test_gpu_models.py", "test_gpu_general.py", "test_gpu_batch.py", "test_gpu_layout.py",
-         "test_gpu_multi.py", "test_gpu_frontend.py", "test_gpu_sync_giveup.py", "test_gpu_built_pairs.py")
+         "test_gpu_multi.py", "test_gpu_frontend.py", "test_gpu_sync_giveup.py", "test_gpu_built_pairs.py", "test_gpu_built_operators.py")
 LATE = ("test_gpu_driver.py", "test_gpu_suite.py", "test_gpu_rt_plan.py", "test_bench_contract.py")
 LAST = ("test_zz_no_alloc.py",)
 

@@ -1,0 +1,85 @@
+"""build_operators (the counterpart of the reference generating a kernel for whatever arguments an operator id has,
+scripts/configure_kernels.py:40-69): which ids the templates take, the tiling rule, the text of the translation unit,
+and `configure --build-missing` over the in-tree example (compiled by the build step)."""
+import os
+
+import pytest
+import yaml
+
+from bfuse_project_amd import build_operators as bo
+from bfuse_project_amd import configure
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_default_gemm_tiling_divides_the_problem():
+    assert bo.gemm_tiling(96, 80, 48) == (32, 80, 1)
+    assert bo.gemm_tiling(48, 96, 160) == (16, 96, 1)
+    assert bo.gemm_tiling(512, 512, 512) == (64, 64, 2)
+    assert bo.gemm_tiling(1024, 4096, 4096) == (64, 64, 4)
+    assert bo.gemm_tiling(16, 16, 16) == (16, 16, 1)
+    for m, n, k in ((208, 208, 80), (1024, 14336, 4096), (48, 112, 528)):
+        bm, bn, ks = bo.gemm_tiling(m, n, k)
+        assert m % bm == 0 and n % bn == 0 and k % (16 * ks) == 0
+
+
+def test_what_the_templates_do_not_take_is_said():
+    assert bo.unsupported("conv2d_0", [1, 8, 8, 16, 16, 3, 3, 1, 1]) is None
+    assert bo.unsupported("conv2d_0", [1, 8, 8, 16, 3, 3, 3, 1, 1]) is None
+    assert "groups of 16" in bo.unsupported("conv2d_0", [1, 8, 8, 16, 24, 3, 3, 1, 1])
+    assert "multiples of 16" in bo.unsupported("conv2d_0", [1, 8, 8, 20, 16, 3, 3, 1, 1])
+    assert "empty" in bo.unsupported("conv2d_0", [1, 2, 2, 16, 16, 5, 5, 1, 0])
+    assert "multiples of 16" in bo.unsupported("dense_0", [48, 100, 96])
+    assert bo.unsupported("bgemm_0", [7, 96, 48, 80]) is None          # the batch is not a matrix dimension
+    with pytest.raises(ValueError, match="dense_9"):
+        bo.registration("dense_9", [48, 100, 96])
+    with pytest.raises(ValueError):
+        bo.registration("pool_0", [1, 2, 3])
+
+
+def test_translation_unit_text():
+    ids = {"conv2d_0": [4, 20, 20, 32, 16, 3, 3, 1, 1], "conv2d_7": [4, 20, 20, 32, 16, 3, 3, 1, 1], "bgemm_0": [6, 96, 48, 80], "dense_0": [48, 160, 96]}
+    t = bo.source_text(ids)
+    assert t.count("BFUSE_KERNEL(") == 3                                  # two ids with the same arguments share a kernel
+    assert "using Op_conv3x3s1p1_f32_4x16x20x20_32 = ConvF32Auto<16, 32, 20, 20, 3, 3, 1, 1, 4>;" in t
+    assert "BFUSE_KERNEL(conv3x3s1p1_f32_4x16x20x20_32, Op_conv3x3s1p1_f32_4x16x20x20_32, ({{4, 16, 20, 20}, 4}), ({{32, 16, 3, 3}, 4}), ({{4, 32, 20, 20}, 4}))" in t
+    assert "GemmF32<96, 80, 48, 32, 80, 1, kEpiNone, 2, 1, true, 6>" in t and "({{6, 96, 48, 1}, 4}), ({{6, 80, 48, 1}, 4}), ({{6, 96, 80, 1}, 4})" in t
+    # dense: weight (out, in), the reference's layout -- the name says so and configure resolves dense ids to it
+    assert "using Op_gemm_f32_48x160x96_nk = GemmF32<48, 96, 160, 16, 96, 1, kEpiNone, 2, 1, true>;" in t
+    assert "({{48, 160, 1, 1}, 4}), ({{96, 160, 1, 1}, 4}), ({{48, 96, 1, 1}, 4})" in t
+    assert configure.candidate_names("dense_0", [48, 160, 96], None) == ["gemm_f32_48x160x96", "gemm_f32_48x160x96_nk"]
+    assert "BFUSE_MODULE_PROLOGUE()" in t and '#include "ops_conv_rect.h"' in t
+
+
+def test_written_without_compiling(tmp_path):
+    r = bo.build(str(tmp_path / "s"), {"bgemm_0": [6, 96, 48, 80]}, compile_=False)
+    assert r["kernels"] == {"bgemm_0": "bgemm_f32_6x96x48x80"} and r["module"] is None
+    assert os.path.exists(tmp_path / "s" / "hip" / "operators" / "pairs_operators.hip")
+    assert bo.rebuild_and_load(str(tmp_path / "none")) is None
+    bo.name_module(str(tmp_path / "s"), "hip/libbfuse_pairs.so")
+    bo.name_module(str(tmp_path / "s"), "hip/operators/libbfuse_pairs.so", first=True)
+    bo.name_module(str(tmp_path / "s"), "hip/libbfuse_pairs.so")
+    with open(tmp_path / "s" / "config" / "modules.yaml") as f:
+        assert yaml.safe_load(f) == ["hip/operators/libbfuse_pairs.so", "hip/libbfuse_pairs.so"]
+
+
+def test_missing_ids_are_refused_reported_or_built(tmp_path):
+    cfg = os.path.join(ROOT, "bfuse-project_amd", "examples", "new_shapes.yaml")
+    with pytest.raises(LookupError, match="conv2d_0"):
+        configure.configure(cfg, str(tmp_path / "a"))
+    assert not os.path.exists(tmp_path / "a")
+    bad = tmp_path / "bad.yaml"
+    bad.write_text(yaml.safe_dump({"FusionSet": [{"Set": ["dense_0"]}, {"Set": ["dense_1"]}], "KernelInfo": {"dense_0": [48, 100, 96], "dense_1": [512, 768, 768]}}))
+    with pytest.raises(ValueError, match="multiples of 16"):
+        configure.configure(str(bad), str(tmp_path / "b"), build_missing=True)
+    assert not os.path.exists(tmp_path / "b")
+    # the in-tree example as the build step configured and compiled it
+    built = os.path.join(ROOT, "bfuse-project_amd", "examples", "built", "new_shapes", "config")
+    if not os.path.exists(os.path.join(built, "info.yaml")):
+        pytest.skip("the build step has not run")
+    with open(os.path.join(built, "info.yaml")) as f:
+        info = yaml.safe_load(f)
+    assert info["FusionSet"][0]["Set"] == ["conv3x3s1p1_f32_4x16x20x20_32", "conv1x1s1p0_f32_24x32x12x12_48", "conv5x5s2p2_f32_2x3x70x70_16"]
+    assert info["FusionSet"][1]["Set"] == ["bgemm_f32_6x96x48x80", "gemm_f32_48x160x96_nk", "gemm_f32_512x768x768"]
+    with open(os.path.join(built, "modules.yaml")) as f:
+        assert yaml.safe_load(f) == ["hip/operators/libbfuse_pairs.so", "hip/libbfuse_pairs.so"]
