@@ -283,6 +283,19 @@ def measure(number, K, W, spec, ceilings, power_check=True):
         b_f, b_ser = float(np.median(q_f)), float(np.median(q_ser))
         b_k1 = op.time_batched("kernel1", warmup=BW, reps=R)
         b_k2 = op.time_batched("kernel2", warmup=BW, reps=R)
+        # The same three things replayed from a HIP graph (20 repetitions captured as one graph: the two kernels
+        # as dependent nodes / as independent nodes between a fork and a join / the fused kernel): what is left of
+        # each figure when the host's launch path is out of it.  The unfused pair as a graph is the strongest
+        # unfused baseline a caller has.
+        GC, GR = 20, max(3, R // 20)
+        for mode, f in ((kind, fused), ("serial", None), ("parallel", None)):
+            op.time_graph(mode, f, chain=GC, reps=1)
+        graph = {"chain": GC,
+                 "fused_us": round(float(np.median([op.time_graph(kind, fused, chain=GC, reps=GR) for _ in range(3)])), 3),
+                 "back_to_back_us": round(float(np.median([op.time_graph("serial", chain=GC, reps=GR) for _ in range(3)])), 3),
+                 "two_branches_us": round(float(np.median([op.time_graph("parallel", chain=GC, reps=GR) for _ in range(3)])), 3)}
+        graph["fused_over_back_to_back"] = round(graph["fused_us"] / graph["back_to_back_us"], 4)
+        graph["fused_over_best_unfused_graph"] = round(graph["fused_us"] / min(graph["back_to_back_us"], graph["two_branches_us"]), 4)
 
         # The same fused kernel over constant operands (every element of the contraction's two inputs = 1):
         # the same instructions and the same memory traffic, but no bits toggle in the matrix cores'
@@ -364,6 +377,7 @@ def measure(number, K, W, spec, ceilings, power_check=True):
         "batched_fused_over_back_to_back": round(b_f / b_ser, 4),
         "fused_over_back_to_back": round(b_f / b_ser, 4),
         "best_unfused": best,
+        "hip_graph": graph,
         "batched_rounds": {"fused_us": [round(x, 3) for x in q_f], "back_to_back_us": [round(x, 3) for x in q_ser]},
         "ms_per_step": round(wall_ms, 6),
         "baseline_reps": R,

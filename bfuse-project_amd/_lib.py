@@ -64,7 +64,7 @@ EXPORTS = [
     "run_kernel1", "run_kernel2", "run_parallel", "run_fuse",
     "bfuse_upload", "bfuse_zero_output", "bfuse_download", "bfuse_synchronize", "bfuse_launch",
     "bfuse_upload_part", "bfuse_download_part", "bfuse_checksum_output", "bfuse_fill_uniform_device",
-    "bfuse_time", "bfuse_time_batched", "bfuse_module_load", "bfuse_module_unload", "bfuse_module_launch",
+    "bfuse_time", "bfuse_time_batched", "bfuse_time_graph", "bfuse_module_load", "bfuse_module_unload", "bfuse_module_launch",
     "bfuse_initialize_side", "bfuse_finalize_side", "bfuse_launch_list", "bfuse_time_list",
     "bfuse_fill_uniform", "bfuse_fill_normal", "bfuse_f32_to_bf16", "bfuse_bf16_to_f32", "bfuse_check_matrix",
 ]
@@ -125,6 +125,7 @@ def lib():
         fp = C.POINTER(C.c_float)
         l.bfuse_time.argtypes = [C.c_int, vp, up, up, vp, up, up, C.c_int, C.c_int, fp, fp, fp]
         l.bfuse_time_batched.argtypes = [C.c_int, vp, up, up, vp, up, up, C.c_int, C.c_int, fp]
+        l.bfuse_time_graph.argtypes = [C.c_int, vp, up, up, vp, up, up, C.c_int, C.c_int, fp]
         l.bfuse_initialize_side.argtypes = [C.c_int, ip, ip, ip]
         l.bfuse_finalize_side.argtypes = [C.c_int]
         l.bfuse_launch_list.argtypes = [C.c_int, C.POINTER(LaunchDescC)]

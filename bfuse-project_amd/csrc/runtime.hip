@@ -1178,6 +1178,70 @@ int bfuse_time_batched(int mode, const void* fa, const unsigned* ga, const unsig
     return BFUSE_OK;
 }
 
+// One repetition of `mode` recorded into the capture that is open on s0 (s1: the second stream of mode 2).
+static int capture_mode(int mode, const void* fa, const unsigned* ga, const unsigned* ba, const void* fb,
+                        const unsigned* gb, const unsigned* bb, hipStream_t s0, hipStream_t s1, hipEvent_t fork, hipEvent_t join)
+{
+    int rc;
+    switch (mode) {
+        case BFUSE_MODE_KERNEL1: return launch3(fa, ga, ba, 0, s0);
+        case BFUSE_MODE_KERNEL2: return launch3(fa, ga, ba, 1, s0);
+        case BFUSE_MODE_SERIAL:
+            if ((rc = launch3(fa, ga, ba, 0, s0))) return rc;
+            return launch3(fb, gb, bb, 1, s0);
+        case BFUSE_MODE_PARALLEL:
+            HIP_TRY(hipEventRecord(fork, s0));
+            HIP_TRY(hipStreamWaitEvent(s1, fork, 0));
+            if ((rc = launch3(fa, ga, ba, 0, s0))) return rc;
+            if ((rc = launch3(fb, gb, bb, 1, s1))) return rc;
+            HIP_TRY(hipEventRecord(join, s1));
+            HIP_TRY(hipStreamWaitEvent(s0, join, 0));
+            return BFUSE_OK;
+        case BFUSE_MODE_HFUSE:
+        case BFUSE_MODE_BFUSE: return launch6(fa, ga, ba, s0);
+    }
+    return fail(BFUSE_ERR_ARG, "unknown mode %d", mode);
+}
+
+int bfuse_time_graph(int mode, const void* fa, const unsigned* ga, const unsigned* ba, const void* fb,
+                     const unsigned* gb, const unsigned* bb, int chain, int reps, float* us_per_repetition)
+{
+    int rc;
+    if (chain < 1 || chain > 1000 || reps < 1 || !us_per_repetition) return fail(BFUSE_ERR_ARG, "bad repetition count or null output");
+    if ((rc = validate_mode(mode, fa, ga, ba, fb, gb, bb))) return rc;
+    if ((rc = sync_and_check())) return rc;   // nothing of an earlier launch is pending when the capture starts
+    hipStream_t s0 = g.side[mode == BFUSE_MODE_KERNEL2 ? 1 : 0].stream, s1 = g.side[1].stream;   // the legacy stream cannot be captured
+    if (!s0 || (mode == BFUSE_MODE_PARALLEL && !s1)) return fail(BFUSE_ERR_STATE, "the side has no stream: initialize_kernel first");
+    EventList evl(4);
+    for (int i = 0; i < 2; ++i) HIP_TRY(hipEventCreateWithFlags(&evl.v[i], hipEventDisableTiming));   // fork, join
+    for (int i = 2; i < 4; ++i) HIP_TRY(hipEventCreate(&evl.v[i]));
+    struct Graph {
+        hipGraph_t g = nullptr;
+        hipGraphExec_t x = nullptr;
+        ~Graph()
+        {
+            if (x) (void)hipGraphExecDestroy(x);
+            if (g) (void)hipGraphDestroy(g);
+        }
+    } gr;
+    HIP_TRY(hipStreamBeginCapture(s0, hipStreamCaptureModeThreadLocal));
+    for (int c = 0; c < chain && rc == BFUSE_OK; ++c) rc = capture_mode(mode, fa, ga, ba, fb, gb, bb, s0, s1, evl.v[0], evl.v[1]);
+    const hipError_t ended = hipStreamEndCapture(s0, &gr.g);   // always: the stream must leave capture mode
+    if (rc) return rc;
+    HIP_TRY(ended);
+    HIP_TRY(hipGraphInstantiate(&gr.x, gr.g, nullptr, nullptr, 0));
+    HIP_TRY(hipGraphLaunch(gr.x, s0));
+    if ((rc = sync_and_check())) return rc;
+    HIP_TRY(hipEventRecord(evl.v[2], s0));
+    for (int r = 0; r < reps; ++r) HIP_TRY(hipGraphLaunch(gr.x, s0));
+    HIP_TRY(hipEventRecord(evl.v[3], s0));
+    if ((rc = sync_and_check())) return rc;
+    float ms = 0.f;
+    HIP_TRY(hipEventElapsedTime(&ms, evl.v[2], evl.v[3]));
+    *us_per_repetition = ms * 1000.f / ((float)reps * (float)chain);
+    return BFUSE_OK;
+}
+
 // ---- launch lists: any registered kernel over any sides -------------------------------------
 static int validate_list(int n, const bfuse_launch_desc* l)
 {

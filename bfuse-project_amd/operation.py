@@ -238,6 +238,14 @@ class Operation:
         _lib.check(self.l.bfuse_time_batched(MODES[mode], *self._mode_args(mode, fused), warmup, reps, C.byref(us)))
         return us.value
 
+    def time_graph(self, mode: str, fused: Optional[KernelHandle] = None, chain: int = 20, reps: int = 10) -> float:
+        """Mean microseconds per repetition of `mode` when `chain` repetitions are captured into one HIP graph and
+        the graph is replayed `reps` times ('serial': the two kernels as dependent nodes; 'parallel': as independent
+        nodes between a fork and a join)."""
+        us = C.c_float()
+        _lib.check(self.l.bfuse_time_graph(MODES[mode], *self._mode_args(mode, fused), chain, reps, C.byref(us)))
+        return us.value
+
 
 class GroupOperation:
     """Two to four sides for fusions of more than two kernels (the reference's fuser takes a list of

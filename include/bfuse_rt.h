@@ -272,6 +272,17 @@ int bfuse_time_batched(int mode, const void* func_a, const unsigned* grid_a, con
                        const void* func_b, const unsigned* grid_b, const unsigned* block_b, int warmup,
                        int reps, float* us_per_launch);
 
+/* The same measurement with the launches replayed from a HIP graph: `chain` repetitions of `mode` are captured
+ * once (mode 5: the two kernels as a chain of dependent nodes; mode 2: as two independent nodes between a fork
+ * and a join, repetition after repetition; modes 0, 1, 3, 4: one node per repetition), the graph is launched
+ * once untimed and `reps` times between two stream events; returns the mean microseconds per repetition of
+ * `mode`.  What it tells: how much of the back-to-back figure is the host's launch path -- the unfused pair as a
+ * graph is the strongest form of the baseline the reference's run_kernel1 + run_kernel2 stand for
+ * (operation_cu.py:128-197; the reference has no graph path).  Only kernel nodes are captured. */
+int bfuse_time_graph(int mode, const void* func_a, const unsigned* grid_a, const unsigned* block_a,
+                     const void* func_b, const unsigned* grid_b, const unsigned* block_b, int chain,
+                     int reps, float* us_per_repetition);
+
 /* ------------------------------------------------------------------------------------------
  * More than two kernels.  The reference's harness is two-sided (operation_h.py:9-27) while its
  * fuser takes a list of kernels of any length (horizontal-fuser/src/Algorithms.cc:23-35,540-566;
