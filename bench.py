@@ -288,14 +288,17 @@ def measure(number, K, W, spec, ceilings, power_check=True):
         # each figure when the host's launch path is out of it.  The unfused pair as a graph is the strongest
         # unfused baseline a caller has.
         GC, GR = 20, max(3, R // 20)
-        for mode, f in ((kind, fused), ("serial", None), ("parallel", None)):
-            op.time_graph(mode, f, chain=GC, reps=1)
-        graph = {"chain": GC,
-                 "fused_us": round(float(np.median([op.time_graph(kind, fused, chain=GC, reps=GR) for _ in range(3)])), 3),
-                 "back_to_back_us": round(float(np.median([op.time_graph("serial", chain=GC, reps=GR) for _ in range(3)])), 3),
-                 "two_branches_us": round(float(np.median([op.time_graph("parallel", chain=GC, reps=GR) for _ in range(3)])), 3)}
-        graph["fused_over_back_to_back"] = round(graph["fused_us"] / graph["back_to_back_us"], 4)
-        graph["fused_over_best_unfused_graph"] = round(graph["fused_us"] / min(graph["back_to_back_us"], graph["two_branches_us"]), 4)
+        try:
+            for mode, f in ((kind, fused), ("serial", None), ("parallel", None)):
+                op.time_graph(mode, f, chain=GC, reps=1)
+            graph = {"chain": GC,
+                     "fused_us": round(float(np.median([op.time_graph(kind, fused, chain=GC, reps=GR) for _ in range(3)])), 3),
+                     "back_to_back_us": round(float(np.median([op.time_graph("serial", chain=GC, reps=GR) for _ in range(3)])), 3),
+                     "two_branches_us": round(float(np.median([op.time_graph("parallel", chain=GC, reps=GR) for _ in range(3)])), 3)}
+            graph["fused_over_back_to_back"] = round(graph["fused_us"] / graph["back_to_back_us"], 4)
+            graph["fused_over_best_unfused_graph"] = round(graph["fused_us"] / min(graph["back_to_back_us"], graph["two_branches_us"]), 4)
+        except bf._lib.BfuseError as e:      # refused under rocprofv3 (its tracing does not survive graph launches)
+            graph = {"skipped": str(e)}
 
         # The same fused kernel over constant operands (every element of the contraction's two inputs = 1):
         # the same instructions and the same memory traffic, but no bits toggle in the matrix cores'

@@ -1209,6 +1209,14 @@ int bfuse_time_graph(int mode, const void* fa, const unsigned* ga, const unsigne
     int rc;
     if (chain < 1 || chain > 1000 || reps < 1 || !us_per_repetition) return fail(BFUSE_ERR_ARG, "bad repetition count or null output");
     if ((rc = validate_mode(mode, fa, ga, ba, fb, gb, bb))) return rc;
+    // rocprofv3's kernel tracing takes a segmentation fault in its own code on the first graph launch here
+    // (ROCm 7.2): refused with a message instead
+    {
+        const char* pre = getenv("LD_PRELOAD");
+        const char* tool = getenv("ROCP_TOOL_LIBRARIES");
+        if ((pre && strstr(pre, "rocprofiler")) || (tool && *tool))
+            return fail(BFUSE_ERR_STATE, "graph replays are not timed under rocprofv3: its tracing does not survive a graph launch on this ROCm");
+    }
     if ((rc = sync_and_check())) return rc;   // nothing of an earlier launch is pending when the capture starts
     hipStream_t s0 = g.side[mode == BFUSE_MODE_KERNEL2 ? 1 : 0].stream, s1 = g.side[1].stream;   // the legacy stream cannot be captured
     if (!s0 || (mode == BFUSE_MODE_PARALLEL && !s1)) return fail(BFUSE_ERR_STATE, "the side has no stream: initialize_kernel first");

@@ -278,7 +278,8 @@ int bfuse_time_batched(int mode, const void* func_a, const unsigned* grid_a, con
  * once untimed and `reps` times between two stream events; returns the mean microseconds per repetition of
  * `mode`.  What it tells: how much of the back-to-back figure is the host's launch path -- the unfused pair as a
  * graph is the strongest form of the baseline the reference's run_kernel1 + run_kernel2 stand for
- * (operation_cu.py:128-197; the reference has no graph path).  Only kernel nodes are captured. */
+ * (operation_cu.py:128-197; the reference has no graph path).  Only kernel nodes are captured.  Under rocprofv3
+ * (whose kernel tracing crashes on a graph launch on ROCm 7.2) the call is refused with BFUSE_ERR_STATE. */
 int bfuse_time_graph(int mode, const void* func_a, const unsigned* grid_a, const unsigned* block_a,
                      const void* func_b, const unsigned* grid_b, const unsigned* block_b, int chain,
                      int reps, float* us_per_repetition);
