@@ -224,4 +224,26 @@ __device__ __forceinline__ T* opaque_pointer(T* p)
     return (T*)(__attribute__((address_space(1))) T*)bits;
 }
 
+// An operator with BYTES more of LDS per workgroup than it uses: bounds how many of its workgroups are resident
+// on a CU (160 KB / (BYTES + its own)).  The one-wave batched products run best at one wave per SIMD -- every wave
+// streams its operands straight into registers, and the two or three waves per SIMD their registers allow only
+// queue behind each other in the memory pipeline: with 32 KB reserved (four workgroups per CU) the 1024-fold
+// products with 64 x 64 tiles took 461 / 703 / 124 / 147 us instead of 561 / 937 / 131 / 166, and 208 x 208 x 64
+// with 208 x 32 tiles 75 us instead of 94 (24 KB, six per CU: 119; 40 KB, three per CU: 92).  The one-wave
+// convolutions on three input channels want about three waves per SIMD (the 7 x 7 on RGB at batch 1024: 3.53 ms
+// with twelve workgroups per CU, 4.43 with the sixteen its registers allow, 4.2 with six).
+template <class Op, int BYTES>
+struct LdsReserve : Op {
+    struct Smem {
+        typename Op::Smem s;
+        unsigned char reserve[BYTES];
+    };
+    template <class Sync>
+    __device__ static __forceinline__ void run(int vblock, int tid, Smem& sm, const void* I, const void* F, void* O, Sync sync)
+    {
+        if (vblock < 0) sm.reserve[tid] = 1;   // never true (workgroup ids are not negative): keeps the reservation allocated
+        Op::run(vblock, tid, sm.s, I, F, O, sync);
+    }
+};
+
 }  // namespace bfuse
