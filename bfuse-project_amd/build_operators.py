@@ -36,9 +36,14 @@ HEADERS = ("fuse.h", "ops_conv_rect.h", "ops_gemm_f32.h")
 
 def gemm_tiling(m: int, n: int, k: int) -> Tuple[int, int, int]:
     """(BM, BN, KS) of GemmF32 for an m x n x k product: 64 rows (else 32, 16) by 64 columns (else 96, 80, 48, 32,
-    16), whichever divides it first, and two or four waves over K when K is long."""
+    16), whichever divides it first -- but 64 where only 16 would divide a dimension above 64 (208 = 13 x 16: the
+    last tile then overlaps its neighbour, which GemmF32 allows) -- and two or four waves over K when K is long."""
     bm = next(t for t in (64, 32, 16) if m % t == 0)
     bn = next(t for t in (64, 96, 80, 48, 32, 16) if n % t == 0)
+    if bm == 16 and m > 64:
+        bm = 64
+    if bn == 16 and n > 64:
+        bn = 64
     ks = 4 if k >= 2048 and k % 64 == 0 else 2 if k >= 512 and k % 32 == 0 else 1
     return bm, bn, ks
 

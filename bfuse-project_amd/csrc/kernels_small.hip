@@ -50,6 +50,8 @@ using SyncProbeB = SyncProbe<6, 1>;
 using GemmS1 = GemmF32<64, 48, 32, 16, 48, 1>;                        // one wave, a 32- and a 16-column group
 using GemmS2 = GemmF32<96, 192, 128, 32, 64, 2, kEpiGeluTanh, 3>;     // 2 waves, GELU, 3 register stages
 using GemmS3 = GemmF32<32, 144, 256, 32, 144, 4>;                     // the 64+64+16 column split, one tile
+using GemmS7 = GemmF32<80, 112, 32, 32, 64, 1>;                        // tiles that do not divide the problem: rows 0, 32, 48 and columns 0, 48 (the last tiles overlap their neighbours)
+using GemmS8 = GemmF32<48, 80, 64, 32, 64, 2, kEpiNone, 2, 1, true, 3>;   // the same on three batched products with B [N, K] and two waves over K
 using GemmS5 = GemmF32Dma<128, 192, 160, 32, 96, 2>;                  // private LDS rings, two waves split K, ten 8-k stages each
 using GemmS6 = GemmF32Dma<64, 288, 192, 32, 144, 4, kEpiGeluTanh>;    // the 32x144 tile (partial last B load), four waves, GELU
 using BiasReluS = BiasRelu<4096, 64, 4>;
@@ -74,6 +76,8 @@ using NormRopeS = RmsNormRope<6, 8, 128, 2>;
 BFUSE_KERNEL(gemm_f32_64x32x48, GemmS1, ({{64, 32, 1, 1}, 4}), ({{32, 48, 1, 1}, 4}), ({{64, 48, 1, 1}, 4}))
 BFUSE_KERNEL(gemm_gelu_f32_96x128x192, GemmS2, ({{96, 128, 1, 1}, 4}), ({{128, 192, 1, 1}, 4}), ({{96, 192, 1, 1}, 4}))
 BFUSE_KERNEL(gemm_f32_32x256x144, GemmS3, ({{32, 256, 1, 1}, 4}), ({{256, 144, 1, 1}, 4}), ({{32, 144, 1, 1}, 4}))
+BFUSE_KERNEL(gemm_f32_80x32x112, GemmS7, ({{80, 32, 1, 1}, 4}), ({{32, 112, 1, 1}, 4}), ({{80, 112, 1, 1}, 4}))
+BFUSE_KERNEL(bgemm_f32_3x48x64x80, GemmS8, ({{3, 48, 64, 1}, 4}), ({{3, 80, 64, 1}, 4}), ({{3, 48, 80, 1}, 4}))
 BFUSE_KERNEL(gemm_f32_128x160x192_d, GemmS5, ({{128, 160, 1, 1}, 4}), ({{160, 192, 1, 1}, 4}), ({{128, 192, 1, 1}, 4}))
 BFUSE_KERNEL(gemm_gelu_f32_64x192x288_d, GemmS6, ({{64, 192, 1, 1}, 4}), ({{192, 288, 1, 1}, 4}), ({{64, 288, 1, 1}, 4}))
 BFUSE_KERNEL(bias_relu_4096, BiasReluS, ({{4096, 1, 1, 1}, 4}), ({{4096, 1, 1, 1}, 4}), ({{4096, 1, 1, 1}, 4}))
@@ -147,6 +151,9 @@ BFUSE_BFUSE_KERNEL(conv1x1s1p0_f32_3x32x5x5_32, Conv1S1, layernorm_8x256, LayerN
 BFUSE_HFUSE_KERNEL(conv1x1s1p0_f32_5x96x9x9_48, Conv1S2, bias_relu_4096, BiasReluS)
 BFUSE_HFUSE_KERNEL(conv1x1s1p0_f32_5x96x9x9_48, Conv1S2, conv3x3_f32_32x12x12_32, ConvS2)
 BFUSE_BFUSE_KERNEL(conv1x1s2p0_f32_2x16x9x7_16, Conv1S3, bias_relu_4096, BiasReluS, , bfuse::kZigzag, 1, 1)
+// overlapping last tiles: the shared elements are written twice with the same bits, also inside fused kernels
+BFUSE_BFUSE_KERNEL(gemm_f32_80x32x112, GemmS7, layernorm_8x256, LayerNormS, , bfuse::kZigzag, 1, 1)
+BFUSE_HFUSE_KERNEL(bgemm_f32_3x48x64x80, GemmS8, bias_relu_4096, BiasReluS)
 // the give-up path of the side barrier, forced from the host with a small spin limit
 BFUSE_KERNEL(selftest_sync_a, SyncProbeA, ({{512, 1, 1, 1}, 4}), ({{512, 1, 1, 1}, 4}), ({{512, 1, 1, 1}, 4}))
 BFUSE_KERNEL(selftest_sync_b, SyncProbeB, ({{768, 1, 1, 1}, 4}), ({{768, 1, 1, 1}, 4}), ({{768, 1, 1, 1}, 4}))

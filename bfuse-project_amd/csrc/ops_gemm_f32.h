@@ -71,13 +71,17 @@ struct GemmF32 {
     static constexpr int STAGE = 16;            // k per stage (one 128-bit A load)
     static constexpr int NSTAGE = KW / STAGE;
     static constexpr int NBUF = NBUF_;          // register stages in flight (>= 2)
-    static_assert(M % BM == 0 && N % BN == 0, "tile must divide the problem");
+    // A tile that does not divide the problem: the last row (column) tile starts BM rows (BN columns) before the
+    // end instead of running past it.  It overlaps its neighbour, and both write the same bits to what they
+    // share: an element of the product is the same sequence of multiply-adds over k in every tile.
+    static constexpr int MT = (M + BM - 1) / BM, NT = (N + BN - 1) / BN;   // row and column tiles
+    static_assert(M >= BM && N >= BN && M % 4 == 0, "a tile is not larger than the problem");
     static_assert(BM % 16 == 0 && BN % 16 == 0 && K % (KS * STAGE) == 0, "shape/tile mismatch");
     static_assert(N % 4 == 0 && K % 4 == 0, "rows must be 16-byte aligned");
     static_assert(NSTAGE >= NBUF - 1, "k-range shorter than the prefetch depth");
 
-    static constexpr int TILES = (N / BN) * (M / BM);
-    static constexpr Dims3 GRID{N / BN, M / BM, BATCH};
+    static constexpr int TILES = NT * MT;
+    static constexpr Dims3 GRID{NT, MT, BATCH};
     static constexpr Dims3 BLOCK{64 * KS, 1, 1};
     static constexpr int THREADS = 64 * KS;
     static constexpr bool HAS_BARRIERS = KS > 1;
@@ -240,9 +244,10 @@ struct GemmF32 {
         const float* __restrict__ A = static_cast<const float*>(I) + (size_t)batch * M * K;
         const float* __restrict__ B = static_cast<const float*>(F) + (size_t)batch * K * N;
         float* __restrict__ C = static_cast<float*>(O) + (size_t)batch * M * N;
-        const Dims3 vb = PRODUCT_PER_XCD ? Dims3{vblock % (N / BN), vblock / (N / BN), 0}
-                                         : XcdTiles<N / BN, M / BM, BM, BN>::tile(BATCH > 1 ? vblock % TILES : vblock);   // tiles dealt so that each XCD's L2 fetches as little as possible
-        const int m0 = vb.y * BM, n0 = vb.x * BN;
+        const Dims3 vb = PRODUCT_PER_XCD ? Dims3{vblock % NT, vblock / NT, 0}
+                                         : XcdTiles<NT, MT, BM, BN>::tile(BATCH > 1 ? vblock % TILES : vblock);   // tiles dealt so that each XCD's L2 fetches as little as possible
+        const int m0 = (M % BM != 0 && (int)vb.y == MT - 1) ? M - BM : vb.y * BM;
+        const int n0 = (N % BN != 0 && (int)vb.x == NT - 1) ? N - BN : vb.x * BN;
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;   // wave-uniform: addresses built on it stay in scalar registers
         const int kbeg = wave * KW;
 

@@ -18,9 +18,12 @@ def test_default_gemm_tiling_divides_the_problem():
     assert bo.gemm_tiling(512, 512, 512) == (64, 64, 2)
     assert bo.gemm_tiling(1024, 4096, 4096) == (64, 64, 4)
     assert bo.gemm_tiling(16, 16, 16) == (16, 16, 1)
-    for m, n, k in ((208, 208, 80), (1024, 14336, 4096), (48, 112, 528)):
+    assert bo.gemm_tiling(208, 80, 208) == (64, 80, 1)       # 208 = 13 x 16: 64-row tiles, the last one overlapping
+    assert bo.gemm_tiling(208, 208, 80) == (64, 64, 1)
+    assert bo.gemm_tiling(48, 112, 528) == (16, 64, 1)
+    for m, n, k in ((208, 208, 80), (1024, 14336, 4096), (48, 112, 528), (16, 272, 64)):
         bm, bn, ks = bo.gemm_tiling(m, n, k)
-        assert m % bm == 0 and n % bn == 0 and k % (16 * ks) == 0
+        assert bm <= m and bn <= n and bm % 16 == 0 and bn % 16 == 0 and k % (16 * ks) == 0
 
 
 def test_what_the_templates_do_not_take_is_said():

@@ -35,6 +35,10 @@ def _cases():
     return {
         "gemm_f32_64x32x48": (lambda s: (fill_uniform(s, 64 * 32, -1, 1), fill_uniform(s + 1, 32 * 48, -1, 1)),
                               lambda I, F: orf.gemm_f32(I.reshape(64, 32), F.reshape(32, 48)), 1e-5, False),
+        "gemm_f32_80x32x112": (lambda s: (fill_uniform(s, 80 * 32, -1, 1), fill_uniform(s + 1, 32 * 112, -1, 1)),
+                               lambda I, F: orf.gemm_f32(I.reshape(80, 32), F.reshape(32, 112)), 1e-5, False),
+        "bgemm_f32_3x48x64x80": (lambda s: (fill_uniform(s, 3 * 48 * 64, -1, 1), fill_uniform(s + 1, 3 * 80 * 64, -1, 1)),
+                                 lambda I, F: np.stack([orf.gemm_f32(I.reshape(3, 48, 64)[b], F.reshape(3, 80, 64)[b], b_is_nk=True) for b in range(3)]), 1e-5, False),
         "gemm_gelu_f32_96x128x192": (lambda s: (fill_normal(s, 96 * 128, 0, 1), fill_normal(s + 1, 128 * 192, 0, 0.1)),
                                      lambda I, F: orf.gemm_f32(I.reshape(96, 128), F.reshape(128, 192), epilogue=1), 1e-5, False),
         "gemm_f32_32x256x144": (lambda s: (fill_normal(s, 32 * 256, 0, 1), fill_normal(s + 1, 256 * 144, 0, 0.05)),
@@ -103,6 +107,8 @@ FUSIONS = [
     ("conv1x1s1p0_f32_5x96x9x9_48", "bias_relu_4096", "hfuse", ""),                # a barrier per filter chunk beside a side without any: LDS arrival counters
     ("conv1x1s1p0_f32_5x96x9x9_48", "conv3x3_f32_32x12x12_32", "hfuse", ""),       # both sides synchronise
     ("conv1x1s2p0_f32_2x16x9x7_16", "bias_relu_4096", "bfuse", ""),
+    ("gemm_f32_80x32x112", "layernorm_8x256", "bfuse", ""),                        # GEMM tiles that overlap (80 = 32 + 32 + 16 rows)
+    ("bgemm_f32_3x48x64x80", "bias_relu_4096", "hfuse", ""),
 ]
 
 
