@@ -75,7 +75,7 @@ struct GemmF32 {
     // end instead of running past it.  It overlaps its neighbour, and both write the same bits to what they
     // share: an element of the product is the same sequence of multiply-adds over k in every tile.
     static constexpr int MT = (M + BM - 1) / BM, NT = (N + BN - 1) / BN;   // row and column tiles
-    static_assert(M >= BM && N >= BN && M % 4 == 0, "a tile is not larger than the problem");
+    static_assert(M >= BM && N >= BN, "a tile is not larger than the problem");
     static_assert(BM % 16 == 0 && BN % 16 == 0 && K % (KS * STAGE) == 0, "shape/tile mismatch");
     static_assert(N % 4 == 0 && K % 4 == 0, "rows must be 16-byte aligned");
     static_assert(NSTAGE >= NBUF - 1, "k-range shorter than the prefetch depth");
