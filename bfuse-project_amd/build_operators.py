@@ -16,8 +16,10 @@ library's flags and build checks, into a kernel module of their own, `<suite>/hi
 from the suite's fused kernels.  `configure --build-missing` calls it; the suite, the quick start and the
 `benchmark` driver find the new operators by name once the module is loaded.
 
-What the templates take: matrix dimensions that are multiples of 16; input channels in groups of 16 (or at most
-4) and output channels in multiples of 16.  An id outside that is reported with the reason.
+What the templates take: products of at least 16 rows and 16 columns, columns in multiples of 4 and a contracted
+dimension in multiples of 16 (tiles need not divide rows or columns: the last tile overlaps its neighbour); input
+channels in groups of 16 (or at most 4) and output channels in multiples of 16.  An id outside that is reported
+with the reason.
 """
 import os
 import subprocess
@@ -34,18 +36,21 @@ UNIT = "pairs_operators.hip"
 HEADERS = ("fuse.h", "ops_conv_rect.h", "ops_gemm_f32.h")
 
 
+def _tile(d: int, divisors: Sequence[int]) -> int:
+    """A tile extent for a dimension of d: the first of `divisors` that divides it; where none does, or only 16
+    divides a dimension above 64 (208 = 13 x 16), the largest of 64, 32, 16 that fits -- the last tile then
+    overlaps its neighbour, which GemmF32 allows."""
+    t = next((c for c in divisors if d % c == 0), None)
+    if t is None or (t == 16 and d > 64):
+        t = next(c for c in (64, 32, 16) if c <= d)
+    return t
+
+
 def gemm_tiling(m: int, n: int, k: int) -> Tuple[int, int, int]:
     """(BM, BN, KS) of GemmF32 for an m x n x k product: 64 rows (else 32, 16) by 64 columns (else 96, 80, 48, 32,
-    16), whichever divides it first -- but 64 where only 16 would divide a dimension above 64 (208 = 13 x 16: the
-    last tile then overlaps its neighbour, which GemmF32 allows) -- and two or four waves over K when K is long."""
-    bm = next(t for t in (64, 32, 16) if m % t == 0)
-    bn = next(t for t in (64, 96, 80, 48, 32, 16) if n % t == 0)
-    if bm == 16 and m > 64:
-        bm = 64
-    if bn == 16 and n > 64:
-        bn = 64
+    16), and two or four waves over K when K is long."""
     ks = 4 if k >= 2048 and k % 64 == 0 else 2 if k >= 512 and k % 32 == 0 else 1
-    return bm, bn, ks
+    return _tile(m, (64, 32, 16)), _tile(n, (64, 96, 80, 48, 32, 16)), ks
 
 
 def unsupported(kernel_id: str, args) -> Optional[str]:
@@ -61,11 +66,15 @@ def unsupported(kernel_id: str, args) -> Optional[str]:
         if min(n, h, w, co, ci, kh, kw) < 1 or (h - kh + 2 * pad) < 0 or (w - kw + 2 * pad) < 0:
             return "empty operand or result"
         return None
-    dims = args[1:] if op == "bgemm" else args
     if min(args) < 1:
         return "empty operand or result"
-    if any(d % 16 for d in dims):
-        return "matrix dimensions come in multiples of 16"
+    m, k, n = (args[1], args[2], args[3]) if op == "bgemm" else (args[0], args[1], args[2])
+    if m < 16 or n < 16:
+        return "a matrix product has at least 16 rows and 16 columns (one MFMA block)"
+    if n % 4 != 0:
+        return "output rows are whole 16-byte chunks: columns in multiples of 4"
+    if k % 16 != 0:
+        return "the contracted dimension comes in multiples of 16"
     return None
 
 

@@ -32,7 +32,11 @@ def test_what_the_templates_do_not_take_is_said():
     assert "groups of 16" in bo.unsupported("conv2d_0", [1, 8, 8, 16, 24, 3, 3, 1, 1])
     assert "multiples of 16" in bo.unsupported("conv2d_0", [1, 8, 8, 20, 16, 3, 3, 1, 1])
     assert "empty" in bo.unsupported("conv2d_0", [1, 2, 2, 16, 16, 5, 5, 1, 0])
-    assert "multiples of 16" in bo.unsupported("dense_0", [48, 100, 96])
+    assert "multiples of 16" in bo.unsupported("dense_0", [48, 100, 96])       # the contracted dimension
+    assert bo.unsupported("dense_0", [50, 96, 100]) is None                     # rows and columns need no tile that divides them
+    assert "multiples of 4" in bo.unsupported("dense_0", [48, 96, 98])
+    assert "at least 16" in bo.unsupported("dense_0", [1, 96, 96])
+    assert bo.gemm_tiling(100, 72, 32) == (64, 64, 1) and bo.gemm_tiling(50, 100, 96) == (32, 64, 1) and bo.gemm_tiling(20, 20, 16) == (16, 16, 1)
     assert bo.unsupported("bgemm_0", [7, 96, 48, 80]) is None          # the batch is not a matrix dimension
     with pytest.raises(ValueError, match="dense_9"):
         bo.registration("dense_9", [48, 100, 96])
@@ -83,6 +87,6 @@ def test_missing_ids_are_refused_reported_or_built(tmp_path):
     with open(os.path.join(built, "info.yaml")) as f:
         info = yaml.safe_load(f)
     assert info["FusionSet"][0]["Set"] == ["conv3x3s1p1_f32_4x16x20x20_32", "conv1x1s1p0_f32_24x32x12x12_48", "conv5x5s2p2_f32_2x3x70x70_16"]
-    assert info["FusionSet"][1]["Set"] == ["bgemm_f32_6x96x48x80", "gemm_f32_48x160x96_nk", "gemm_f32_512x768x768"]
+    assert info["FusionSet"][1]["Set"] == ["bgemm_f32_6x96x48x80", "bgemm_f32_5x100x32x72", "gemm_f32_48x160x96_nk", "gemm_f32_512x768x768"]
     with open(os.path.join(built, "modules.yaml")) as f:
         assert yaml.safe_load(f) == ["hip/operators/libbfuse_pairs.so", "hip/libbfuse_pairs.so"]
