@@ -12,7 +12,8 @@
   [5/6] profile the benchmark                      [2/3] `suite`: every pair in every mode, validated, traces under OUT/exec
                                                    (--resident: operands written and outputs compared on the device, for
                                                    operators at batch 1024 whose tensors run to GB)
-  [6/6] draw profile results                       [3/3] speed-up table: OUT/summary.md, OUT/summary.json
+  [6/6] draw profile results                       [3/3] speed-up table: OUT/summary.md, OUT/summary.json; the reference's speed-up
+                                                   figure: OUT/exec_figure.png
 """
 import argparse
 import json
@@ -65,6 +66,10 @@ def main(argv=None) -> int:
     with open(os.path.join(args.file, "summary.md"), "w") as f:
         f.write(md)
     print(md)
+    try:      # the reference's [6/6]: its speed-up figure (profile/exec_figure.png)
+        print(suite.draw_speedup_figure(rows, os.path.join(args.file, "exec_figure.png")))
+    except ImportError:
+        pass
     return 0
 
 

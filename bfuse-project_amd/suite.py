@@ -457,6 +457,54 @@ def to_markdown(rows: Sequence[dict]) -> str:
     return head + body + tail + "\n"
 
 
+def speedup_statistics(rows: Sequence[dict]) -> Dict[str, dict]:
+    """max, min, geometric mean and standard deviation of every form's speed-up over serial: the block the reference
+    prints under its figure (scripts/analyze_test_suite.py:1203-1209), plus the chooser's form."""
+    out = {}
+    for k in ("parallel", "hfuse", "bfuse", "chooser"):
+        v = [r[k + "_speedup"] for r in rows if k + "_speedup" in r]
+        if v:
+            out[k] = {"pairs": len(v), "max": float(np.max(v)), "min": float(np.min(v)), "avg": geomean(v), "std": float(np.std(v))}
+    return out
+
+
+def draw_speedup_figure(rows: Sequence[dict], path: str, per_row: int = 21) -> str:
+    """The reference's speed-up figure (scripts/analyze_test_suite.py:1134-1201, its `exec_figure.png`): one group of bars
+    per pair -- two streams, thread-level fusion, block fusion, and here also the chooser's form -- 21 pairs to a row of
+    the figure, the serial baseline dashed at 1, the y axis 0 .. 2, and the geometric means after the last pair."""
+    import math
+    import matplotlib
+    matplotlib.use("Agg")
+    import matplotlib.pyplot as plt
+    forms = [k for k in ("parallel", "hfuse", "bfuse", "chooser") if any(k + "_speedup" in r for r in rows)]
+    n, width = len(rows), 0.8 / max(len(forms), 1)
+    n_rows = max(1, math.ceil(n / per_row))
+    fig, axes = plt.subplots(n_rows, 1, figsize=(10, 1.6 * n_rows + 0.6), squeeze=False)
+    for a in range(n_rows):
+        ax = axes[a][0]
+        lo, hi = a * per_row, min(n, (a + 1) * per_row)
+        x = np.arange(hi - lo)
+        for f, k in enumerate(forms):
+            ax.bar(x + (f - (len(forms) - 1) / 2) * width, [rows[i].get(k + "_speedup", 0.0) for i in range(lo, hi)], width=width, label=k)
+        ax.axhline(y=1, color="r", linewidth=0.5, linestyle="--")
+        ax.set_ylim(0, 2)
+        ax.set_ylabel("Speed up", fontsize=6)
+        ax.tick_params(axis="both", labelsize=5)
+        ax.set_xticks(x)
+        ax.set_xticklabels([str(i) for i in range(lo, hi)])
+        if a == n_rows - 1:       # the geometric means, one slot to the right of the last pair
+            ax.axvline(x=x[-1] + 1, color="gray", linewidth=0.5, linestyle="--")
+            for f, k in enumerate(forms):
+                ax.bar([x[-1] + 2 + (f - (len(forms) - 1) / 2) * width], [geomean([r.get(k + "_speedup") for r in rows])], width=width,
+                       color=f"C{f}")
+        if a == 0:
+            ax.legend(ncol=len(forms), loc="upper left", fontsize=5)
+    fig.tight_layout()
+    fig.savefig(path, dpi=200)
+    plt.close(fig)
+    return path
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
     ap.add_argument("file", help="info.yaml with the two fusion sets")
@@ -467,6 +515,7 @@ def main(argv=None) -> int:
     ap.add_argument("--no-validate", action="store_true")
     ap.add_argument("--rows", metavar="LO:HI", help="run only the pairs whose first operator is LO <= i < HI of the first set")
     ap.add_argument("--resident", action="store_true", help="operands written and results compared on the device (operators at batch 1024)")
+    ap.add_argument("--figure", action="store_true", help="also draw OUT/exec_figure.png, the reference's speed-up figure, and print its statistics")
     ap.add_argument("--benchmark", default=os.path.join(os.path.dirname(os.path.abspath(__file__)), "benchmark"))
     args = ap.parse_args(argv)
     try:
@@ -497,6 +546,12 @@ def main(argv=None) -> int:
     with open(os.path.join(args.out, "summary.md"), "w") as f:
         f.write(md)
     print(md)
+    if args.figure:
+        print("==== EXEC_FIGURE ====\n---------------------------------------")
+        for k, st in speedup_statistics(rows).items():
+            print(f"{k:8s} | max: {st['max']}, min: {st['min']}, avg: {st['avg']}, std: {st['std']}")
+        print("---------------------------------------")
+        print(draw_speedup_figure(rows, os.path.join(args.out, "exec_figure.png")))
     return 0
 
 

@@ -61,6 +61,8 @@ def test_quick_start_command(tmp_path):
     assert r.returncode == 0, r.stdout[-1500:] + r.stderr[-1500:]
     assert "[1/3]" in r.stdout and "[3/3]" in r.stdout and "gemm_f32_512x768x2304" in r.stdout
     assert os.path.exists(out / "summary.md") and os.path.exists(out / "config" / "kernels.yaml") and os.path.exists(out / "exec" / "2_0_0.csv")
+    with open(out / "exec_figure.png", "rb") as f:      # the reference's [6/6]: its speed-up figure
+        assert f.read(4) == b"\x89PNG"
     # a second run into the same directory is refused, as the reference's configure step refuses it
     r = subprocess.run([sys.executable, "-m", "bfuse_project_amd.quick_start", str(cfg), "-o", str(out)], capture_output=True, text=True, cwd=root, timeout=120)
     assert r.returncode == 1 and "already exists" in r.stderr

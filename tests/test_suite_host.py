@@ -198,3 +198,22 @@ def test_numeric_ids_without_an_info_file_are_an_error_and_names_keep_working(tm
     one.write_text("FusionSet:\n- Set:\n  - bias_relu_4096\n")
     r, _ = _dry(["-i", str(one), "0", "0", "0"], cwd=str(tmp_path))
     assert r.returncode != 0 and "only 2" in r.stderr
+
+
+def test_speedup_statistics_and_figure(tmp_path):
+    """The block the reference prints under its speed-up figure (scripts/analyze_test_suite.py:1203-1209: max, min,
+    geometric mean, standard deviation per form) and the figure itself, over rows written down here."""
+    import json
+    rows = [{"kernel1": "a", "kernel2": "b", "parallel_speedup": 1.0, "hfuse_speedup": 0.5, "bfuse_speedup": 2.0, "chooser_speedup": 2.0},
+            {"kernel1": "a", "kernel2": "c", "parallel_speedup": 1.21, "bfuse_speedup": 0.5, "chooser_speedup": 1.0}]
+    rows += [{"kernel1": "x", "kernel2": str(i), "parallel_speedup": 1.0, "bfuse_speedup": 1.0, "chooser_speedup": 1.0} for i in range(25)]
+    st = suite.speedup_statistics(rows)
+    assert st["hfuse"] == {"pairs": 1, "max": 0.5, "min": 0.5, "avg": 0.5, "std": 0.0}
+    assert st["bfuse"]["pairs"] == 27 and st["bfuse"]["max"] == 2.0 and st["bfuse"]["min"] == 0.5
+    assert st["bfuse"]["avg"] == pytest.approx(1.0)                      # 2 x 0.5 x 1 ... = 1
+    assert st["parallel"]["avg"] == pytest.approx(1.21 ** (1 / 27))
+    assert st["chooser"]["avg"] == pytest.approx(2.0 ** (1 / 27)) and "serial" not in st
+    path = suite.draw_speedup_figure(rows, str(tmp_path / "exec_figure.png"))      # 27 pairs: two rows of the figure
+    with open(path, "rb") as f:
+        assert f.read(8) == b"\x89PNG\r\n\x1a\n"
+    assert suite.speedup_statistics([]) == {}
