@@ -485,8 +485,25 @@ KernelEntry make_fused_entry(const char* name, const void* func, int kind, const
     }                                                                                               \
     static const bfuse::ModuleHooks bfuse_module_hooks{&bfuse_module_read_sync_timeouts, &bfuse_module_set_spin_limit};
 
+namespace bfuse {
+// The waves per SIMD a kernel is compiled for (the register budget of its waves: 512 / waves): kMinWavesPerEu,
+// unless one of its operators says that it needs more of the register file (MIN_WAVES_PER_EU).  A fused kernel
+// takes the smallest of its sides': it holds the registers of the side that needs most.
+template <class Op, class = void>
+struct min_waves_of : std::integral_constant<int, kMinWavesPerEu> {};
+template <class Op>
+struct min_waves_of<Op, std::void_t<decltype(Op::MIN_WAVES_PER_EU)>> : std::integral_constant<int, Op::MIN_WAVES_PER_EU> {};
+template <class... Ops>
+constexpr int min_waves()
+{
+    int m = kMinWavesPerEu;
+    ((m = min_waves_of<Ops>::value < m ? min_waves_of<Ops>::value : m), ...);
+    return m;
+}
+}  // namespace bfuse
+
 #define BFUSE_KERNEL(NAME, OP, IDESC, FDESC, ODESC)                                                  \
-    extern "C" __global__ __launch_bounds__(OP::THREADS, bfuse::kMinWavesPerEu) void NAME(const void* __restrict__ I,       \
+    extern "C" __global__ __launch_bounds__(OP::THREADS, bfuse::min_waves<OP>()) void NAME(const void* __restrict__ I,       \
                                                                    const void* __restrict__ F,       \
                                                                    void* __restrict__ O)             \
     {                                                                                               \
@@ -497,7 +514,7 @@ KernelEntry make_fused_entry(const char* name, const void* func, int kind, const
         bfuse_module_hooks));
 
 #define BFUSE_BFUSE_KERNEL(K1, OP1, K2, OP2, SUFFIX, PATTERN, P0, P1)                                \
-    extern "C" __global__ __launch_bounds__((bfuse::BfusePair<OP1, OP2, PATTERN, P0, P1>::THREADS), bfuse::kMinWavesPerEu)  \
+    extern "C" __global__ __launch_bounds__((bfuse::BfusePair<OP1, OP2, PATTERN, P0, P1>::THREADS), (bfuse::min_waves<OP1, OP2>()))  \
     void K1##_##K2##_fused_bfuse##SUFFIX(const void* __restrict__ I1, const void* __restrict__ F1,   \
                                          void* __restrict__ O1, const void* __restrict__ I2,         \
                                          const void* __restrict__ F2, void* __restrict__ O2)         \
@@ -511,7 +528,7 @@ KernelEntry make_fused_entry(const char* name, const void* func, int kind, const
             bfuse_module_hooks));
 
 #define BFUSE_HFUSE_KERNEL(K1, OP1, K2, OP2)                                                         \
-    extern "C" __global__ __launch_bounds__((bfuse::HfusePair<OP1, OP2>::THREADS), bfuse::kMinWavesPerEu)                  \
+    extern "C" __global__ __launch_bounds__((bfuse::HfusePair<OP1, OP2>::THREADS), (bfuse::min_waves<OP1, OP2>()))                  \
     void K1##_##K2##_fused_hfuse(const void* __restrict__ I1, const void* __restrict__ F1,           \
                                  void* __restrict__ O1, const void* __restrict__ I2,                 \
                                  const void* __restrict__ F2, void* __restrict__ O2)                 \
@@ -527,7 +544,7 @@ KernelEntry make_fused_entry(const char* name, const void* func, int kind, const
 // (scalar loads that hit at once) instead of costing every workgroup a chain of dependent loads
 // from device memory before it can start.  The host keeps the installed plan and appends it at launch.
 #define BFUSE_BFUSE_RT_KERNEL(K1, OP1, K2, OP2)                                                      \
-    extern "C" __global__ __launch_bounds__((bfuse::BfuseRtPair<OP1, OP2>::THREADS), bfuse::kMinWavesPerEu)                 \
+    extern "C" __global__ __launch_bounds__((bfuse::BfuseRtPair<OP1, OP2>::THREADS), (bfuse::min_waves<OP1, OP2>()))                 \
     void K1##_##K2##_fused_bfuse_rt(const void* __restrict__ I1, const void* __restrict__ F1,        \
                                     void* __restrict__ O1, const void* __restrict__ I2,              \
                                     const void* __restrict__ F2, void* __restrict__ O2,              \

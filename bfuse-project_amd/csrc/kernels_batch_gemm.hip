@@ -26,8 +26,10 @@ DENSE_F32(1024, 14336, 4096, 64, 128, 4)
     using Bgemm_##B##x##M##x##K##x##N = GemmF32<M, N, K, BM, BN, KS, kEpiNone, 2, 1, true, B>;                    \
     BFUSE_KERNEL(bgemm_f32_##B##x##M##x##K##x##N, Bgemm_##B##x##M##x##K##x##N, ({{B, M, K, 1}, 4}), ({{B, N, K, 1}, 4}), ({{B, M, N, 1}, 4}))
 // the one-wave products reserve 32 KB of LDS per workgroup: four workgroups per CU, one wave per SIMD (see LdsReserve).
-// (128 x 64 tiles run the K <= 128 products 7-16 % faster but need 300 registers: a fused kernel, which is compiled
-// for two waves per SIMD, has 256, so those stay on 64 x 64.)
+// (128 x 64 tiles run the K <= 128 products 7-16 % faster alone, but their 300 registers make every kernel they are part
+// of a kernel of one wave per SIMD (GemmF32::MIN_WAVES_PER_EU): block-fused with them, the pairs of the reference's
+// tests/interleave_scheduler suite read 0.79 of the unfused time instead of 0.90.  The operators of a fusion library
+// stay good partners: 64 x 64.)
 #define BGEMM_F32_RESERVE(B, M, K, N, BM, BN, KS, BYTES)                                                         \
     using Bgemm_##B##x##M##x##K##x##N = LdsReserve<GemmF32<M, N, K, BM, BN, KS, kEpiNone, 2, 1, true, B>, BYTES>; \
     BFUSE_KERNEL(bgemm_f32_##B##x##M##x##K##x##N, Bgemm_##B##x##M##x##K##x##N, ({{B, M, K, 1}, 4}), ({{B, N, K, 1}, 4}), ({{B, M, N, 1}, 4}))

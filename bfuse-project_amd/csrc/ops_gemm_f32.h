@@ -86,6 +86,8 @@ struct GemmF32 {
     static constexpr int THREADS = 64 * KS;
     static constexpr bool HAS_BARRIERS = KS > 1;
     static constexpr int NUNIT = TM * (G4 + G2 + G1);  // reduction / store units (one column group of one row block)
+    // 32 accumulator blocks (a 128 x 64 tile) and their operand stages do not fit the 256 registers of two waves per SIMD
+    static constexpr int MIN_WAVES_PER_EU = TM * NB >= 32 ? 1 : 2;
 
     // partial tiles of every wave, in accumulator layout
     struct Smem {
