@@ -52,6 +52,7 @@ using GemmS2 = GemmF32<96, 192, 128, 32, 64, 2, kEpiGeluTanh, 3>;     // 2 waves
 using GemmS3 = GemmF32<32, 144, 256, 32, 144, 4>;                     // the 64+64+16 column split, one tile
 using GemmS7 = GemmF32<80, 112, 32, 32, 64, 1>;                        // tiles that do not divide the problem: rows 0, 32, 48 and columns 0, 48 (the last tiles overlap their neighbours)
 using GemmS8 = GemmF32<48, 80, 64, 32, 64, 2, kEpiNone, 2, 1, true, 3>;   // the same on three batched products with B [N, K] and two waves over K
+using GemmS9 = GemmF32<256, 64, 32, 128, 64, 1>;                       // 128 x 64 tiles: 32 accumulator blocks, a kernel of one wave per SIMD (MIN_WAVES_PER_EU), also when fused
 using GemmS5 = GemmF32Dma<128, 192, 160, 32, 96, 2>;                  // private LDS rings, two waves split K, ten 8-k stages each
 using GemmS6 = GemmF32Dma<64, 288, 192, 32, 144, 4, kEpiGeluTanh>;    // the 32x144 tile (partial last B load), four waves, GELU
 using BiasReluS = BiasRelu<4096, 64, 4>;
@@ -78,6 +79,7 @@ BFUSE_KERNEL(gemm_gelu_f32_96x128x192, GemmS2, ({{96, 128, 1, 1}, 4}), ({{128, 1
 BFUSE_KERNEL(gemm_f32_32x256x144, GemmS3, ({{32, 256, 1, 1}, 4}), ({{256, 144, 1, 1}, 4}), ({{32, 144, 1, 1}, 4}))
 BFUSE_KERNEL(gemm_f32_80x32x112, GemmS7, ({{80, 32, 1, 1}, 4}), ({{32, 112, 1, 1}, 4}), ({{80, 112, 1, 1}, 4}))
 BFUSE_KERNEL(bgemm_f32_3x48x64x80, GemmS8, ({{3, 48, 64, 1}, 4}), ({{3, 80, 64, 1}, 4}), ({{3, 48, 80, 1}, 4}))
+BFUSE_KERNEL(gemm_f32_256x32x64_t128, GemmS9, ({{256, 32, 1, 1}, 4}), ({{32, 64, 1, 1}, 4}), ({{256, 64, 1, 1}, 4}))
 BFUSE_KERNEL(gemm_f32_128x160x192_d, GemmS5, ({{128, 160, 1, 1}, 4}), ({{160, 192, 1, 1}, 4}), ({{128, 192, 1, 1}, 4}))
 BFUSE_KERNEL(gemm_gelu_f32_64x192x288_d, GemmS6, ({{64, 192, 1, 1}, 4}), ({{192, 288, 1, 1}, 4}), ({{64, 288, 1, 1}, 4}))
 BFUSE_KERNEL(bias_relu_4096, BiasReluS, ({{4096, 1, 1, 1}, 4}), ({{4096, 1, 1, 1}, 4}), ({{4096, 1, 1, 1}, 4}))
@@ -151,6 +153,11 @@ BFUSE_BFUSE_KERNEL(conv1x1s1p0_f32_3x32x5x5_32, Conv1S1, layernorm_8x256, LayerN
 BFUSE_HFUSE_KERNEL(conv1x1s1p0_f32_5x96x9x9_48, Conv1S2, bias_relu_4096, BiasReluS)
 BFUSE_HFUSE_KERNEL(conv1x1s1p0_f32_5x96x9x9_48, Conv1S2, conv3x3_f32_32x12x12_32, ConvS2)
 BFUSE_BFUSE_KERNEL(conv1x1s2p0_f32_2x16x9x7_16, Conv1S3, bias_relu_4096, BiasReluS, , bfuse::kZigzag, 1, 1)
+// a side that needs more than the 256 registers of two waves per SIMD: the fused kernels are compiled for one
+static_assert(bfuse::min_waves<GemmS9>() == 1 && bfuse::min_waves<GemmS9, BiasReluS>() == 1 && bfuse::min_waves<GemmS1, BiasReluS>() == bfuse::kMinWavesPerEu,
+              "a fused kernel takes the smallest wave count of its sides");
+BFUSE_BFUSE_KERNEL(gemm_f32_256x32x64_t128, GemmS9, bias_relu_4096, BiasReluS, , bfuse::kZigzag, 1, 1)
+BFUSE_HFUSE_KERNEL(gemm_f32_256x32x64_t128, GemmS9, bias_relu_4096, BiasReluS)
 // overlapping last tiles: the shared elements are written twice with the same bits, also inside fused kernels
 BFUSE_BFUSE_KERNEL(gemm_f32_80x32x112, GemmS7, layernorm_8x256, LayerNormS, , bfuse::kZigzag, 1, 1)
 BFUSE_HFUSE_KERNEL(bgemm_f32_3x48x64x80, GemmS8, bias_relu_4096, BiasReluS)

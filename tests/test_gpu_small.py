@@ -35,6 +35,8 @@ def _cases():
     return {
         "gemm_f32_64x32x48": (lambda s: (fill_uniform(s, 64 * 32, -1, 1), fill_uniform(s + 1, 32 * 48, -1, 1)),
                               lambda I, F: orf.gemm_f32(I.reshape(64, 32), F.reshape(32, 48)), 1e-5, False),
+        "gemm_f32_256x32x64_t128": (lambda s: (fill_uniform(s, 256 * 32, -1, 1), fill_uniform(s + 1, 32 * 64, -1, 1)),
+                                    lambda I, F: orf.gemm_f32(I.reshape(256, 32), F.reshape(32, 64)), 1e-5, False),
         "gemm_f32_80x32x112": (lambda s: (fill_uniform(s, 80 * 32, -1, 1), fill_uniform(s + 1, 32 * 112, -1, 1)),
                                lambda I, F: orf.gemm_f32(I.reshape(80, 32), F.reshape(32, 112)), 1e-5, False),
         "bgemm_f32_3x48x64x80": (lambda s: (fill_uniform(s, 3 * 48 * 64, -1, 1), fill_uniform(s + 1, 3 * 80 * 64, -1, 1)),
@@ -107,6 +109,8 @@ FUSIONS = [
     ("conv1x1s1p0_f32_5x96x9x9_48", "bias_relu_4096", "hfuse", ""),                # a barrier per filter chunk beside a side without any: LDS arrival counters
     ("conv1x1s1p0_f32_5x96x9x9_48", "conv3x3_f32_32x12x12_32", "hfuse", ""),       # both sides synchronise
     ("conv1x1s2p0_f32_2x16x9x7_16", "bias_relu_4096", "bfuse", ""),
+    ("gemm_f32_256x32x64_t128", "bias_relu_4096", "bfuse", ""),                    # a side of 128 x 64 tiles: the fused kernels are kernels of one wave per SIMD
+    ("gemm_f32_256x32x64_t128", "bias_relu_4096", "hfuse", ""),
     ("gemm_f32_80x32x112", "layernorm_8x256", "bfuse", ""),                        # GEMM tiles that overlap (80 = 32 + 32 + 16 rows)
     ("bgemm_f32_3x48x64x80", "bias_relu_4096", "hfuse", ""),
 ]
