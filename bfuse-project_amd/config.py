@@ -148,7 +148,7 @@ def choose_fusion(a: KernelInfo, b: KernelInfo, lds_a: int, lds_b: int, cus: int
       nothing to give each other but their ends: whatever the fused form, one side's workgroups only
       take the place of the other's.  Such a pair is left unfused.  (Measured on the reference's
       benchmark arrangement -- 903 pairs of GEMMs, batched products and convolutions at batch 1024,
-      all of this kind: block fusion 0.88x, thread-level fusion 0.64x, two streams 1.00x.)
+      all of this kind: block fusion 0.88x, thread-level fusion 0.63x, two streams 1.00x.)
     """
     ta, tb = a.dims.block[0] * a.dims.block[1] * a.dims.block[2], b.dims.block[0] * b.dims.block[1] * b.dims.block[2]
     wa, wb = -(-ta // 64), -(-tb // 64)

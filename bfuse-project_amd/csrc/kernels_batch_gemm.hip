@@ -41,7 +41,7 @@ BGEMM_F32_RESERVE(1024, 256, 64, 256, 64, 64, 1, 32768)
 BGEMM_F32_RESERVE(1024, 256, 256, 64, 64, 64, 1, 32768)
 BGEMM_F32_RESERVE(1024, 256, 80, 256, 64, 64, 1, 32768)
 BGEMM_F32_RESERVE(1024, 256, 256, 80, 64, 80, 1, 32768)
-BGEMM_F32(1024, 208, 64, 208, 16, 208, 1)
+BGEMM_F32_RESERVE(1024, 208, 64, 208, 112, 64, 1, 32768)
 BGEMM_F32_RESERVE(1024, 208, 208, 64, 208, 32, 1, 32768)
 BGEMM_F32_RESERVE(1024, 208, 80, 208, 112, 64, 1, 32768)     // 208 = 112 + 96 rows, 3 x 64 + 16 columns: the last tiles overlap their neighbours
 BGEMM_F32_RESERVE(1024, 208, 208, 80, 64, 80, 1, 32768)

@@ -133,7 +133,7 @@ def test_the_footprint_rule_on_the_headline_pairs_with_and_without_times():
 def test_two_kernels_that_each_keep_every_matrix_pipe_busy_are_left_unfused():
     """The reference's benchmark arrangement (every dense layer, batched product and convolution at batch 1024
     against every other: bfuse-project_amd/examples/benchmark_batch1024.yaml, 903 pairs): measured on MI355X,
-    block fusion 0.88x, thread-level fusion 0.64x of the two kernels one after the other -- each kernel already
+    block fusion 0.88x, thread-level fusion 0.63x of the two kernels one after the other -- each kernel already
     has a wave on every SIMD for its whole run.  The rule leaves every such pair unfused, from the registry's
     metadata alone; a matrix-core kernel that does not cover the chip (196 workgroups of a batch-1 convolution)
     or a side that is not a matrix-core kernel keeps the decision the footprints give."""
