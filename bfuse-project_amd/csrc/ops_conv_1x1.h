@@ -10,8 +10,8 @@
 // there; here the image goes from memory straight into the registers of the MFMA that consumes it.
 //
 // One wave owns 64 consecutive pixels of one image (a tile) and BM output channels; the NW waves of a
-// workgroup own NW consecutive tiles of the batch-wide tile sequence (image after image; the last tile of an
-// image is ragged when H*W is not a multiple of 64) and share the filter rows co0 .. co0+BM-1, which the
+// workgroup own NW consecutive tiles of the batch-wide tile sequence (image after image) and share the filter
+// rows co0 .. co0+BM-1, which the
 // workgroup stages in LDS in chunks of up to 64 input channels, double-buffered, one barrier per chunk.
 //
 // Lane (j = lane % 16, q = lane / 16) loads, for step s = 0..3 of a 16-channel group g, the 16 bytes
